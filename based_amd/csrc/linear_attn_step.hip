@@ -1,0 +1,199 @@
+// Recurrent decode step of Taylor linear attention for gfx950 (HBM-bandwidth bound).
+//
+// One workgroup per (batch, head); one wavefront per 16 rows of the (dv x 273) fp32 state.
+// A wavefront's 16 rows are 4368 contiguous floats = 1092 aligned float4, which it streams
+// with fully coalesced 128-bit loads and stores (lane i of iteration t touches float4
+// 64 t + i).  Since 256 floats per iteration < 273, an iteration touches at most two state
+// rows and, after full unrolling, which two is a compile-time constant: partial dot
+// products go to per-lane accumulators indexed by row, and one transposing butterfly at
+// the end reduces all 16 rows across the wavefront.  phi(q) and phi(k) are expanded once
+// per workgroup into LDS, in four copies shifted by 0..3 floats so that each lane's four
+// consecutive features are one aligned 128-bit LDS read; the copies run 3 entries past 273
+// and wrap, which is exactly where a float4 straddles into the next state row.
+#include "common.hpp"
+
+namespace based {
+
+constexpr int kTabLen = 280;                     // 273 + 3 wrap entries, padded to 16 B multiple
+constexpr int kRowsPerWave = 16;
+constexpr int kVec4PerWave = kRowsPerWave * kExp / 4;  // 1092
+constexpr int kIters = (kVec4PerWave + kWave - 1) / kWave;  // 18
+constexpr int kBatch = 9;                        // loads in flight per lane
+
+__device__ __forceinline__ float phi_elem(const float* x, int f) {
+  // TaylorExp element f of a 16-vector x: [1 | x/2 | x_i x_j / (4 sqrt 2)], row-major i,j.
+  if (f == 0) return 1.0f;
+  if (f <= kFeat) return x[f - 1] * 0.5f;
+  int g = f - 1 - kFeat;
+  return x[g >> 4] * x[g & 15] * 0.17677669529663687f;
+}
+
+template <typename T, int kMaxThreads>
+__global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+    float* __restrict__ kv_state, float* __restrict__ k_state, T* __restrict__ y,
+    int H, int dv, long q_sb, long q_sh, long k_sb, long k_sh, long v_sb, long v_sh,
+    long y_sb, long y_sh, float eps) {
+  __shared__ float s_x[2][kFeat];                            // [0] = k, [1] = q
+  __shared__ __align__(16) float s_tab[2][4][kTabLen];       // [0] = phi(k), [1] = phi(q)
+  __shared__ float s_v[256];
+  __shared__ float s_den;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const long bh = blockIdx.x;
+  const int b = (int)(bh / H), h = (int)(bh % H);
+
+  if (tid < 2 * kFeat) {
+    const int which = tid >> 4, i = tid & 15;
+    const T* src = which ? (q + b * q_sb + h * q_sh) : (k + b * k_sb + h * k_sh);
+    s_x[which][i] = to_f32(src[i]);
+  }
+  if (tid < dv) s_v[tid] = to_f32(v[b * v_sb + h * v_sh + tid]);
+  __syncthreads();
+
+  for (int idx = tid; idx < 2 * 4 * kTabLen; idx += blockDim.x) {
+    const int which = idx / (4 * kTabLen);
+    const int rem = idx - which * (4 * kTabLen);
+    const int m = rem / kTabLen, i = rem - m * kTabLen;
+    const int e = i + m;
+    float val = 0.0f;
+    if (e < kExp + 3) val = phi_elem(s_x[which], e >= kExp ? e - kExp : e);
+    s_tab[which][m][i] = val;
+  }
+  __syncthreads();
+
+  // Normaliser: k_state += phi(k); den = phi(q) . k_state.  One wavefront owns it.
+  if (wave == 0) {
+    float* ks = k_state + bh * kExp;
+    float part = 0.0f;
+    for (int f = lane; f < kExp; f += kWave) {
+      const float nk = ks[f] + s_tab[0][0][f];
+      ks[f] = nk;
+      part += s_tab[1][0][f] * nk;
+    }
+    part = wave_sum(part);
+    if (lane == 0) s_den = part;
+  }
+
+  // State rows [16*wave, 16*wave+16) of this (b, h).  v is wave-uniform: keep it scalar.
+  float vrow[kRowsPerWave];
+#pragma unroll
+  for (int r = 0; r < kRowsPerWave; ++r)
+    vrow[r] = __builtin_bit_cast(
+        float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s_v[kRowsPerWave * wave + r])));
+
+  f32x4* base = reinterpret_cast<f32x4*>(kv_state + (bh * dv + (long)kRowsPerWave * wave) * kExp);
+
+  float acc[kRowsPerWave];
+#pragma unroll
+  for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
+
+  const int e_lane = 4 * lane;
+  // Two batches of 9 iterations: all loads of a batch are issued before its first use.
+#pragma unroll
+  for (int t0 = 0; t0 < kIters; t0 += kBatch) {
+    f32x4 d[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int t = t0 + u;
+      const int j = t * kWave + lane;
+      if (t < kIters - 1 || j < kVec4PerWave) d[u] = __builtin_nontemporal_load(base + j);
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int t = t0 + u;
+      const int j = t * kWave + lane;
+      const int rb = (256 * t) / kExp;              // first row touched by this iteration
+      const int bnd = (rb + 1) * kExp - 256 * t;    // local element index where row rb+1 starts
+      const bool two_rows = bnd < 256;
+      if (t < kIters - 1 || j < kVec4PerWave) {
+        const bool lane_hi = two_rows && (e_lane >= bnd);
+        const int f0 = (256 * t - rb * kExp) + e_lane - (lane_hi ? kExp : 0);
+        const int m = f0 & 3;
+        const f32x4 pk = *reinterpret_cast<const f32x4*>(&s_tab[0][m][f0 - m]);
+        const f32x4 pq = *reinterpret_cast<const f32x4*>(&s_tab[1][m][f0 - m]);
+        const float v_lo = vrow[rb];
+        const float v_hi = vrow[rb + 1 < kRowsPerWave ? rb + 1 : rb];
+        f32x4 x = d[u];
+        float s_lo = 0.0f, s_hi = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const bool hi = two_rows && (e_lane + c >= bnd);
+          const float nv = __builtin_fmaf(hi ? v_hi : v_lo, pk[c], x[c]);
+          x[c] = nv;
+          const float p = pq[c] * nv;
+          s_lo += hi ? 0.0f : p;
+          s_hi += hi ? p : 0.0f;
+        }
+        __builtin_nontemporal_store(x, base + j);
+        acc[rb] += s_lo;
+        if (two_rows && rb + 1 < kRowsPerWave) acc[rb + 1] += s_hi;
+      }
+    }
+  }
+
+  // Transposing butterfly: 16 per-lane row sums -> lane l holds the total of row l >> 2.
+#pragma unroll
+  for (int half = 8, mask = 32; half >= 1; half >>= 1, mask >>= 1) {
+    const bool up = (lane & mask) != 0;
+#pragma unroll
+    for (int i = 0; i < half; ++i) {
+      const float a = acc[i], bb = acc[i + half];
+      const float keep = up ? bb : a;
+      const float send = up ? a : bb;
+      acc[i] = keep + __shfl_xor(send, mask, 64);
+    }
+  }
+  float num = acc[0];
+  num += __shfl_xor(num, 2, 64);
+  num += __shfl_xor(num, 1, 64);
+
+  __syncthreads();
+  if ((lane & 3) == 0) {
+    const int e = kRowsPerWave * wave + (lane >> 2);
+    y[b * y_sb + h * y_sh + e] = from_f32<T>(num / (s_den + eps));
+  }
+}
+
+}  // namespace based
+
+extern "C" BASED_API int based_linear_attn_step(const void* q, const void* k, const void* v,
+                                      float* kv_state, float* k_state, void* y,
+                                      int64_t B, int64_t H, int64_t dv,
+                                      int64_t q_sb, int64_t q_sh, int64_t k_sb, int64_t k_sh,
+                                      int64_t v_sb, int64_t v_sh, int64_t y_sb, int64_t y_sh,
+                                      float eps, int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(q && k && v && kv_state && k_state && y, BASED_ERR_ARG,
+                "linear_attn_step: null pointer argument");
+  BASED_REQUIRE(B >= 0 && H > 0, BASED_ERR_ARG, "linear_attn_step: bad sizes B=%ld H=%ld",
+                (long)B, (long)H);
+  BASED_REQUIRE(dv >= 16 && dv <= 256 && dv % 16 == 0, BASED_ERR_SHAPE,
+                "linear_attn_step: head dim %ld unsupported (multiple of 16 in [16, 256])", (long)dv);
+  BASED_REQUIRE((reinterpret_cast<uintptr_t>(kv_state) & 15) == 0, BASED_ERR_ALIGN,
+                "linear_attn_step: kv_state must be 16-byte aligned");
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE,
+                "linear_attn_step: io_dtype %d unsupported", io_dtype);
+  BASED_REQUIRE(B * H < (1ll << 31), BASED_ERR_SHAPE, "linear_attn_step: B*H too large");
+  if (B == 0) return BASED_OK;
+  dim3 grid((unsigned)(B * H)), block((unsigned)(dv / 16 * 64));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define BASED_LAUNCH_STEP(T, MAXT)                                                              \
+  hipLaunchKernelGGL((lin_step_kernel<T, MAXT>), grid, block, 0, s, (const T*)q, (const T*)k,   \
+                     (const T*)v, kv_state, k_state, (T*)y, (int)H, (int)dv, q_sb, q_sh, k_sb,  \
+                     k_sh, v_sb, v_sh, y_sb, y_sh, eps)
+  // The register budget follows the workgroup size: 4 waves (dv <= 64) may use 256 VGPRs.
+  if (io_dtype == BASED_BF16) {
+    if (dv <= 64) BASED_LAUNCH_STEP(__bf16, 256);
+    else if (dv <= 128) BASED_LAUNCH_STEP(__bf16, 512);
+    else BASED_LAUNCH_STEP(__bf16, 1024);
+  } else {
+    if (dv <= 64) BASED_LAUNCH_STEP(float, 256);
+    else if (dv <= 128) BASED_LAUNCH_STEP(float, 512);
+    else BASED_LAUNCH_STEP(float, 1024);
+  }
+#undef BASED_LAUNCH_STEP
+  return check_launch("linear_attn_step");
+}

@@ -1,0 +1,65 @@
+"""Tensor-level wrappers over the C ABI: validate, take pointers/strides, enqueue on torch's
+current stream.  PyTorch is used for device memory and streams only."""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+FEATURE_DIM = 16
+EXPANDED_DIM = 273
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return _lib.BASED_BF16
+    if t.dtype == torch.float32:
+        return _lib.BASED_F32
+    raise ValueError(f"unsupported dtype {t.dtype} (bfloat16 or float32)")
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_cuda(*ts: torch.Tensor) -> None:
+    dev = ts[0].device
+    for t in ts:
+        if not t.is_cuda:
+            raise ValueError("based_amd kernels need tensors on a HIP device (no CPU path)")
+        if t.device != dev:
+            raise ValueError("all tensors must live on the same device")
+
+
+def linear_attn_step(q, k, v, kv_state, k_state, eps: float = 1e-12) -> torch.Tensor:
+    """One decode step.  q, k: (B, H, 1, 16) raw; v: (B, H, 1, dv); kv_state (B,H,1,dv,273)
+    and k_state (B,H,1,1,273) fp32 contiguous, updated in place.  Returns y (B, H, 1, dv)."""
+    _require_cuda(q, k, v, kv_state, k_state)
+    B, H, l, d = q.shape
+    assert l == 1, f"q.shape is {tuple(q.shape)} but should be ({B}, {H}, 1, {d})"
+    dv = v.shape[-1]
+    if d != FEATURE_DIM or k.shape != q.shape or v.shape[:3] != q.shape[:3]:
+        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+    if kv_state.dtype != torch.float32 or k_state.dtype != torch.float32:
+        raise ValueError("decode states must be float32")
+    if tuple(kv_state.shape) != (B, H, 1, dv, EXPANDED_DIM) or tuple(k_state.shape) != (B, H, 1, 1, EXPANDED_DIM):
+        raise ValueError(f"bad state shapes {tuple(kv_state.shape)} {tuple(k_state.shape)}")
+    if not (kv_state.is_contiguous() and k_state.is_contiguous()):
+        raise ValueError("decode states must be contiguous")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share a dtype")
+    for t in (q, k, v):
+        if t.stride(-1) != 1:
+            raise ValueError("innermost dimension must be contiguous")
+    y = torch.empty(B, H, 1, dv, dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().based_linear_attn_step(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), kv_state.data_ptr(), k_state.data_ptr(), y.data_ptr(),
+            B, H, dv,
+            q.stride(0), q.stride(1), k.stride(0), k.stride(1),
+            v.stride(0), v.stride(1), y.stride(0), y.stride(1),
+            float(eps), _dtype_code(q), _stream_ptr(q)))
+    return y

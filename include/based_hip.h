@@ -1,0 +1,142 @@
+/*
+ * based_hip.h — C ABI of libbased_hip.so, the MI355X (gfx950) kernels behind the Based
+ * sequence mixers.
+ *
+ * Every entry point takes raw device pointers, element strides and sizes, and a HIP
+ * stream (passed as void*; NULL = the default stream).  Launches are asynchronous on that
+ * stream; pointers are borrowed until the work on the stream has finished.  Nothing here
+ * allocates, synchronises or reads device memory from the host, so every call can be
+ * captured into a HIP graph.
+ *
+ * Return value: BASED_OK (0) on success, otherwise one of the BASED_ERR_* codes; a
+ * human-readable reason is then available from based_hip_last_error() (thread-local).
+ * Unsupported shapes are rejected before anything is launched.
+ *
+ * Citations name the reference (HazyResearch/based) code each entry point stands in for.
+ */
+#ifndef BASED_HIP_H
+#define BASED_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BASED_API __attribute__((visibility("default")))
+
+enum {
+  BASED_OK = 0,
+  BASED_ERR_SHAPE = 1,  /* unsupported size (feature dim, head dim, window ...) */
+  BASED_ERR_DTYPE = 2,  /* unsupported element type */
+  BASED_ERR_ALIGN = 3,  /* pointer or stride not aligned as the kernel requires */
+  BASED_ERR_ARG = 4,    /* null pointer / negative size */
+  BASED_ERR_LAUNCH = 5  /* the HIP runtime refused the launch */
+};
+
+/* element types of q / k / v / y tensors */
+enum { BASED_BF16 = 0, BASED_F32 = 1 };
+
+/* feature dimension of the TaylorExp map this library is built for, and its expansion
+ * 1 + d + d*d (based/models/mixers/linear_attention.py:255-256). */
+#define BASED_FEATURE_DIM 16
+#define BASED_EXPANDED_DIM 273
+
+BASED_API int based_hip_version(void);
+BASED_API const char* based_hip_last_error(void);
+
+/*
+ * Recurrent decode step of Taylor linear attention, feature map fused.
+ * Replaces TaylorExp.forward on q,k + LinearAttention.recurrent_forward up to (not
+ * including) out_proj: based/models/mixers/linear_attention.py:136-140,230-249.
+ *
+ *   kv_state[b,h,e,f] += v[b,h,e] * phi(k[b,h])[f]          (in place, fp32)
+ *   k_state [b,h,f]   += phi(k[b,h])[f]                     (in place, fp32)
+ *   y[b,h,e] = sum_f phi(q)[f] kv_state[b,h,e,f] / (sum_f phi(q)[f] k_state[b,h,f] + eps)
+ *
+ * q, k : raw 16-dim vectors, element (b,h,i) at  q[b*q_sb + h*q_sh + i]
+ * v, y : dv-dim vectors,     element (b,h,e) at  v[b*v_sb + h*v_sh + e]
+ * kv_state : contiguous fp32 (B, H, 1, dv, 273); k_state : contiguous fp32 (B, H, 1, 1, 273)
+ *            (layout of LinearAttention.allocate_inference_cache, linear_attention.py:258-269)
+ * dv must be a multiple of 16, 16 <= dv <= 256.  kv_state must be 16-byte aligned.
+ * io_dtype is the element type of q, k, v and y.
+ */
+BASED_API int based_linear_attn_step(const void* q, const void* k, const void* v,
+                           float* kv_state, float* k_state, void* y,
+                           int64_t B, int64_t H, int64_t dv,
+                           int64_t q_sb, int64_t q_sh, int64_t k_sb, int64_t k_sh,
+                           int64_t v_sb, int64_t v_sh, int64_t y_sb, int64_t y_sh,
+                           float eps, int io_dtype, void* stream);
+
+/*
+ * Causal Taylor linear attention over a whole sequence (prefill), feature map,
+ * normaliser and decode-state construction fused.
+ * Replaces LinearAttention.parallel_forward up to (not including) out_proj, and the
+ * state einsums that follow it: based/models/mixers/linear_attention.py:169-183,220-222
+ * (same arithmetic as the O(L) causal product in
+ * train/csrc/causal_dot_prod/causal_attention.cpp:82-124 plus its normaliser).
+ *
+ *   y[b,h,i,:] = sum_{j<=i} (phi(q_i).phi(k_j)) v_j / (phi(q_i).sum_{j<=i} phi(k_j) + eps)
+ *   kv_state[b,h,e,f] = sum_n v[n,e] phi(k_n)[f],  k_state[b,h,f] = sum_n phi(k_n)[f]
+ *
+ * q, k : element (b,h,l,i) at q[b*q_sb + h*q_sh + l*q_sl + i]   (i < 16 contiguous)
+ * v, y : element (b,h,l,e) at v[b*v_sb + h*v_sh + l*v_sl + e]   (e < dv contiguous)
+ * kv_state / k_state: as above; either both NULL (training-style forward, no state
+ * written) or both non-NULL (overwritten, not accumulated).
+ * dv in {64, 128}; any L >= 1.  Row starts of q, k (32 B for bf16) and v, y must be
+ * 16-byte aligned.
+ */
+BASED_API int based_linear_attn_prefill(const void* q, const void* k, const void* v, void* y,
+                              float* kv_state, float* k_state,
+                              int64_t B, int64_t H, int64_t L, int64_t dv,
+                              int64_t q_sb, int64_t q_sh, int64_t q_sl,
+                              int64_t k_sb, int64_t k_sh, int64_t k_sl,
+                              int64_t v_sb, int64_t v_sh, int64_t v_sl,
+                              int64_t y_sb, int64_t y_sh, int64_t y_sl,
+                              float eps, int io_dtype, void* stream);
+
+/*
+ * Sliding-window causal softmax attention over a whole sequence.
+ * Replaces the flash-attn call behind FlashSelfAttention / FlashCrossAttention with
+ * causal=True, window_size=(w_left, 0): based/models/mixers/slide_attention.py:100-106,
+ * 206-213.  Query i attends keys j in [i - w_left, i].
+ *
+ * q, k, v, o : element (b,l,h,c) at p[b*sb + l*sl + h*sh + c], c < 64 contiguous.
+ * head dim is 64; 0 <= w_left <= 64 (pass window_size // 2 of the module).  bf16 only.
+ */
+BASED_API int based_swa_prefill(const void* q, const void* k, const void* v, void* o,
+                      int64_t B, int64_t H, int64_t L,
+                      int64_t q_sb, int64_t q_sl, int64_t q_sh,
+                      int64_t k_sb, int64_t k_sl, int64_t k_sh,
+                      int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                      int64_t o_sb, int64_t o_sl, int64_t o_sh,
+                      int w_left, float scale, int io_dtype, void* stream);
+
+/*
+ * Sliding-window decode step against a linear KV cache.
+ * Replaces flash_attn_with_kvcache(q, k_cache, v_cache, k_new, v_new, cache_seqlens,
+ * causal=True, window_size=(w_left,0)): based/models/mixers/slide_attention.py:471-481
+ * (and the cache write of _update_kv_cache, :255-281).
+ *
+ * Writes k_new/v_new (B,1,H,64) into row `pos` of the caches, then attends rows
+ * [pos - w_left, pos].  pos is cache_seqlens[b] when cache_seqlens (device int32, B
+ * entries) is non-NULL — nothing is read on the host, so the call is graph-capturable —
+ * else pos_host for every b.
+ *
+ * kcache, vcache : element (b,t,h,c) at p[b*c_sb + t*c_st + h*c_sh + c]; the reference's
+ *   packed (B, max_seqlen, 2, H, 64) cache is passed as two pointers 1 plane apart.
+ * q, k_new, v_new, o : element (b,h,c) at p[b*sb + h*sh + c].
+ */
+BASED_API int based_swa_step(const void* q, const void* k_new, const void* v_new,
+                   void* kcache, void* vcache, void* o,
+                   const int32_t* cache_seqlens, int64_t pos_host,
+                   int64_t B, int64_t H, int64_t max_seqlen,
+                   int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
+                   int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
+                   int64_t c_sb, int64_t c_st, int64_t c_sh,
+                   int w_left, float scale, int io_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BASED_HIP_H */

@@ -1,0 +1,209 @@
+"""Pure-PyTorch CPU restatement of the Based sequence-mixer arithmetic.
+
+TEST INFRASTRUCTURE ONLY: the shipped package never imports this file.  Each
+function states, as plainly as possible, what the reference computes; the
+citations are into the reference tree (paths relative to its root).
+
+Pinning status (what independent evidence each function is checked against in
+tests/test_oracle.py):
+
+  taylor_exp              closed form  phi(q).phi(k) == 1 + s + s^2/2, element order,
+                          phi(0) == e_0                                   -> pinned
+  linear_attn_quadratic   brute-force per-element formula on tiny inputs, running-mean
+                          special case, causality, the compiled reference C++ causal
+                          product (oracle/_ref) for the numerator         -> pinned
+  linear_attn_cumsum      equality with linear_attn_quadratic + reference C++ -> pinned
+  linear_attn_prefill_state / linear_attn_step
+                          recurrent == parallel invariant (the reference's own
+                          test), closed-form state sums                   -> pinned
+  sliding_window_attn     reduction to F.scaled_dot_product_attention(is_causal) when
+                          the window covers the sequence, w=0 => o=v, q=0 => running
+                          window mean, per-element brute force            -> pinned
+                          against the textbook definition; the reference delegates
+                          this arithmetic to flash-attn 2.5.2 (absent from the tree),
+                          so agreement with THAT library is "parity unpinned".
+  sliding_window_step     decode == prefill invariant                     -> pinned (same caveat)
+  rms_norm / swiglu_mlp / short_conv(_step)
+                          closed forms + F.conv1d + step == parallel      -> pinned
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+# ----------------------------------------------------------------------------------------------
+# TaylorExp feature map  (based/models/mixers/linear_attention.py:52-75)
+# ----------------------------------------------------------------------------------------------
+def taylor_exp(x: torch.Tensor) -> torch.Tensor:
+    """phi(x) = [1, x / d^(1/4), vec(x x^T) / (sqrt(2) sqrt(d))]  ->  (..., 1 + d + d*d).
+
+    Second-order block is the FULL outer product in row-major order (index 1+d+i*d+j),
+    exactly as `(x.unsqueeze(-1) * x.unsqueeze(-2)).flatten(-2)` at linear_attention.py:69.
+    Arithmetic is done in the dtype of `x` (the reference does not upcast).
+    """
+    d = x.shape[-1]
+    rd = math.sqrt(d)
+    rrd = math.sqrt(rd)
+    r2 = math.sqrt(2.0)
+    outer = x[..., :, None] * x[..., None, :]
+    second = outer.reshape(*x.shape[:-1], d * d) / r2
+    ones = torch.ones_like(x[..., :1])
+    return torch.cat([ones, x / rrd, second / rd], dim=-1)
+
+
+def taylor_dot(q: torch.Tensor, k: torch.Tensor) -> torch.Tensor:
+    """Closed form of phi(q).phi(k):  1 + s + s^2/2 with s = q.k / sqrt(d)."""
+    s = (q * k).sum(-1) / math.sqrt(q.shape[-1])
+    return 1.0 + s + 0.5 * s * s
+
+
+# ----------------------------------------------------------------------------------------------
+# Causal linear attention, parallel forms
+# ----------------------------------------------------------------------------------------------
+def linear_attn_quadratic(q, k, v, eps: float = 1e-12):
+    """Reference "quadratic" branch (linear_attention.py:169-183) without the out_proj.
+
+    q, k: (B, H, L, d) raw (un-mapped);  v: (B, H, L, dv).  Returns y (B, H, L, dv) with
+        y_i = sum_{j<=i} (phi(q_i).phi(k_j)) v_j / (phi(q_i) . sum_{j<=i} phi(k_j) + eps)
+    """
+    fq, fk = taylor_exp(q), taylor_exp(k)
+    a = torch.einsum("bhnd,bhmd->bhnm", fq, fk)
+    a = torch.tril(a)
+    y = torch.einsum("bhnm,bhme->bhne", a, v)
+    z = 1.0 / (torch.einsum("bhld,bhld->bhl", fq, fk.cumsum(2)) + eps)
+    return y * z[..., None]
+
+
+def linear_attn_cumsum(q, k, v, eps: float = 1e-12, chunk: int = 64):
+    """O(L) form: running kv = sum phi(k) (x) v, as in the reference's C++ causal product
+    (train/csrc/causal_dot_prod/causal_attention.cpp:82-124) and its smoke script
+    (train/csrc/causal_dot_prod/test.py:22-27).  Evaluated chunk-wise so the
+    (L, D, dv) cumulative tensor is never materialised.
+    """
+    fq, fk = taylor_exp(q), taylor_exp(k)
+    B, H, L, D = fq.shape
+    dv = v.shape[-1]
+    kv = torch.zeros(B, H, D, dv, dtype=fq.dtype)
+    ks = torch.zeros(B, H, D, dtype=fq.dtype)
+    out = torch.empty(B, H, L, dv, dtype=fq.dtype)
+    for s in range(0, L, chunk):
+        e = min(L, s + chunk)
+        kvc = kv[:, :, None] + torch.cumsum(fk[:, :, s:e, :, None] * v[:, :, s:e, None, :], dim=2)
+        ksc = ks[:, :, None] + torch.cumsum(fk[:, :, s:e], dim=2)
+        num = torch.einsum("bhld,bhlde->bhle", fq[:, :, s:e], kvc)
+        den = torch.einsum("bhld,bhld->bhl", fq[:, :, s:e], ksc) + eps
+        out[:, :, s:e] = num / den[..., None]
+        kv, ks = kvc[:, :, -1], ksc[:, :, -1]
+    return out
+
+
+def linear_attn_prefill_state(k, v):
+    """Decode state left behind by a prefill (linear_attention.py:220-222).
+
+    Returns kv_state (B, H, 1, dv, D) with kv_state[b,h,0,e,f] = sum_n v[n,e] phi(k)[n,f]
+    and k_state (B, H, 1, 1, D) = sum_n phi(k)[n].
+    """
+    fk = taylor_exp(k)
+    kv_state = torch.einsum("bhnd,bhnf->bhfd", fk, v)[:, :, None]
+    k_state = fk.sum(dim=2)[:, :, None, None]
+    return kv_state, k_state
+
+
+def linear_attn_step(kv_state, k_state, q, k, v, eps: float = 1e-12):
+    """One recurrent decode step (linear_attention.py:230-252) without the out_proj.
+
+    q, k: (B, H, 1, d) raw;  v: (B, H, 1, dv).  Mutates kv_state (B,H,1,dv,D) and
+    k_state (B,H,1,1,D) IN PLACE, returns y (B, H, 1, dv) in the dtype of the states.
+    """
+    fq, fk = taylor_exp(q), taylor_exp(k)
+    fq, fk, vv = fq.unsqueeze(-2), fk.unsqueeze(-2), v.unsqueeze(-1)
+    kv_state += (fk[:, :, -1:] * vv[:, :, -1:]).to(kv_state.dtype)
+    k_state += fk[:, :, -1:].to(k_state.dtype)
+    num = (fq.to(kv_state.dtype) * kv_state).sum(dim=-1)
+    den = (fq.to(k_state.dtype) * k_state).sum(dim=-1) + eps
+    return num / den
+
+
+# ----------------------------------------------------------------------------------------------
+# Sliding-window causal softmax attention
+# ----------------------------------------------------------------------------------------------
+def sliding_window_attn(q, k, v, w_left: int = 64, scale: float | None = None):
+    """Textbook masked softmax with the flash-attn window convention the reference passes
+    (`window_size=(W//2, 0)`, causal: slide_attention.py:97-106,332-336): query i attends
+    keys j in [i - w_left, i].  Statement follows the in-tree textbook attention
+    (based/models/mixers/mha.py:243-275) with the band mask added.
+
+    q, k, v: (B, L, H, D).  Returns (B, L, H, D) in fp32 arithmetic, cast to q.dtype.
+    """
+    B, L, H, D = q.shape
+    scale = 1.0 / math.sqrt(D) if scale is None else scale
+    qf, kf, vf = q.float(), k.float(), v.float()
+    scores = torch.einsum("bthd,bshd->bhts", qf, kf) * scale
+    i = torch.arange(L)[:, None]
+    j = torch.arange(L)[None, :]
+    keep = (j <= i) & (j >= i - w_left)
+    scores = scores.masked_fill(~keep, float("-inf"))
+    p = torch.softmax(scores, dim=-1)
+    return torch.einsum("bhts,bshd->bthd", p, vf).to(q.dtype)
+
+
+def sliding_window_step(q, k_new, v_new, kv_cache, pos: int, w_left: int = 64, scale: float | None = None):
+    """Decode step with a linear KV cache (slide_attention.py:430-481): write the new k, v at
+    row `pos` of kv_cache (B, max_seqlen, 2, H, D), then attend keys [pos - w_left, pos].
+
+    q, k_new, v_new: (B, 1, H, D).  Mutates kv_cache in place.  Returns (B, 1, H, D).
+    """
+    B, _, H, D = q.shape
+    scale = 1.0 / math.sqrt(D) if scale is None else scale
+    kv_cache[:, pos, 0] = k_new[:, 0].to(kv_cache.dtype)
+    kv_cache[:, pos, 1] = v_new[:, 0].to(kv_cache.dtype)
+    lo = max(0, pos - w_left)
+    kf = kv_cache[:, lo:pos + 1, 0].float()
+    vf = kv_cache[:, lo:pos + 1, 1].float()
+    scores = torch.einsum("bthd,bshd->bhts", q.float(), kf) * scale
+    p = torch.softmax(scores, dim=-1)
+    return torch.einsum("bhts,bshd->bthd", p, vf).to(q.dtype)
+
+
+# ----------------------------------------------------------------------------------------------
+# Stack glue used only by the 27-layer configuration
+# ----------------------------------------------------------------------------------------------
+def rms_norm(x, weight, eps: float = 1e-5):
+    """x * rsqrt(mean(x^2) + eps) * w  (based/ops/triton/layer_norm.py:117-118), fp32 math."""
+    xf = x.float()
+    rstd = torch.rsqrt(xf.square().mean(dim=-1, keepdim=True) + eps)
+    return (xf * rstd * weight.float()).to(x.dtype)
+
+
+def swiglu_mlp(x, w1, w2):
+    """fc2( y * silu(gate) ) with y, gate = fc1(x).chunk(2)  (based/models/mlp.py:141-157)."""
+    y, gate = F.linear(x, w1).chunk(2, dim=-1)
+    return F.linear(y * F.silu(gate), w2)
+
+
+def short_conv(x, weight):
+    """Depthwise causal convolution (based/models/mixers/convolution.py:47-83, non-CUDA path):
+    y[b, t, c] = sum_{i<K} weight[c, i] * x[b, t - (K-1) + i, c], zero left padding.
+    x: (B, L, C); weight: (C, K).
+    """
+    B, L, C = x.shape
+    K = weight.shape[-1]
+    y = torch.zeros_like(x)
+    for i in range(K):
+        shift = K - 1 - i
+        if shift == 0:
+            y += x * weight[:, i]
+        elif shift < L:
+            y[:, shift:] += x[:, : L - shift] * weight[:, i]
+    return y
+
+
+def short_conv_step(x, state, weight):
+    """Single-token update of the rolling (B, C, K) state (convolution.py:85-109, non-CUDA
+    path): shift left, append x (B, 1, C), return sum_k state * weight as (B, 1, C)."""
+    state.copy_(torch.roll(state, shifts=-1, dims=-1))
+    state[:, :, -1] = x[:, 0]
+    return torch.einsum("bck,ck->bc", state, weight).to(x.dtype).unsqueeze(1)
