@@ -1,8 +1,300 @@
-// placeholder until the sliding-window kernels land
+// Sliding-window causal softmax attention for gfx950: prefill (MFMA) and decode step.
+//
+// Prefill.  One workgroup of four wavefronts covers 64 consecutive queries of one
+// (batch, head); wavefront w owns queries [q0+16w, q0+16w+16) and the 80 keys
+// [n0-64, n0+16) they can see (window <= 64 to the left plus the causal diagonal).
+//   S^T = K Q^T   : 5 key tiles x 2 MFMA 16x16x32 (head dim 64), operands loaded straight
+//                   from global memory (a lane's 8 consecutive bf16 of one row = 16 bytes).
+//   softmax       : S^T leaves the MFMA with lane <-> query and registers <-> keys, so the
+//                   row max / row sum are in-lane loops plus two cross-lane steps.
+//   O^T = V^T P^T : the accumulator layout of S^T is already the B-operand layout for a
+//                   product contracted over keys, so P never leaves registers.  V^T (lane
+//                   <-> channel, registers <-> keys) is the one operand that needs a
+//                   transpose; the workgroup stages its 128 keys of V through LDS,
+//                   transposed on the way in.
+// Whole-window softmax in one pass: 80 keys fit in registers, so no online rescaling.
+//
+// Decode.  One wavefront per (batch, head): lane <-> key for the scores, lane <-> channel
+// for the output, against the last w_left+1 rows of a linear cache.
 #include "common.hpp"
-extern "C" BASED_API int based_swa_prefill(const void*, const void*, const void*, void*, int64_t, int64_t, int64_t,
-    int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,
-    int, float, int, void*) { based::set_error("swa_prefill: not built yet"); return BASED_ERR_SHAPE; }
-extern "C" BASED_API int based_swa_step(const void*, const void*, const void*, void*, void*, void*, const int32_t*, int64_t,
-    int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,
-    int64_t, int64_t, int64_t, int, float, int, void*) { based::set_error("swa_step: not built yet"); return BASED_ERR_SHAPE; }
+
+namespace based {
+
+constexpr int kHeadDim = 64;
+constexpr int kQTile = 64;          // queries per workgroup
+constexpr int kVtStride = 136;      // bf16 elements per V^T row in LDS (128 + pad)
+
+__global__ __launch_bounds__(256) void swa_prefill_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
+    __bf16* __restrict__ o, int L, long q_sb, long q_sl, long q_sh, long k_sb, long k_sl,
+    long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh, int w_left,
+    float scale_log2e) {
+  __shared__ __align__(16) __bf16 s_vt[kHeadDim * kVtStride];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 15;   // query (B operand / accumulator column), or row of an A tile
+  const int grp = lane >> 4;   // 0..3: which 8 contraction slots / which 4 accumulator rows
+  const int q0 = blockIdx.x * kQTile;
+  const int h = blockIdx.y, b = blockIdx.z;
+
+  q += b * q_sb + h * q_sh;
+  k += b * k_sb + h * k_sh;
+  v += b * v_sb + h * v_sh;
+  o += b * o_sb + h * o_sh;
+
+  // ---- stage V^T for keys [q0-64, q0+64): thread t -> key t/2, channels 32*(t%2)..+32 ----
+  {
+    const int kk = tid >> 1, half = tid & 1;
+    const int key = q0 - 64 + kk;
+    const bool ok = key >= 0 && key < L;
+    const bf16x8* src = reinterpret_cast<const bf16x8*>(v + (long)key * v_sl + 32 * half);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (ok) x = src[c];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s_vt[(32 * half + 8 * c + i) * kVtStride + kk] = x[i];
+    }
+  }
+
+  // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
+  const int n0 = q0 + 16 * wave;            // first query of this wavefront
+  const int n = n0 + col;                   // this lane's query
+  bf16x8 bq[2];
+#pragma unroll
+  for (int ds = 0; ds < 2; ++ds) {
+    bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (n < L) x = *reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp);
+    bq[ds] = x;
+  }
+  f32x4 st[5];
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    const int key = n0 - 64 + 16 * i + col;  // A-tile row = key
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ds = 0; ds < 2; ++ds) {
+      bf16x8 a = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (key >= 0 && key < L)
+        a = *reinterpret_cast<const bf16x8*>(k + (long)key * k_sl + 32 * ds + 8 * grp);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[ds], acc, 0, 0, 0);
+    }
+    st[i] = acc;
+  }
+
+  // ---- masked softmax over keys; lane holds keys 16 i + 4 grp + r of query n ----
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < 5; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int key = n0 - 64 + 16 * i + 4 * grp + r;
+      const bool keep = key >= 0 && key <= n && key >= n - w_left;
+      const float s = keep ? st[i][r] * scale_log2e : -INFINITY;
+      st[i][r] = s;
+      mx = fmaxf(mx, s);
+    }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 5; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float p = __builtin_amdgcn_exp2f(st[i][r] - mx);  // exp2(-inf) = 0 for masked keys
+      st[i][r] = p;
+      sum += p;
+    }
+  sum += __shfl_xor(sum, 16, 64);
+  sum += __shfl_xor(sum, 32, 64);
+
+  __syncthreads();  // V^T staged
+
+  // ---- O^T = V^T P^T: 4 channel tiles x 3 key slabs of 32 (last slab half empty) ----
+  f32x4 ot[4];
+#pragma unroll
+  for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent for s = 2)
+    uint32_t pb[4];
+    pb[0] = pack_bf16(st[2 * s][0], st[2 * s][1]);
+    pb[1] = pack_bf16(st[2 * s][2], st[2 * s][3]);
+    if (s < 2) {
+      pb[2] = pack_bf16(st[2 * s + 1][0], st[2 * s + 1][1]);
+      pb[3] = pack_bf16(st[2 * s + 1][2], st[2 * s + 1][3]);
+    } else {
+      pb[2] = 0u;
+      pb[3] = 0u;
+    }
+    const bf16x8 bp = __builtin_bit_cast(bf16x8, *reinterpret_cast<const __attribute__((ext_vector_type(4))) uint32_t*>(pb));
+    const int kk0 = 16 * wave + 32 * s + 4 * grp;  // LDS key slot of operand slot 0
+#pragma unroll
+    for (int et = 0; et < 4; ++et) {
+      const __bf16* row = s_vt + (16 * et + col) * kVtStride;
+      bf16x4 lo = *reinterpret_cast<const bf16x4*>(row + kk0);
+      bf16x4 hi = {0, 0, 0, 0};
+      if (s < 2) hi = *reinterpret_cast<const bf16x4*>(row + kk0 + 16);
+      const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bp, ot[et], 0, 0, 0);
+    }
+  }
+
+  // ---- normalise and store: lane holds channels 16 et + 4 grp + r of query n ----
+  if (n < L) {
+    const float inv = 1.0f / sum;
+#pragma unroll
+    for (int et = 0; et < 4; ++et) {
+      uint32_t w2[2];
+      w2[0] = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
+      w2[1] = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
+      *reinterpret_cast<uint2*>(o + (long)n * o_sl + 16 * et + 4 * grp) = make_uint2(w2[0], w2[1]);
+    }
+  }
+}
+
+// One wavefront per (b, h).  Keys lo..pos, lo = max(0, pos - w_left); at most 65.
+__global__ __launch_bounds__(64) void swa_step_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k_new, const __bf16* __restrict__ v_new,
+    __bf16* __restrict__ kcache, __bf16* __restrict__ vcache, __bf16* __restrict__ o,
+    const int32_t* __restrict__ cache_seqlens, int pos_host, int H, int max_seqlen, long q_sb,
+    long q_sh, long kn_sb, long kn_sh, long vn_sb, long vn_sh, long o_sb, long o_sh, long c_sb,
+    long c_st, long c_sh, int w_left, float scale_log2e) {
+  __shared__ float s_q[kHeadDim];
+  const int lane = threadIdx.x;
+  const int bh = blockIdx.x;
+  const int b = bh / H, h = bh % H;
+  int pos = cache_seqlens ? cache_seqlens[b] : pos_host;
+  pos = __builtin_amdgcn_readfirstlane(pos);
+  if (pos < 0 || pos >= max_seqlen) return;  // out-of-range position: nothing to attend or write
+
+  const __bf16 kn = k_new[b * kn_sb + h * kn_sh + lane];
+  const __bf16 vn = v_new[b * vn_sb + h * vn_sh + lane];
+  __bf16* kc = kcache + b * c_sb + h * c_sh;
+  __bf16* vc = vcache + b * c_sb + h * c_sh;
+  kc[(long)pos * c_st + lane] = kn;
+  vc[(long)pos * c_st + lane] = vn;
+  s_q[lane] = to_f32(q[b * q_sb + h * q_sh + lane]);
+  __syncthreads();
+
+  const int lo = pos - w_left > 0 ? pos - w_left : 0;
+  const int nkeys = pos - lo + 1;  // 1..65, the last one is the new token itself
+
+  // scores: pass 0 -> key lo+lane, pass 1 -> key lo+64+lane (only lane 0 can be live)
+  float sc[2];
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int j = 64 * pass + lane;
+    float s = -INFINITY;
+    if (j < nkeys) {
+      const __bf16* row = (j == nkeys - 1) ? (k_new + b * kn_sb + h * kn_sh) : (kc + (long)(lo + j) * c_st);
+      float acc = 0.f;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(row + 8 * c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(to_f32(x[i]), s_q[8 * c + i], acc);
+      }
+      s = acc * scale_log2e;
+    }
+    sc[pass] = s;
+  }
+  float mx = fmaxf(sc[0], sc[1]);
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+  sc[0] = __builtin_amdgcn_exp2f(sc[0] - mx);
+  sc[1] = __builtin_amdgcn_exp2f(sc[1] - mx);
+  const float denom = wave_sum(sc[0] + sc[1]);
+
+  // output channel = lane
+  float acc = 0.f;
+  const int ncached = nkeys - 1;
+  for (int j0 = 0; j0 < ncached; j0 += 8) {
+    float vv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int j = j0 + u;
+      vv[u] = j < ncached ? to_f32(vc[(long)(lo + j) * c_st + lane]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int j = j0 + u;
+      const float p = __shfl(sc[j >> 6], j & 63, 64);
+      acc = __builtin_fmaf(j < ncached ? p : 0.f, vv[u], acc);
+    }
+  }
+  {
+    const int j = nkeys - 1;
+    const float p = __shfl(sc[j >> 6], j & 63, 64);
+    acc = __builtin_fmaf(p, to_f32(vn), acc);
+  }
+  o[b * o_sb + h * o_sh + lane] = (__bf16)(acc / denom);
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace based
+
+extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const void* v, void* o,
+                                           int64_t B, int64_t H, int64_t L,
+                                           int64_t q_sb, int64_t q_sl, int64_t q_sh,
+                                           int64_t k_sb, int64_t k_sl, int64_t k_sh,
+                                           int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                                           int64_t o_sb, int64_t o_sl, int64_t o_sh,
+                                           int w_left, float scale, int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(q && k && v && o, BASED_ERR_ARG, "swa_prefill: null pointer argument");
+  BASED_REQUIRE(B >= 0 && H > 0 && L >= 0, BASED_ERR_ARG, "swa_prefill: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_prefill: only bf16 is supported");
+  BASED_REQUIRE(w_left >= 0 && w_left <= 64, BASED_ERR_SHAPE,
+                "swa_prefill: left window %d unsupported (0..64)", w_left);
+  BASED_REQUIRE(H < 65536 && B < 65536 && L < (1ll << 31) - 64, BASED_ERR_SHAPE,
+                "swa_prefill: grid too large");
+  const int64_t strides[] = {q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh};
+  for (int64_t s : strides)
+    BASED_REQUIRE(s % 8 == 0, BASED_ERR_ALIGN, "swa_prefill: strides must be multiples of 8 elements");
+  BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o), BASED_ERR_ALIGN,
+                "swa_prefill: tensors must be 16-byte aligned");
+  if (B == 0 || L == 0) return BASED_OK;
+  dim3 grid((unsigned)((L + kQTile - 1) / kQTile), (unsigned)H, (unsigned)B), block(256);
+  hipLaunchKernelGGL(swa_prefill_kernel, grid, block, 0, static_cast<hipStream_t>(stream),
+                     (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o, (int)L, q_sb,
+                     q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh, w_left,
+                     scale * 1.4426950408889634f);
+  return check_launch("swa_prefill");
+}
+
+extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const void* v_new,
+                                        void* kcache, void* vcache, void* o,
+                                        const int32_t* cache_seqlens, int64_t pos_host,
+                                        int64_t B, int64_t H, int64_t max_seqlen,
+                                        int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
+                                        int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
+                                        int64_t c_sb, int64_t c_st, int64_t c_sh,
+                                        int w_left, float scale, int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(q && k_new && v_new && kcache && vcache && o, BASED_ERR_ARG,
+                "swa_step: null pointer argument");
+  BASED_REQUIRE(B >= 0 && H > 0 && max_seqlen > 0, BASED_ERR_ARG, "swa_step: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_step: only bf16 is supported");
+  BASED_REQUIRE(w_left >= 0 && w_left <= 64, BASED_ERR_SHAPE,
+                "swa_step: left window %d unsupported (0..64)", w_left);
+  BASED_REQUIRE(max_seqlen < (1ll << 31) && B * H < (1ll << 31), BASED_ERR_SHAPE, "swa_step: sizes too large");
+  if (!cache_seqlens)
+    BASED_REQUIRE(pos_host >= 0 && pos_host < max_seqlen, BASED_ERR_ARG,
+                  "swa_step: position %ld outside the cache (max_seqlen %ld)", (long)pos_host,
+                  (long)max_seqlen);
+  BASED_REQUIRE(c_sb % 8 == 0 && c_st % 8 == 0 && c_sh % 8 == 0 && kn_sb % 8 == 0 && kn_sh % 8 == 0,
+                BASED_ERR_ALIGN, "swa_step: cache and k_new strides must be multiples of 8 elements");
+  BASED_REQUIRE(aligned16(kcache) && aligned16(k_new), BASED_ERR_ALIGN,
+                "swa_step: kcache and k_new must be 16-byte aligned");
+  if (B == 0) return BASED_OK;
+  hipLaunchKernelGGL(swa_step_kernel, dim3((unsigned)(B * H)), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), (const __bf16*)q, (const __bf16*)k_new,
+                     (const __bf16*)v_new, (__bf16*)kcache, (__bf16*)vcache, (__bf16*)o, cache_seqlens,
+                     (int)pos_host, (int)H, (int)max_seqlen, q_sb, q_sh, kn_sb, kn_sh, vn_sb, vn_sh,
+                     o_sb, o_sh, c_sb, c_st, c_sh, w_left, scale * 1.4426950408889634f);
+  return check_launch("swa_step");
+}

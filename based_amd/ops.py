@@ -63,3 +63,59 @@ def linear_attn_step(q, k, v, kv_state, k_state, eps: float = 1e-12) -> torch.Te
             v.stride(0), v.stride(1), y.stride(0), y.stride(1),
             float(eps), _dtype_code(q), _stream_ptr(q)))
     return y
+
+
+def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None) -> torch.Tensor:
+    """Sliding-window causal attention.  q, k, v: (B, L, H, 64) bf16 (any strides with the
+    last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i]."""
+    _require_cuda(q, k, v)
+    B, L, H, D = q.shape
+    if D != 64 or k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)} (head dim 64)")
+    for t in (q, k, v):
+        if t.stride(-1) != 1:
+            raise ValueError("innermost dimension must be contiguous")
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    o = torch.empty(B, L, H, D, dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().based_swa_prefill(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+            int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
+    return o
+
+
+def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None) -> torch.Tensor:
+    """Decode step.  q, k_new, v_new: (B, 1, H, 64) bf16; kv_cache (B, max_seqlen, 2, H, 64)
+    bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.
+    pos: int (same for the whole batch) or an int32 device tensor of B positions."""
+    _require_cuda(q, k_new, v_new, kv_cache)
+    B, one, H, D = q.shape
+    if one != 1 or D != 64 or k_new.shape != q.shape or v_new.shape != q.shape:
+        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k_new.shape)} v{tuple(v_new.shape)}")
+    if kv_cache.dim() != 5 or kv_cache.shape[0] < B or kv_cache.shape[2] != 2 or tuple(kv_cache.shape[3:]) != (H, D):
+        raise ValueError(f"bad cache shape {tuple(kv_cache.shape)}")
+    if kv_cache.dtype != q.dtype or kv_cache.stride(-1) != 1:
+        raise ValueError("cache must share q's dtype and have a contiguous last dim")
+    for t in (q, k_new, v_new):
+        if t.stride(-1) != 1:
+            raise ValueError("innermost dimension must be contiguous")
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    if isinstance(pos, torch.Tensor):
+        if pos.dtype != torch.int32 or not pos.is_cuda or pos.numel() < B or not pos.is_contiguous():
+            raise ValueError("cache_seqlens must be a contiguous int32 device tensor with B entries")
+        seq_ptr, pos_host = pos.data_ptr(), 0
+    else:
+        seq_ptr, pos_host = None, int(pos)
+    o = torch.empty(B, 1, H, D, dtype=q.dtype, device=q.device)
+    kc, vc = kv_cache[:, :, 0], kv_cache[:, :, 1]
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().based_swa_step(
+            q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(),
+            seq_ptr, pos_host, B, H, kv_cache.shape[1],
+            q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
+            v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
+            kc.stride(0), kc.stride(1), kc.stride(2),
+            int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
+    return o
