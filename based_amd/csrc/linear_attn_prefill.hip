@@ -1,6 +1,512 @@
-// placeholder until the prefill kernel lands
+// Causal Taylor linear attention over a whole sequence (prefill) for gfx950.
+//
+// Two kernels behind one entry point:
+//
+//  * lin_prefill_mfma_kernel (bf16 in/out): chunked scan, 64 tokens per chunk, ONE wavefront
+//    per (batch, head, 64-channel block) that keeps the whole running state in MFMA
+//    accumulators for the length of the sequence (no state traffic to LDS or HBM).
+//
+//      within a chunk   A = tril(1 + s + s^2/2), s = q.k/4, from a K=16 MFMA on the raw
+//                       16-dim q, k (never expanding the features), then O^T += V^T A^T
+//      across chunks    O^T += S^T psi(q)^T   and afterwards   S += psi(k)^T V
+//
+//    psi is a 160-slot SYMMETRIC packing of the 273 TaylorExp features (x_i x_j and x_j x_i
+//    are one slot with doubled weight), laid out by circular distance t: slot (t, j) holds
+//    x_j * x_{(j - t) mod 16} for t = 0..7; tile 8 holds the 8 distance-8 pairs, the constant
+//    feature and 7 zeros; tile 9 the linear terms.  With that layout
+//      - psi(k)^T (lane <-> slot, registers <-> tokens) is one DPP row-rotate multiply per
+//        element, with the weights folded into a pre-scaled copy of k;
+//      - psi(q)^T (lane <-> token, registers <-> slots) is a product of two registers with
+//        compile-time indices, because each lane group keeps q rotated by 4*group.
+//    The normaliser is carried as a 65th value channel of ones, so numerator and
+//    denominator come out of the same MFMAs.  The state contracts with psi(q) straight from
+//    its accumulator registers (accumulator layout == B/A operand layout for a product
+//    contracted over the accumulator's row index); only V needs a transpose (through LDS).
+//    At the end the 160-slot state is expanded to the (dv, 273) decode layout.
+//
+//  * lin_prefill_f32_kernel (fp32 or bf16 in/out, fp32 arithmetic throughout): a plain
+//    recurrent evaluation, four tokens per round.  It serves fp32 callers (tolerance 1e-4
+//    is out of reach of bf16 operands) and is an independent second implementation that
+//    the tests compare the MFMA kernel against at sizes the CPU cannot reach.
+#include <type_traits>
+#include <utility>
+
 #include "common.hpp"
-extern "C" BASED_API int based_linear_attn_prefill(const void*, const void*, const void*, void*, float*, float*,
-    int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t,
-    int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, float, int, void*) {
-  based::set_error("linear_attn_prefill: not built yet"); return BASED_ERR_SHAPE; }
+
+namespace based {
+
+// ------------------------------------------------------------------------------------------
+// compile-time loop: body(std::integral_constant<int, I>{}) for I in [0, N)
+// ------------------------------------------------------------------------------------------
+template <int N, typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl<N>(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+template <int T>
+__device__ __forceinline__ float row_ror(float x) {
+  // value of lane (i - T) mod 16 within each row of 16 lanes
+  static_assert(T >= 1 && T <= 15, "rotation out of range");
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + T, 0xf, 0xf, false));
+}
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+__device__ __forceinline__ bf16x8 pack8(const float (&x)[8]) {
+  u32x4 w = {pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7])};
+  return __builtin_bit_cast(bf16x8, w);
+}
+
+__device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+constexpr int kChunk = 64;       // tokens per chunk
+constexpr int kFTiles = 10;      // 160 symmetric feature slots = 10 tiles of 16
+constexpr int kETiles = 5;       // 64 value channels + 1 normaliser channel (tile 4, column 0)
+constexpr int kVtStride = 72;    // bf16 per V^T row in LDS: 64 token slots + pad
+constexpr float kSqrt2 = 1.4142135623730951f;
+
+// Position of chunk-relative token tau inside a V^T row / inside the contraction slots:
+// slab s = tau/32 holds, for lane group g, slots jj = 0..7 <-> tokens 32s + 16(jj/4) + 4g + jj%4,
+// which is the order in which accumulator rows (4g + r of tiles 2s, 2s+1) turn into operand slots.
+__device__ __forceinline__ int token_slot(int tau) {
+  const int s = tau >> 5, rem = tau & 31;
+  return 32 * s + 8 * ((rem & 15) >> 2) + 4 * (rem >> 4) + (rem & 3);
+}
+__device__ __forceinline__ int slot_token(int s, int g, int jj) {
+  return 32 * s + 16 * (jj >> 2) + 4 * g + (jj & 3);
+}
+
+__global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
+    __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
+    int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
+    long v_sl, long y_sb, long y_sh, long y_sl, float eps) {
+  __shared__ __align__(16) __bf16 s_q[kChunk * kFeat];
+  __shared__ __align__(16) __bf16 s_k[kChunk * kFeat];
+  __shared__ __align__(16) __bf16 s_vt[64 * kVtStride];
+
+  const int lane = threadIdx.x;
+  const int col = lane & 15;
+  const int grp = lane >> 4;
+  const long bh = blockIdx.x;
+  const int eb = blockIdx.y;  // 64-channel block of the value dimension
+  const int b = (int)(bh / H), h = (int)(bh % H);
+
+  q += b * q_sb + h * q_sh;
+  k += b * k_sb + h * k_sh;
+  v += b * v_sb + h * v_sh + 64 * eb;
+  y += b * y_sb + h * y_sh + 64 * eb;
+
+  // running state S[slot tile][channel tile]: lane <-> channel 16 et + col, regs <-> slots 4 grp + r
+  f32x4 S[kFTiles][kETiles];
+#pragma unroll
+  for (int ft = 0; ft < kFTiles; ++ft)
+#pragma unroll
+    for (int et = 0; et < kETiles; ++et) S[ft][et] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // operand of the normaliser channel: row/column 64 (col == 0) is all ones
+  const uint32_t one2 = col == 0 ? 0x3F803F80u : 0u;
+  const bf16x8 ones_op = __builtin_bit_cast(bf16x8, u32x4{one2, one2, one2, one2});
+  const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
+
+  for (int t0 = 0; t0 < L; t0 += kChunk) {
+    const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
+
+    // ---------------- stage the chunk: q, k row-major, v transposed, into LDS ----------------
+    {
+      // q, k: 64 rows x 32 B; lane <-> row
+      u32x4 qa = {0, 0, 0, 0}, qb = {0, 0, 0, 0}, ka = {0, 0, 0, 0}, kb = {0, 0, 0, 0};
+      if (lane < ntok) {
+        const u32x4* qs = reinterpret_cast<const u32x4*>(q + (long)(t0 + lane) * q_sl);
+        const u32x4* ks = reinterpret_cast<const u32x4*>(k + (long)(t0 + lane) * k_sl);
+        qa = qs[0]; qb = qs[1]; ka = ks[0]; kb = ks[1];
+      }
+      u32x4* dq = reinterpret_cast<u32x4*>(s_q + lane * kFeat);
+      u32x4* dk = reinterpret_cast<u32x4*>(s_k + lane * kFeat);
+      dq[0] = qa; dq[1] = qb; dk[0] = ka; dk[1] = kb;
+      // v: 64 rows x 128 B; pass i: lane <-> (token 8 i + lane/8, channels 8 (lane%8) ..+8)
+      bf16x8 vv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int tau = 8 * i + (lane >> 3);
+        bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (lane & 7));
+        vv[i] = x;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int pos = token_slot(8 * i + (lane >> 3));
+#pragma unroll
+        for (int c = 0; c < 8; ++c) s_vt[(8 * (lane & 7) + c) * kVtStride + pos] = vv[i][c];
+      }
+    }
+    __syncthreads();
+
+    // V^T operand tiles: lane <-> channel 16 et + col, slots <-> tokens of slab s
+    bf16x8 vt[4][2];
+#pragma unroll
+    for (int et = 0; et < 4; ++et)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        vt[et][s] = *reinterpret_cast<const bf16x8*>(s_vt + (16 * et + col) * kVtStride + 32 * s + 8 * grp);
+
+    // output accumulators O^T[channel tile][token tile]: lane <-> token 16 nt + col, regs <-> channel
+    f32x4 O[kETiles][4];
+#pragma unroll
+    for (int et = 0; et < kETiles; ++et)
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) O[et][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // ---------------- within the chunk: A^T = tril(1 + s + s^2/2)^T, O^T += V^T A^T ----------------
+    {
+      bf16x8 kq_a[4], kq_b[4];  // K tiles (A operand, rows = keys), Q tiles (B operand, cols = queries)
+      const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        kq_a[i] = low_half ? *reinterpret_cast<const bf16x8*>(s_k + (16 * i + col) * kFeat + 8 * grp) : zero8;
+        kq_b[i] = low_half ? *reinterpret_cast<const bf16x8*>(s_q + (16 * i + col) * kFeat + 8 * grp) : zero8;
+      }
+      static_for<4>([&](auto NT) {
+        constexpr int nt = decltype(NT)::value;
+        float p[4][4];  // [key tile][r]; tiles above the diagonal stay zero
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) p[mt][r] = 0.f;
+        static_for<nt + 1>([&](auto MT) {
+          constexpr int mt = decltype(MT)::value;
+          const f32x4 a = mfma(kq_a[mt], kq_b[nt], f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float pv = __builtin_fmaf(a[r], __builtin_fmaf(a[r], 1.0f / 32.0f, 0.25f), 1.0f);
+            if (mt == nt) pv = (4 * grp + r <= col) ? pv : 0.f;  // key <= query on the diagonal tile
+            p[mt][r] = pv;
+          }
+        });
+        static_for<nt / 2 + 1>([&](auto SS) {
+          constexpr int s = decltype(SS)::value;
+          const float pb[8] = {p[2 * s][0], p[2 * s][1], p[2 * s][2], p[2 * s][3],
+                               p[2 * s + 1][0], p[2 * s + 1][1], p[2 * s + 1][2], p[2 * s + 1][3]};
+          const bf16x8 bp = pack8(pb);
+#pragma unroll
+          for (int et = 0; et < 4; ++et) O[et][nt] = mfma(vt[et][s], bp, O[et][nt]);
+          O[4][nt] = mfma(ones_op, bp, O[4][nt]);
+        });
+      });
+    }
+
+    // ---------------- across chunks: O^T += S^T psi(q)^T (state before this chunk) ----------------
+    {
+      // q of token 16 nt + col, rotated by 4 grp: qr[nt][r] = q[(4 grp + r) mod 16]
+      float qr[4][16];
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const bf16x4 x = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + ((4 * grp + 4 * i) & 15));
+#pragma unroll
+          for (int c = 0; c < 4; ++c) qr[nt][4 * i + c] = to_f32(x[c]);
+        }
+      const float fix8_0 = (grp == 2) ? 1.0f : 0.0f;  // slot (tile 8, position 8) = constant feature
+
+      static_for<5>([&](auto SG) {
+        constexpr int sg = decltype(SG)::value;  // slab of 32 slots = slot tiles 2 sg, 2 sg + 1
+        bf16x8 sa[kETiles];
+#pragma unroll
+        for (int et = 0; et < kETiles; ++et) {
+          const float x[8] = {S[2 * sg][et][0], S[2 * sg][et][1], S[2 * sg][et][2], S[2 * sg][et][3],
+                              S[2 * sg + 1][et][0], S[2 * sg + 1][et][1], S[2 * sg + 1][et][2], S[2 * sg + 1][et][3]};
+          sa[et] = pack8(x);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+          float f[8];
+          static_for<8>([&](auto JJ) {
+            constexpr int jj = decltype(JJ)::value;
+            constexpr int t = 2 * sg + jj / 4;  // slot tile
+            constexpr int c = jj % 4;           // position 4 grp + c
+            const float own = qr[nt][c];
+            if constexpr (t == 0) {
+              f[jj] = own * own;
+            } else if constexpr (t <= 7) {
+              f[jj] = own * qr[nt][(c - t) & 15];
+            } else if constexpr (t == 8) {
+              const float prod = own * qr[nt][(c - 8) & 15];
+              f[jj] = low_half ? prod : (c == 0 ? fix8_0 : 0.0f);
+            } else {
+              f[jj] = own;
+            }
+          });
+          const bf16x8 bq = pack8(f);
+#pragma unroll
+          for (int et = 0; et < kETiles; ++et) O[et][nt] = mfma(sa[et], bq, O[et][nt]);
+        }
+      });
+    }
+
+    // ---------------- normalise and store the chunk's outputs ----------------
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const float z = __shfl(O[4][nt][0], col, 64);  // denominator sits in lane group 0, register 0
+      const float inv = 1.0f / (z + eps);
+      const int tau = 16 * nt + col;
+      if (tau < ntok) {
+#pragma unroll
+        for (int et = 0; et < 4; ++et) {
+          const uint32_t w0 = pack_bf16(O[et][nt][0] * inv, O[et][nt][1] * inv);
+          const uint32_t w1 = pack_bf16(O[et][nt][2] * inv, O[et][nt][3] * inv);
+          *reinterpret_cast<uint2*>(y + (long)(t0 + tau) * y_sl + 16 * et + 4 * grp) = make_uint2(w0, w1);
+        }
+      }
+    }
+
+    // ---------------- state update: S += psi(k)^T V over the chunk's tokens ----------------
+    {
+      // lane <-> slot position j = col; registers <-> the 8 token slots of each slab
+      float kraw[2][8], k16[2][8], cst[2][8];
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+          const int tau = slot_token(s, grp, jj);
+          const float x = to_f32(s_k[tau * kFeat + col]);
+          kraw[s][jj] = x;
+          k16[s][jj] = x * (1.0f / 16.0f);
+          cst[s][jj] = (col == 8 && tau < ntok) ? 1.0f : 0.0f;  // constant feature, real tokens only
+        }
+      static_for<kFTiles>([&](auto FT) {
+        constexpr int t = decltype(FT)::value;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          float f[8];
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            if constexpr (t == 0) {
+              f[jj] = kraw[s][jj] * k16[s][jj] * 0.5f;
+            } else if constexpr (t <= 7) {
+              f[jj] = row_ror<t>(kraw[s][jj]) * k16[s][jj];
+            } else if constexpr (t == 8) {
+              const float prod = row_ror<8>(kraw[s][jj]) * k16[s][jj];
+              f[jj] = col < 8 ? prod : cst[s][jj];
+            } else {
+              f[jj] = kraw[s][jj] * 0.25f;
+            }
+          }
+          const bf16x8 ak = pack8(f);
+#pragma unroll
+          for (int et = 0; et < 4; ++et) S[t][et] = mfma(ak, vt[et][s], S[t][et]);
+          S[t][4] = mfma(ak, ones_op, S[t][4]);
+        }
+      });
+    }
+    __syncthreads();  // LDS is overwritten by the next chunk
+  }
+
+  // ---------------- expand the 160-slot state into the (dv, 273) decode layout ----------------
+  if (kv_state != nullptr) {
+    float* ks_row = k_state + bh * kExp;
+    static_for<kFTiles>([&](auto FT) {
+      constexpr int t = decltype(FT)::value;
+#pragma unroll
+      for (int et = 0; et < kETiles; ++et) {
+        float* row;
+        bool live;
+        if (et < 4) {
+          row = kv_state + (bh * dv + 64 * eb + 16 * et + col) * kExp;
+          live = true;
+        } else {
+          row = ks_row;
+          live = (col == 0) && (eb == 0);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int j = 4 * grp + r;
+          const float x = S[t][et][r];
+          if (!live) continue;
+          if constexpr (t == 0) {
+            row[1 + kFeat + 17 * j] = x * (4.0f * kSqrt2);
+          } else if constexpr (t <= 7) {
+            const int pj = (j - t) & 15;
+            row[1 + kFeat + 16 * j + pj] = x * (2.0f * kSqrt2);
+            row[1 + kFeat + 16 * pj + j] = x * (2.0f * kSqrt2);
+          } else if constexpr (t == 8) {
+            if (j < 8) {
+              row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
+              row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
+            } else if (j == 8) {
+              row[0] = x;
+            }
+          } else {
+            row[1 + j] = x * 2.0f;
+          }
+        }
+      }
+    });
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// fp32-arithmetic recurrent kernel.  Workgroup = (b, h, 64-channel block), 256 threads:
+// thread (e = tid % 64, fg = tid / 64) owns state entries S[f][e] for f = 4 i + fg.
+// ------------------------------------------------------------------------------------------
+constexpr int kRound = 4;                       // tokens per synchronisation round
+constexpr int kOwn = (kExp + 3) / 4;            // 69 state entries per thread
+
+__device__ __forceinline__ float phi_full(const float* x, int f) {
+  if (f == 0) return 1.0f;
+  if (f <= kFeat) return x[f - 1] * 0.5f;
+  const int g = f - 1 - kFeat;
+  return x[g >> 4] * x[g & 15] * 0.17677669529663687f;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lin_prefill_f32_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ y,
+    float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L, int dv, long q_sb,
+    long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh, long v_sl,
+    long y_sb, long y_sh, long y_sl, float eps) {
+  __shared__ float s_x[kRound][2][kFeat];          // [token][0 = k, 1 = q]
+  __shared__ float s_v[kRound][64];
+  __shared__ float s_phi[kRound][2][kExp + 3];
+  __shared__ float s_part[kRound][4][64];
+  __shared__ float s_den[kRound][4];
+
+  const int tid = threadIdx.x;
+  const int e = tid & 63, fg = tid >> 6;
+  const long bh = blockIdx.x;
+  const int eb = blockIdx.y;
+  const int b = (int)(bh / H), h = (int)(bh % H);
+  const int ew = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // live channels in this block
+  q += b * q_sb + h * q_sh;
+  k += b * k_sb + h * k_sh;
+  v += b * v_sb + h * v_sh + 64 * eb;
+  y += b * y_sb + h * y_sh + 64 * eb;
+
+  float S[kOwn];
+#pragma unroll
+  for (int i = 0; i < kOwn; ++i) S[i] = 0.f;
+  float ks0 = 0.f, ks1 = 0.f;  // normaliser state for features tid and tid + 256
+
+  for (int t0 = 0; t0 < L; t0 += kRound) {
+    const int nt = L - t0 < kRound ? L - t0 : kRound;
+    if (tid < kRound * 2 * kFeat) {
+      const int tt = tid / (2 * kFeat), which = (tid / kFeat) & 1, i = tid % kFeat;
+      float x = 0.f;
+      if (tt < nt) x = to_f32((which ? q : k)[(long)(t0 + tt) * (which ? q_sl : k_sl) + i]);
+      s_x[tt][which][i] = x;
+    }
+    {
+      const int tt = tid >> 6;
+      float x = 0.f;
+      if (tt < nt && e < ew) x = to_f32(v[(long)(t0 + tt) * v_sl + e]);
+      s_v[tt][e] = x;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < kRound * 2 * kExp; idx += 256) {
+      const int tt = idx / (2 * kExp), rem = idx % (2 * kExp);
+      const int which = rem / kExp, f = rem % kExp;
+      s_phi[tt][which][f] = phi_full(s_x[tt][which], f);
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float ve = s_v[tt][e];
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < kOwn; ++i) {
+        const int f = 4 * i + fg;
+        if (f < kExp) {
+          S[i] = __builtin_fmaf(s_phi[tt][0][f], ve, S[i]);
+          acc = __builtin_fmaf(s_phi[tt][1][f], S[i], acc);
+        }
+      }
+      s_part[tt][fg][e] = acc;
+      ks0 += s_phi[tt][0][tid];
+      float dpart = s_phi[tt][1][tid] * ks0;
+      if (tid + 256 < kExp) {
+        ks1 += s_phi[tt][0][tid + 256];
+        dpart = __builtin_fmaf(s_phi[tt][1][tid + 256], ks1, dpart);
+      }
+      dpart = wave_sum(dpart);
+      if (e == 0) s_den[tt][fg] = dpart;
+    }
+    __syncthreads();
+    {
+      const int tt = tid >> 6;
+      if (tt < nt && e < ew) {
+        const float num = s_part[tt][0][e] + s_part[tt][1][e] + s_part[tt][2][e] + s_part[tt][3][e];
+        const float den = s_den[tt][0] + s_den[tt][1] + s_den[tt][2] + s_den[tt][3];
+        y[(long)(t0 + tt) * y_sl + e] = from_f32<T>(num / (den + eps));
+      }
+    }
+    __syncthreads();
+  }
+
+  if (kv_state != nullptr) {
+    if (e < ew) {
+      float* row = kv_state + (bh * dv + 64 * eb + e) * kExp;
+#pragma unroll
+      for (int i = 0; i < kOwn; ++i) {
+        const int f = 4 * i + fg;
+        if (f < kExp) row[f] = S[i];
+      }
+    }
+    if (eb == 0) {
+      k_state[bh * kExp + tid] = ks0;
+      if (tid + 256 < kExp) k_state[bh * kExp + tid + 256] = ks1;
+    }
+  }
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace based
+
+extern "C" BASED_API int based_linear_attn_prefill(
+    const void* q, const void* k, const void* v, void* y, float* kv_state, float* k_state, int64_t B,
+    int64_t H, int64_t L, int64_t dv, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+    int64_t k_sh, int64_t k_sl, int64_t v_sb, int64_t v_sh, int64_t v_sl, int64_t y_sb, int64_t y_sh,
+    int64_t y_sl, float eps, int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(q && k && v && y, BASED_ERR_ARG, "linear_attn_prefill: null pointer argument");
+  BASED_REQUIRE((kv_state == nullptr) == (k_state == nullptr), BASED_ERR_ARG,
+                "linear_attn_prefill: kv_state and k_state must both be given or both be NULL");
+  BASED_REQUIRE(B >= 0 && H > 0 && L >= 0, BASED_ERR_ARG, "linear_attn_prefill: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE,
+                "linear_attn_prefill: io_dtype %d unsupported", io_dtype);
+  BASED_REQUIRE(B * H < (1ll << 31) && L < (1ll << 31), BASED_ERR_SHAPE, "linear_attn_prefill: sizes too large");
+  if (B == 0) return BASED_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (io_dtype == BASED_BF16 && (dv == 64 || dv == 128)) {
+    const int64_t strides[] = {q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl};
+    for (int64_t st : strides)
+      BASED_REQUIRE(st % 8 == 0, BASED_ERR_ALIGN,
+                    "linear_attn_prefill: bf16 strides must be multiples of 8 elements (16 bytes)");
+    BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
+                  "linear_attn_prefill: tensors must be 16-byte aligned");
+    dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(64);
+    hipLaunchKernelGGL(lin_prefill_mfma_kernel, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
+                       (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
+                       q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
+    return check_launch("linear_attn_prefill");
+  }
+  BASED_REQUIRE(dv >= 1 && dv <= 1024, BASED_ERR_SHAPE, "linear_attn_prefill: head dim %ld unsupported",
+                (long)dv);
+  dim3 grid((unsigned)(B * H), (unsigned)((dv + 63) / 64)), block(256);
+  if (io_dtype == BASED_BF16) {
+    hipLaunchKernelGGL(lin_prefill_f32_kernel<__bf16>, grid, block, 0, s, (const __bf16*)q,
+                       (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L,
+                       (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
+  } else {
+    hipLaunchKernelGGL(lin_prefill_f32_kernel<float>, grid, block, 0, s, (const float*)q,
+                       (const float*)k, (const float*)v, (float*)y, kv_state, k_state, (int)H, (int)L,
+                       (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
+  }
+  return check_launch("linear_attn_prefill");
+}

@@ -119,3 +119,37 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
             kc.stride(0), kc.stride(1), kc.stride(2),
             int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
     return o
+
+
+def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False
+                        ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Causal Taylor linear attention.  q, k: (B, H, L, 16) raw; v: (B, H, L, dv); any strides
+    with the last dim contiguous (e.g. `(B, L, H, d).transpose(1, 2)` views).
+
+    Returns (y, kv_state, k_state): y (B, H, L, dv) in q's dtype, stored so that
+    `y.transpose(1, 2).reshape(B, L, H*dv)` is a free view; states are fp32
+    (B, H, 1, dv, 273) / (B, H, 1, 1, 273), or None unless return_state."""
+    _require_cuda(q, k, v)
+    B, H, L, d = q.shape
+    dv = v.shape[-1]
+    if d != FEATURE_DIM or k.shape != q.shape or tuple(v.shape[:3]) != (B, H, L):
+        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)} (feature dim 16)")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("q, k, v must share a dtype")
+    for t in (q, k, v):
+        if t.stride(-1) != 1:
+            raise ValueError("innermost dimension must be contiguous")
+    y = torch.empty(B, L, H, dv, dtype=q.dtype, device=q.device).transpose(1, 2)
+    kv_state = k_state = None
+    if return_state:
+        kv_state = torch.empty(B, H, 1, dv, EXPANDED_DIM, dtype=torch.float32, device=q.device)
+        k_state = torch.empty(B, H, 1, 1, EXPANDED_DIM, dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.lib().based_linear_attn_prefill(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
+            kv_state.data_ptr() if return_state else None, k_state.data_ptr() if return_state else None,
+            B, H, L, dv,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            v.stride(0), v.stride(1), v.stride(2), y.stride(0), y.stride(1), y.stride(2),
+            float(eps), _dtype_code(q), _stream_ptr(q)))
+    return y, kv_state, k_state
