@@ -1,0 +1,89 @@
+"""Gated short convolution mixer (plain PyTorch).  Filler so that the 27-layer Based stack can
+be assembled around the HIP mixers; mirrors based/models/mixers/convolution.py:16-218
+(non-CUDA branch): depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a
+rolling (B, D, K) state for decoding."""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+
+class ShortConvolution(nn.Module):
+    def __init__(self, d_model: int, kernel_size: int, layer_idx=None, conv_bias: bool = False,
+                 device=None, dtype=None, **kwargs):
+        super().__init__()
+        self.d_model = d_model
+        self.kernel_size = kernel_size
+        self.layer_idx = layer_idx
+        self.conv = nn.Conv1d(d_model, d_model, kernel_size=kernel_size, groups=d_model,
+                              padding=kernel_size - 1, bias=conv_bias, device=device, dtype=dtype)
+
+    def forward(self, x: torch.Tensor, inference_params=None, **kwargs):
+        """x (b, l, d) -> (b, l, d)."""
+        b, l, d = x.shape
+        if inference_params is not None:
+            if inference_params.seqlen_offset > 0:
+                return self.step(x, self._get_state(inference_params))
+            self._init_state(inference_params)
+            state = self._get_state(inference_params)
+            kk = min(self.kernel_size, l)
+            state[..., -kk:] = x[:, -kk:].transpose(1, 2)
+        return self.conv(x.transpose(1, 2))[..., :l].transpose(1, 2)
+
+    def step(self, x: torch.Tensor, state: torch.Tensor):
+        state.copy_(torch.roll(state, shifts=-1, dims=-1))
+        state[:, :, -1] = x.squeeze(1)
+        y = torch.einsum("bdk,dgk->bd", state, self.conv.weight).to(x.dtype)
+        if self.conv.bias is not None:
+            y = y + self.conv.bias
+        return y.unsqueeze(1)
+
+    def allocate_inference_cache(self, batch_size: int, max_seqlen: int, dtype=None, **kwargs):
+        return torch.zeros(batch_size, self.d_model, self.kernel_size, device=self.conv.weight.device,
+                           dtype=self.conv.weight.dtype if dtype is None else dtype)
+
+    def _init_state(self, inference_params):
+        outer, inner = self.layer_idx if isinstance(self.layer_idx, tuple) else (self.layer_idx, None)
+        d = inference_params.key_value_memory_dict
+        empty = self.allocate_inference_cache(inference_params.max_batch_size, inference_params.max_seqlen)
+        if inner is None:
+            if outer in d:
+                d[outer].copy_(empty)
+            else:
+                d[outer] = empty
+        else:
+            d.setdefault(outer, {})
+            if inner in d[outer]:
+                d[outer][inner].copy_(empty)
+            else:
+                d[outer][inner] = empty
+
+    def _get_state(self, inference_params):
+        d = inference_params.key_value_memory_dict
+        if isinstance(self.layer_idx, tuple):
+            return d[self.layer_idx[0]][self.layer_idx[1]]
+        return d[self.layer_idx]
+
+
+class BaseConv(nn.Module):
+    def __init__(self, d_model: int, l_max: int = 2048, kernel_size: int = 3, layer_idx=None, use_bias=True,
+                 expand_proj: int = 2, device=None, dtype=None, **kwargs):
+        super().__init__()
+        self.d_model = d_model
+        self.l_max = l_max
+        self.layer_idx = layer_idx
+        self.d_inner = expand_proj * d_model // 2
+        self.in_proj = nn.Linear(d_model, expand_proj * d_model, bias=use_bias, device=device, dtype=dtype)
+        self.out_proj = nn.Linear(self.d_inner, d_model, bias=use_bias, device=device, dtype=dtype)
+        self.conv = ShortConvolution(self.d_inner, kernel_size=kernel_size, layer_idx=(layer_idx, "conv"),
+                                     device=device, dtype=dtype)
+
+    def forward(self, u, position_ids=None, inference_params=None, *args, **kwargs):
+        u = self.in_proj(u)
+        u1, u2 = torch.split(u, self.d_inner, dim=-1)
+        u_conv = F.silu(self.conv(u1, inference_params=inference_params))
+        return self.out_proj(u_conv * u2)
+
+    def allocate_inference_cache(self, batch_size: int, max_seqlen: int, dtype=None, **kwargs):
+        return {"conv": self.conv.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)}

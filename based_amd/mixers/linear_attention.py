@@ -1,0 +1,162 @@
+"""Taylor linear attention mixer backed by the gfx950 kernels.
+
+Drop-in for based/models/mixers/linear_attention.py of the reference: same constructor
+arguments, parameter names (proj_q / proj_k / proj_v / out_proj), forward /
+recurrent_forward / allocate_inference_cache signatures and cache layout.  The q/k/v and
+output projections stay ordinary nn.Linear GEMMs; everything between them (feature map,
+causal product, normaliser, decode-state construction and update) is one HIP kernel call.
+There is no non-HIP path: tensors must live on the GPU.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+
+from .. import ops
+from ..generation import InferenceParams
+
+
+class FeatureMap(nn.Module):
+    """Parent feature map; identity (linear_attention.py:37-50)."""
+
+    def __init__(self, input_dim: int, **kwargs):
+        super().__init__()
+        self.input_dim = input_dim
+
+    def forward(self, x: torch.Tensor):
+        return x
+
+
+class TaylorExp(FeatureMap):
+    """2nd-order Taylor feature map, 16 -> 273 dims (linear_attention.py:52-75).
+
+    Kept as a module so configs and callers that name it keep working.  The mixer's kernels
+    evaluate the map on the fly from the raw 16-dim vectors and never call forward(); forward()
+    is the explicit expansion for callers that want phi(x) itself (e.g. to hand
+    recurrent_forward its pre-mapped arguments)."""
+
+    def __init__(self, input_dim: int, **kwargs):
+        super().__init__(input_dim, **kwargs)
+        self.r2 = math.sqrt(2)
+        self.rd = math.sqrt(input_dim)
+        self.rrd = math.sqrt(self.rd)
+
+    def forward(self, x: torch.Tensor):
+        x2 = (x.unsqueeze(-1) * x.unsqueeze(-2)).flatten(start_dim=-2) / self.r2
+        return torch.cat([x[..., :1] ** 0, x / self.rrd, x2 / self.rd], dim=-1)
+
+    def raw_from_mapped(self, fx: torch.Tensor) -> torch.Tensor:
+        """Inverse on the linear block: phi(x)[1:1+d] = x / d^(1/4)."""
+        return fx[..., 1:1 + self.input_dim] * self.rrd
+
+
+class LinearAttention(nn.Module):
+    def __init__(
+        self,
+        d_model: int,
+        feature_map: FeatureMap = None,
+        l_max: int = 2048,
+        feature_dim: int = 16,
+        head_dim: int = None,
+        num_heads: int = 16,
+        eps: float = 1e-12,
+        layer_idx: int = None,
+        parallel_implementation: str = "quadratic",
+        device=None,
+        dtype=None,
+        **kwargs,
+    ):
+        super().__init__()
+        factory_kwargs = {"device": device, "dtype": dtype}
+        self.layer_idx = layer_idx
+        self.d_model = d_model
+        self.l_max = l_max
+        self.eps = eps
+        # Accepted for config compatibility; there is exactly one implementation here.
+        self.parallel_implementation = parallel_implementation
+
+        self.num_heads = num_heads
+        self.head_dim = self.d_model // self.num_heads if head_dim is None else head_dim
+        self.feature_dim = feature_dim
+        if feature_map is None or isinstance(feature_map, type):
+            feature_map = TaylorExp(input_dim=feature_dim)
+        if not isinstance(feature_map, TaylorExp) or feature_map.input_dim != ops.FEATURE_DIM or feature_dim != ops.FEATURE_DIM:
+            raise NotImplementedError(
+                "the HIP kernels implement the TaylorExp feature map with feature_dim=16 only")
+        self.feature_map = feature_map
+
+        self.proj_q = nn.Linear(self.d_model, self.feature_dim * self.num_heads, bias=False, **factory_kwargs)
+        self.proj_k = nn.Linear(self.d_model, self.feature_dim * self.num_heads, bias=False, **factory_kwargs)
+        self.proj_v = nn.Linear(self.d_model, self.num_heads * self.head_dim, bias=False, **factory_kwargs)
+        self.out_proj = nn.Linear(self.num_heads * self.head_dim, self.d_model, bias=False, **factory_kwargs)
+
+    def forward(self, hidden_states: torch.Tensor, inference_params: InferenceParams = None, *args, **kwargs):
+        """hidden_states (b, l, d_model) -> (b, l, d_model)."""
+        b, l, _ = hidden_states.size()
+        q, k, v = self.proj_q(hidden_states), self.proj_k(hidden_states), self.proj_v(hidden_states)
+        q = q.view(b, l, self.num_heads, self.feature_dim).transpose(1, 2)
+        k = k.view(b, l, self.num_heads, self.feature_dim).transpose(1, 2)
+        v = v.view(b, l, self.num_heads, self.head_dim).transpose(1, 2)
+
+        self.is_inference = inference_params is not None
+        if inference_params is None:
+            return self.parallel_forward(hidden_states, q, k, v)
+        if inference_params.seqlen_offset > 0:
+            kv_state, k_state = self._get_inference_cache(inference_params)
+            return self._step(kv_state, k_state, q, k, v)
+        y, kv_state, k_state = self.parallel_forward(hidden_states, q, k, v)
+        if self.layer_idx in inference_params.key_value_memory_dict:
+            # pre-allocated caches (graph-style decoding) are filled in place
+            inference_params.key_value_memory_dict[self.layer_idx][0].copy_(kv_state)
+            inference_params.key_value_memory_dict[self.layer_idx][1].copy_(k_state)
+        else:
+            inference_params.key_value_memory_dict[self.layer_idx] = (kv_state, k_state)
+        return y
+
+    def parallel_forward(self, x: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+        """q, k: (b, h, l, 16) raw; v: (b, h, l, head_dim).  Returns out_proj(y), plus the decode
+        states when called on the inference path."""
+        is_inference = getattr(self, "is_inference", False)
+        y, kv_state, k_state = ops.linear_attn_prefill(q, k, v, eps=self.eps, return_state=is_inference)
+        b, h, l, d = y.shape
+        y = y.transpose(1, 2).reshape(b, l, h * d)  # 'b h l d -> b l (h d)', a view of the kernel output
+        out = self.out_proj(y.to(x.dtype))
+        if is_inference:
+            return out, kv_state, k_state
+        return out
+
+    def _step(self, kv_state, k_state, q, k, v):
+        y = ops.linear_attn_step(q, k, v, kv_state, k_state, eps=self.eps)
+        b, h, l, d = y.shape
+        return self.out_proj(y.transpose(1, 2).reshape(b, l, h * d))
+
+    def recurrent_forward(self, hidden_states: torch.Tensor, kv_state: torch.Tensor, k_state: torch.Tensor,
+                          q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, decay: torch.Tensor = None):
+        """Reference signature: q, k arrive ALREADY feature-mapped, shape (b, h, 1, 273); v is
+        (b, h, 1, head_dim).  The kernel fuses the map, so the raw vectors are recovered from
+        the linear block of phi (exact: a multiplication by 2)."""
+        b, h, l, d = q.shape
+        assert l == 1, f"q.shape is {q.shape} but should be ({b}, {h}, 1, {d})"
+        if d == self.feature_map.input_dim:
+            raw_q, raw_k = q, k
+        else:
+            raw_q, raw_k = self.feature_map.raw_from_mapped(q), self.feature_map.raw_from_mapped(k)
+        return self._step(kv_state, k_state, raw_q, raw_k, v)
+
+    def expanded_size(self):
+        return self.feature_dim ** 2 + self.feature_dim + 1
+
+    def allocate_inference_cache(self, batch_size: int, max_seqlen: int, dtype=None, **kwargs):
+        """(kv_state (B,H,1,head_dim,273), k_state (B,H,1,1,273)).  The states are carried in
+        fp32 whatever `dtype` asks for: the decode kernel accumulates in place in fp32."""
+        device = self.out_proj.weight.device
+        kv_state = torch.zeros(batch_size, self.num_heads, 1, self.head_dim, self.expanded_size(),
+                               dtype=torch.float32, device=device)
+        k_state = torch.zeros(batch_size, self.num_heads, 1, 1, self.expanded_size(),
+                              dtype=torch.float32, device=device)
+        return (kv_state, k_state)
+
+    def _get_inference_cache(self, inference_params: InferenceParams):
+        return inference_params.key_value_memory_dict[self.layer_idx]

@@ -1,0 +1,263 @@
+"""Minimal Based language-model stack around the HIP mixers (plain PyTorch glue).
+
+Just enough of based/models/gpt.py (create_mixer_cls :64-96, create_block :347-394, _init_weights
+:463-485, GPTModel :510-736, GPTLMHeadModel :739-827), block.py (:114-163), mlp.py (GatedMlp
+:99-157) and the RMSNorm closed form (based/ops/triton/layer_norm.py:117-118) to run the
+27-layer Based-360m shape end to end: embeddings -> [prenorm Block(mixer, SwiGLU MLP)] x N ->
+final norm -> tied LM head, with the generation cache threaded through.  Everything here is
+ordinary torch (GEMMs go to hipBLASLt); the sequence mixers are the HIP kernels.
+"""
+from __future__ import annotations
+
+import math
+from collections import namedtuple
+from functools import partial
+from types import SimpleNamespace
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .generation import GenerationMixin
+from .mixers.convolution import BaseConv
+from .mixers.linear_attention import LinearAttention, TaylorExp
+from .mixers.slide_attention import SlidingAttention
+
+# `_target_` strings accepted in mixer config dicts: the reference's own paths and this package's.
+_TARGETS = {
+    "based.models.mixers.linear_attention.LinearAttention": LinearAttention,
+    "based.models.mixers.linear_attention.TaylorExp": TaylorExp,
+    "based.models.mixers.slide_attention.SlidingAttention": SlidingAttention,
+    "based.models.mixers.convolution.BaseConv": BaseConv,
+    "based_amd.mixers.linear_attention.LinearAttention": LinearAttention,
+    "based_amd.mixers.linear_attention.TaylorExp": TaylorExp,
+    "based_amd.mixers.slide_attention.SlidingAttention": SlidingAttention,
+    "based_amd.mixers.convolution.BaseConv": BaseConv,
+}
+
+
+def _instantiate(spec: dict, *args, **extra):
+    """Tiny stand-in for hydra.utils.instantiate: nested dicts with `_target_` become objects."""
+    spec = dict(spec)
+    cls = _TARGETS[spec.pop("_target_")]
+    kwargs = {k: (_instantiate(v) if isinstance(v, dict) and "_target_" in v else v) for k, v in spec.items()}
+    kwargs.update(extra)
+    return cls(*args, **kwargs)
+
+
+class StackConfig(SimpleNamespace):
+    """Attribute bag with the GPT2Config fields the stack reads (gpt.py:58-61 lets the config
+    carry arbitrary attributes; so does this)."""
+
+    def __init__(self, **kw):
+        defaults = dict(
+            n_embd=1024, n_layer=27, n_head=16, n_inner=None, vocab_size=50277, pad_vocab_size_multiple=8,
+            layer_norm_epsilon=1e-5, rms_norm=True, residual_in_fp32=True, initializer_range=0.02,
+            tie_word_embeddings=True, activation_function="swiglu", mlp_fc1_bias=False, mlp_fc2_bias=False,
+            qkv_proj_bias=False, out_proj_bias=False, rotary_emb_fraction=0.0, rotary_emb_base=10000.0,
+            rotary_emb_interleaved=False, scale_attn_weights=True, max_position_embeddings=0,
+            mixer=None, alt_mixer=None, alt_mixer_layers=None, alt_mixer_2=None, alt_mixer_2_layers=None,
+        )
+        defaults.update(kw)
+        super().__init__(**defaults)
+
+    @property
+    def hidden_size(self):
+        return self.n_embd
+
+    @property
+    def num_hidden_layers(self):
+        return self.n_layer
+
+    @property
+    def num_attention_heads(self):
+        return self.n_head
+
+
+def based_360m_config(**overrides) -> StackConfig:
+    """Shape of the released Based-360m: BaseConv everywhere except Taylor linear attention at
+    layers {1,6,11,16,21} and sliding-window attention at {2,7,12,17,22}
+    (train/configs/experiment/reference/based-360m.yaml:53-65), window 64 to the left."""
+    cfg = dict(
+        n_embd=1024, n_layer=27, n_head=16, n_inner=2048, vocab_size=50277,
+        mixer={"_target_": "based.models.mixers.convolution.BaseConv", "l_max": 2048, "use_bias": True,
+               "expand_proj": 4, "kernel_size": 3},
+        alt_mixer={"_target_": "based.models.mixers.linear_attention.LinearAttention", "l_max": 2048,
+                   "feature_map": {"_target_": "based.models.mixers.linear_attention.TaylorExp", "input_dim": 16},
+                   "feature_dim": 16, "num_heads": 16},
+        alt_mixer_layers=[1, 6, 11, 16, 21],
+        alt_mixer_2={"_target_": "based.models.mixers.slide_attention.SlidingAttention", "window_size": 128,
+                     "num_heads": 16, "causal": True},
+        alt_mixer_2_layers=[2, 7, 12, 17, 22],
+    )
+    cfg.update(overrides)
+    return StackConfig(**cfg)
+
+
+def create_mixer_cls(config, layer_idx=None, device=None, dtype=None):
+    """Layer -> mixer routing of gpt.py:64-96."""
+    value = config.mixer
+    if config.alt_mixer_2_layers is not None and layer_idx in config.alt_mixer_2_layers:
+        value = config.alt_mixer_2
+    elif config.alt_mixer_layers is not None and layer_idx in config.alt_mixer_layers:
+        value = config.alt_mixer
+    if value is None:
+        raise NotImplementedError("plain multi-head attention layers are outside this build")
+    value = dict(value)
+    if "slide" in value["_target_"]:
+        head_dim = config.hidden_size // config.num_attention_heads
+        value.update({
+            "num_heads": config.num_attention_heads,
+            "qkv_proj_bias": config.qkv_proj_bias,
+            "out_proj_bias": config.out_proj_bias,
+            "softmax_scale": head_dim ** (-0.5) if config.scale_attn_weights else 1.0,
+            "causal": True,
+            "rotary_emb_dim": int(config.rotary_emb_fraction * head_dim),
+            "rotary_emb_base": config.rotary_emb_base,
+            "rotary_emb_interleaved": config.rotary_emb_interleaved,
+        })
+    return partial(_instantiate, value, device=device, dtype=dtype, layer_idx=layer_idx)
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, hidden_size, eps=1e-5, device=None, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size, device=device, dtype=dtype))
+
+    def forward(self, x):
+        xf = x.float()
+        rstd = torch.rsqrt(xf.square().mean(dim=-1, keepdim=True) + self.eps)
+        return (xf * rstd * self.weight.float()).to(self.weight.dtype)
+
+
+class GatedMlp(nn.Module):
+    """SwiGLU MLP: fc2(y * silu(gate)), y, gate = fc1(x).chunk(2) (mlp.py:141-151)."""
+
+    def __init__(self, in_features, hidden_features=None, bias1=False, bias2=False, multiple_of=256,
+                 device=None, dtype=None):
+        super().__init__()
+        hidden_features = hidden_features if hidden_features is not None else int(8 * in_features / 3)
+        hidden_features = (hidden_features + multiple_of - 1) // multiple_of * multiple_of
+        self.fc1 = nn.Linear(in_features, 2 * hidden_features, bias=bias1, device=device, dtype=dtype)
+        self.fc2 = nn.Linear(hidden_features, in_features, bias=bias2, device=device, dtype=dtype)
+
+    def forward(self, x):
+        y, gate = self.fc1(x).chunk(2, dim=-1)
+        return self.fc2(y * F.silu(gate))
+
+
+class Block(nn.Module):
+    """Prenorm block: add -> norm1 -> mixer -> add -> norm2 -> mlp, returning (hidden, residual)
+    (block.py:134-163, dropout-free)."""
+
+    def __init__(self, dim, mixer_cls, mlp_cls, norm_cls, residual_in_fp32=True, layer_idx=None):
+        super().__init__()
+        self.residual_in_fp32 = residual_in_fp32
+        self.layer_idx = layer_idx
+        self.mixer = mixer_cls(dim)
+        self.norm1 = norm_cls(dim)
+        self.mlp = mlp_cls(dim)
+        self.norm2 = norm_cls(dim)
+
+    def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None, **kwargs):
+        return self.mixer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
+
+    def forward(self, hidden_states, residual=None, mixer_kwargs=None, position_ids=None, decay=None):
+        residual = (hidden_states + residual) if residual is not None else hidden_states
+        hidden_states = self.norm1(residual.to(dtype=self.norm1.weight.dtype))
+        if self.residual_in_fp32:
+            residual = residual.to(torch.float32)
+        mixer_kwargs = mixer_kwargs or {}
+        if position_ids is not None or decay is not None:
+            hidden_states = self.mixer(hidden_states, position_ids=position_ids, decay=decay, **mixer_kwargs)
+        else:
+            hidden_states = self.mixer(hidden_states, **mixer_kwargs)
+        residual = hidden_states + residual
+        hidden_states = self.norm2(residual.to(dtype=self.norm2.weight.dtype))
+        if self.residual_in_fp32:
+            residual = residual.to(torch.float32)
+        return self.mlp(hidden_states), residual
+
+
+def _init_weights(module, n_layer, initializer_range=0.02):
+    if isinstance(module, nn.Linear):
+        nn.init.normal_(module.weight, std=initializer_range)
+        if module.bias is not None:
+            nn.init.zeros_(module.bias)
+    elif isinstance(module, nn.Embedding):
+        nn.init.normal_(module.weight, std=initializer_range)
+    for name, p in module.named_parameters():
+        if name in ["out_proj.weight", "fc2.weight"]:
+            nn.init.normal_(p, mean=0.0, std=initializer_range / math.sqrt(2 * n_layer))
+
+
+class GPTModel(nn.Module):
+    def __init__(self, config: StackConfig, device=None, dtype=None):
+        super().__init__()
+        fk = {"device": device, "dtype": dtype}
+        self.config = config
+        self.residual_in_fp32 = config.residual_in_fp32
+        vocab = math.ceil(config.vocab_size / config.pad_vocab_size_multiple) * config.pad_vocab_size_multiple
+        self.embeddings = nn.Module()
+        self.embeddings.word_embeddings = nn.Embedding(vocab, config.hidden_size, **fk)
+        if config.max_position_embeddings > 0:
+            self.embeddings.position_embeddings = nn.Embedding(config.max_position_embeddings, config.hidden_size, **fk)
+        norm_cls = partial(RMSNorm if config.rms_norm else nn.LayerNorm, eps=config.layer_norm_epsilon, **fk)
+        mlp_cls = partial(GatedMlp, hidden_features=config.n_inner, bias1=config.mlp_fc1_bias,
+                          bias2=config.mlp_fc2_bias, **fk)
+        self.layers = nn.ModuleList([
+            Block(config.hidden_size, create_mixer_cls(config, layer_idx=i, **fk), mlp_cls, norm_cls,
+                  residual_in_fp32=config.residual_in_fp32, layer_idx=i)
+            for i in range(config.num_hidden_layers)
+        ])
+        self.ln_f = norm_cls(config.hidden_size)
+        self.apply(partial(_init_weights, n_layer=config.num_hidden_layers,
+                           initializer_range=config.initializer_range))
+
+    def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None, **kwargs):
+        return {i: layer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
+                for i, layer in enumerate(self.layers)}
+
+    def forward(self, input_ids, position_ids=None, inference_params=None, stream=None):
+        hidden_states = self.embeddings.word_embeddings(input_ids)
+        if self.config.max_position_embeddings > 0:
+            if position_ids is None:
+                position_ids = torch.arange(input_ids.shape[1], dtype=torch.long, device=input_ids.device)
+            hidden_states = hidden_states + self.embeddings.position_embeddings(position_ids)
+        residual = None
+        mixer_kwargs = {}
+        if inference_params is not None:
+            mixer_kwargs["inference_params"] = inference_params
+            mixer_kwargs["stream"] = stream
+        for layer in self.layers:
+            hidden_states, residual = layer(hidden_states, residual=residual, position_ids=position_ids,
+                                            mixer_kwargs=mixer_kwargs)
+        residual = hidden_states + residual
+        return self.ln_f(residual.to(dtype=self.ln_f.weight.dtype))
+
+
+class GPTLMHeadModel(nn.Module, GenerationMixin):
+    def __init__(self, config: StackConfig, device=None, dtype=None):
+        super().__init__()
+        self.config = config
+        self.transformer = GPTModel(config, device=device, dtype=dtype)
+        vocab = self.transformer.embeddings.word_embeddings.num_embeddings
+        self.lm_head = nn.Linear(config.n_embd, vocab, bias=False, device=device, dtype=dtype)
+        self.apply(partial(_init_weights, n_layer=config.num_hidden_layers,
+                           initializer_range=config.initializer_range))
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.transformer.embeddings.word_embeddings.weight
+
+    def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None, **kwargs):
+        return self.transformer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
+
+    def forward(self, input_ids, position_ids=None, inference_params=None, num_last_tokens=0, stream=None, **kwargs):
+        assert input_ids.ndim == 2, f"Expected `input_ids` to have shape [b, slen], but got shape {input_ids.shape}"
+        hidden_states = self.transformer(input_ids, position_ids=position_ids, inference_params=inference_params,
+                                         stream=stream)
+        if num_last_tokens > 0:
+            hidden_states = hidden_states[:, -num_last_tokens:]
+        CausalLMOutput = namedtuple("CausalLMOutput", ["logits"])
+        return CausalLMOutput(logits=self.lm_head(hidden_states))

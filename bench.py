@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the Based sequence-mixer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa]
+
+Headline workload (`value`): the recurrent decode step of Taylor linear attention at
+B=128, H=16, dv=64 — fp32 kv_state (128,16,1,64,273) + k_state, initialised from a seeded
+512-token prefill, bf16 q/k/v ~ N(0,1), K consecutive single-token steps.  One "step" is
+one kernel launch over the whole batch; value = B / time-per-step (tokens/s, one layer).
+Inputs and state are resident in HBM before the timed region.
+
+The same JSON line also carries, as secondary objects, the linear-attention prefill at
+L=4096 (tokens/s and fraction of bf16 MFMA peak) and the sliding-window attention prefill +
+decode of the B=8, H=16, L=4096 configuration.
+
+`roofline.achieved` = algorithmic bytes (or FLOPs) per launch / average launch duration,
+timed with HIP events on the stream the kernels are launched on (torch's current stream).
+`cpu_baseline` = the CPU oracle (a PyTorch restatement of the reference arithmetic) timed on
+this host's cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+D_EXP = 273
+
+# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); None until a counter run for that kernel has been committed.
+MEASURED_TRAFFIC_BYTES = {
+    "lin_step_kernel": None,
+    "lin_prefill_mfma_kernel": None,
+    "swa_prefill_kernel": None,
+}
+
+
+def _events_ms(torch, fn, steps, warmup):
+    """Average milliseconds per call of fn(), HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return e0.elapsed_time(e1) / steps, wall
+
+
+def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512):
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(0)
+    # state from a seeded prefill (same kernels; q only shapes the outputs, not the state)
+    kp = torch.randn(B, H, prefill_len, 16, generator=g).bfloat16().to(dev)
+    vp = torch.randn(B, H, prefill_len, dv, generator=g).bfloat16().to(dev)
+    _, kv_state, k_state = ops.linear_attn_prefill(kp, kp, vp, return_state=True)
+    del kp, vp
+    n_in = 8  # distinct pre-generated inputs cycled through the steps
+    qs = [torch.randn(B, H, 1, 16, generator=g).bfloat16().to(dev) for _ in range(n_in)]
+    ks = [torch.randn(B, H, 1, 16, generator=g).bfloat16().to(dev) for _ in range(n_in)]
+    vs = [torch.randn(B, H, 1, dv, generator=g).bfloat16().to(dev) for _ in range(n_in)]
+    y = torch.empty(B, H, 1, dv, dtype=torch.bfloat16, device=dev)
+    from based_amd import _lib
+
+    lib = _lib.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    args = [(qs[i].data_ptr(), ks[i].data_ptr(), vs[i].data_ptr()) for i in range(n_in)]
+    it = [0]
+
+    def step():
+        a = args[it[0] % n_in]
+        it[0] += 1
+        rc = lib.based_linear_attn_step(a[0], a[1], a[2], kv_state.data_ptr(), k_state.data_ptr(), y.data_ptr(),
+                                        B, H, dv, H * 16, 16, H * 16, 16, H * dv, dv, H * dv, dv,
+                                        1e-12, 0, stream)
+        if rc:
+            _lib.check(rc)
+
+    ms, wall = _events_ms(torch, step, steps, warmup)
+    bytes_per_launch = B * H * (2 * D_EXP * dv * 4 + 2 * D_EXP * 4 + (2 * 16 + 2 * dv) * 2)
+    gbs = bytes_per_launch / (ms * 1e-3) / 1e9
+    assert torch.isfinite(y.float()).all() and torch.isfinite(kv_state).all()
+    return {
+        "tok_s": B / (ms * 1e-3),
+        "ms": ms,
+        "wall_ms": wall,
+        "roofline": {"kernel": "lin_step_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"],
+                     "algorithmic_bytes_per_launch": bytes_per_launch},
+        "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, bf16 q/k/v",
+    }
+
+
+def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(1)
+    # (B, L, H*d) projection layout viewed (B, H, L, d), as the module hands it over
+    q = torch.randn(B, L, H, 16, generator=g).bfloat16().to(dev).transpose(1, 2)
+    k = torch.randn(B, L, H, 16, generator=g).bfloat16().to(dev).transpose(1, 2)
+    v = torch.randn(B, L, H, dv, generator=g).bfloat16().to(dev).transpose(1, 2)
+    ms, _ = _events_ms(torch, lambda: ops.linear_attn_prefill(q, k, v, return_state=True), steps, warmup)
+    flops = B * L * H * (4 * D_EXP * dv + 4 * D_EXP)
+    byts = B * L * H * (2 * 16 + 2 * dv) * 2
+    tf = flops / (ms * 1e-3) / 1e12
+    return {
+        "tok_s": B * L / (ms * 1e-3), "ms": ms, "B": B, "L": L, "dv": dv,
+        "roofline": {"kernel": "lin_prefill_mfma_kernel", "bound": "mfma", "achieved": round(tf, 2),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["lin_prefill_mfma_kernel"],
+                     "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": byts,
+                     "hbm_gbs": round(byts / (ms * 1e-3) / 1e9, 1)},
+    }
+
+
+def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256):
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(2)
+    qkv = torch.randn(B, L, 3, H, 64, generator=g).bfloat16().to(dev)
+    ms, _ = _events_ms(torch, lambda: ops.swa_prefill(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=64), steps, warmup)
+    byts = B * L * H * 4 * 64 * 2
+    gbs = byts / (ms * 1e-3) / 1e9
+    cache = torch.zeros(B, L + decode_steps, 2, H, 64, dtype=torch.bfloat16, device=dev)
+    cache[:, :L] = qkv[:, :, 1:]
+    qn = torch.randn(B, 1, 3, H, 64, generator=g).bfloat16().to(dev)
+    pos = [L]
+
+    def dstep():
+        ops.swa_step(qn[:, :, 0], qn[:, :, 1], qn[:, :, 2], cache, pos[0], w_left=64)
+        pos[0] = L + (pos[0] + 1 - L) % decode_steps
+
+    dms, _ = _events_ms(torch, dstep, decode_steps, 8)
+    return {
+        "prefill_tok_s": B * L / (ms * 1e-3), "prefill_ms": ms, "decode_tok_s": B / (dms * 1e-3), "decode_us": dms * 1e3,
+        "B": B, "L": L, "window": 64,
+        "roofline": {"kernel": "swa_prefill_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["swa_prefill_kernel"], "algorithmic_bytes_per_launch": byts},
+    }
+
+
+def cpu_baseline_decode(torch, B=128, H=16, dv=64, sample_steps=8):
+    """The oracle's recurrent step on the host: `sample_steps` of the 256 steps at full batch."""
+    from oracle import based_oracle as O
+
+    g = torch.Generator().manual_seed(0)
+    kv = torch.randn(B, H, 1, dv, D_EXP, generator=g)
+    ks = torch.randn(B, H, 1, 1, D_EXP, generator=g).abs() + 1
+    q = torch.randn(B, H, 1, 16, generator=g).bfloat16()
+    k = torch.randn(B, H, 1, 16, generator=g).bfloat16()
+    v = torch.randn(B, H, 1, dv, generator=g).bfloat16()
+    O.linear_attn_step(kv, ks, q.float(), k.float(), v.float())  # warm-up
+    t0 = time.perf_counter()
+    for _ in range(sample_steps):
+        O.linear_attn_step(kv, ks, q.float(), k.float(), v.float())
+    dt = (time.perf_counter() - t0) / sample_steps
+    return {"value": round(B / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{sample_steps} of 256 decode steps at B={B}, H={H}, dv={dv} (oracle linear_attn_step, fp32, torch CPU)",
+            "host_cpu_count": os.cpu_count(), "ms_per_step": round(dt * 1e3, 2)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", choices=["decode", "prefill", "swa"], default=None)
+    ap.add_argument("--prefill-batch", type=int, default=8)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU (every (batch, head) pair is independent; "
+              "nothing here uses a second device). Re-run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    from based_amd import ops
+
+    out = {
+        "metric": "prefill tok/s @L=4096 + decode tok/s @B=128, Based-360m mixers, 1 GPU",
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+    }
+    if args.only in (None, "decode"):
+        d = bench_decode(torch, ops, args.steps, args.warmup)
+        out.update({"value": round(d["tok_s"], 1), "ms_per_step": round(d["ms"], 5),
+                    "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
+                    "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5)})
+    if args.only in (None, "prefill"):
+        pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({1, args.prefill_batch, 64})]
+        out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
+    if args.only in (None, "swa"):
+        s = bench_swa(torch, ops, 20, 3)
+        out["swa"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in s.items()}
+    if args.only == "prefill":
+        p = out["prefill"][-1]
+        out.update({"value": round(p["tok_s"], 1), "ms_per_step": p["ms"], "dtype": "bf16",
+                    "config": {"workload": f"linear-attn prefill B={p['B']} L={p['L']} dv={p['dv']}"}, "roofline": p["roofline"]})
+    if args.only == "swa":
+        out.update({"value": round(out["swa"]["prefill_tok_s"], 1), "ms_per_step": out["swa"]["prefill_ms"], "dtype": "bf16",
+                    "config": {"workload": "configs[2]: sliding-window prefill B=8 H=16 L=4096 w=64"},
+                    "roofline": out["swa"]["roofline"]})
+    if not args.no_cpu and args.only in (None, "decode"):
+        out["cpu_baseline"] = cpu_baseline_decode(torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,120 @@
+"""Host-side logic that needs no GPU: module construction and parameter names, cache
+shapes, config routing, sampling, and loud failure when tensors are not on a HIP device."""
+import pytest
+import torch
+
+import based_amd
+from based_amd import ops
+from based_amd.generation import InferenceParams, sample
+from based_amd.mixers import BaseConv, LinearAttention, SlidingAttention, TaylorExp
+from based_amd.stack import GPTLMHeadModel, based_360m_config
+from oracle import based_oracle as O
+
+
+def test_linear_attention_parameters_and_cache():
+    m = LinearAttention(d_model=1024, feature_map=TaylorExp(input_dim=16), feature_dim=16, num_heads=16, layer_idx=3)
+    names = dict(m.named_parameters())
+    assert set(names) == {"proj_q.weight", "proj_k.weight", "proj_v.weight", "out_proj.weight"}
+    assert names["proj_q.weight"].shape == (256, 1024) and names["proj_v.weight"].shape == (1024, 1024)
+    assert m.head_dim == 64 and m.expanded_size() == 273
+    kv, ks = m.allocate_inference_cache(5, 100, dtype=torch.bfloat16)
+    assert kv.shape == (5, 16, 1, 64, 273) and ks.shape == (5, 16, 1, 1, 273)
+    assert kv.dtype == torch.float32  # state is carried in fp32
+
+
+def test_taylor_module_matches_oracle():
+    x = torch.randn(2, 3, 4, 16)
+    fm = TaylorExp(input_dim=16)
+    assert torch.allclose(fm(x), O.taylor_exp(x))
+    assert torch.allclose(fm.raw_from_mapped(fm(x)), x)
+
+
+def test_unsupported_feature_map_is_rejected():
+    from based_amd.mixers import FeatureMap
+    with pytest.raises(NotImplementedError):
+        LinearAttention(d_model=64, feature_map=FeatureMap(input_dim=16), num_heads=4)
+    with pytest.raises(NotImplementedError):
+        LinearAttention(d_model=64, feature_map=TaylorExp(input_dim=8), feature_dim=8, num_heads=4)
+
+
+def test_sliding_attention_parameters_and_cache():
+    m = SlidingAttention(embed_dim=1024, num_heads=16, qkv_proj_bias=False, out_proj_bias=False, window_size=128, layer_idx=2)
+    assert set(dict(m.named_parameters())) == {"Wqkv.weight", "out_proj.weight"}
+    assert m.Wqkv.weight.shape == (3072, 1024) and m.window == (64, 0)
+    assert m.allocate_inference_cache(3, 77).shape == (3, 77, 2, 16, 64)
+    with pytest.raises(NotImplementedError):
+        SlidingAttention(embed_dim=1024, num_heads=16, num_heads_kv=4)
+    with pytest.raises(NotImplementedError):
+        SlidingAttention(embed_dim=1024, num_heads=16, window_size=256)
+    with pytest.raises(NotImplementedError):
+        SlidingAttention(embed_dim=512, num_heads=16)
+
+
+def test_cpu_tensors_fail_loudly():
+    q = torch.zeros(1, 1, 1, 16)
+    with pytest.raises(ValueError):
+        ops.linear_attn_step(q, q, torch.zeros(1, 1, 1, 64), torch.zeros(1, 1, 1, 64, 273), torch.zeros(1, 1, 1, 1, 273))
+    with pytest.raises(ValueError):
+        ops.linear_attn_prefill(q, q, torch.zeros(1, 1, 1, 64))
+    x = torch.zeros(1, 4, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.swa_prefill(x, x, x)
+
+
+def test_stack_routing_and_state_dict_names():
+    cfg = based_360m_config(n_layer=8, vocab_size=1000)
+    model = GPTLMHeadModel(cfg)
+    kinds = [type(l.mixer).__name__ for l in model.transformer.layers]
+    assert kinds == ["BaseConv", "LinearAttention", "SlidingAttention", "BaseConv", "BaseConv", "BaseConv",
+                     "LinearAttention", "SlidingAttention"]
+    sd = model.state_dict()
+    for key in ("transformer.layers.1.mixer.proj_q.weight", "transformer.layers.2.mixer.Wqkv.weight",
+                "transformer.layers.0.mixer.in_proj.weight", "transformer.layers.0.mixer.conv.conv.weight",
+                "transformer.layers.0.mlp.fc1.weight", "transformer.layers.0.norm1.weight",
+                "transformer.embeddings.word_embeddings.weight", "transformer.ln_f.weight", "lm_head.weight"):
+        assert key in sd, key
+    assert sd["transformer.layers.0.mlp.fc1.weight"].shape == (4096, 1024)
+    assert sd["transformer.layers.0.mlp.fc2.weight"].shape == (1024, 2048)
+    assert sd["transformer.layers.0.mixer.conv.conv.weight"].shape == (2048, 1, 3)
+    assert model.lm_head.weight is model.transformer.embeddings.word_embeddings.weight
+    assert sd["lm_head.weight"].shape[0] % 8 == 0
+
+
+def test_full_360m_parameter_count():
+    model = GPTLMHeadModel(based_360m_config(), device="meta")
+    n = sum(p.numel() for p in model.parameters())
+    assert 355e6 < n < 370e6
+
+
+def test_base_conv_step_equals_parallel_cpu():
+    torch.manual_seed(0)
+    m = BaseConv(d_model=32, l_max=64, layer_idx=0, expand_proj=4)
+    x = torch.randn(2, 10, 32)
+    y_par = m(x)
+    ip = InferenceParams(max_seqlen=10, max_batch_size=2)
+    y0 = m(x[:, :6], inference_params=ip)
+    assert torch.allclose(y0, y_par[:, :6], atol=1e-5)
+    ip.seqlen_offset = 6
+    for t in range(6, 10):
+        y = m(x[:, t:t + 1], inference_params=ip)
+        assert torch.allclose(y, y_par[:, t:t + 1], atol=1e-5)
+        ip.seqlen_offset += 1
+
+
+def test_sampling():
+    logits = torch.tensor([[0.1, 3.0, -1.0, 2.0], [5.0, 0.0, 0.0, 0.0]])
+    assert sample(logits, top_k=1).tolist() == [1, 0]
+    torch.manual_seed(0)
+    for _ in range(20):
+        t = sample(logits.clone(), top_k=2)
+        assert t[0].item() in (1, 3) and t[1].item() in (0, 1, 2, 3)
+    t = sample(logits.clone(), top_k=0, top_p=0.5)
+    assert t[1].item() == 0
+
+
+def test_inference_params_reset():
+    ip = InferenceParams(max_seqlen=8, max_batch_size=2, lengths_per_sample=torch.ones(2, dtype=torch.int32))
+    ip.seqlen_offset = 5
+    ip.reset(16, 4)
+    assert (ip.max_seqlen, ip.max_batch_size, ip.seqlen_offset) == (16, 4, 0)
+    assert ip.lengths_per_sample.sum() == 0
