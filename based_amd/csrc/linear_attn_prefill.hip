@@ -63,13 +63,25 @@ __device__ __forceinline__ bf16x8 pack8(const float (&x)[8]) {
 }
 
 __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
+#ifdef BASED_EXP_NO_MFMA
+  asm volatile("" ::"v"(a), "v"(b));
+  return c;
+#else
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+#endif
 }
 
 constexpr int kChunk = 64;       // tokens per chunk
 constexpr int kFTiles = 10;      // 160 symmetric feature slots = 10 tiles of 16
 constexpr int kETiles = 5;       // 64 value channels + 1 normaliser channel (tile 4, column 0)
 constexpr int kVtStride = 72;    // bf16 per V^T row in LDS: 64 token slots + pad
+
+// V^T lives in LDS as 64 rows (channels) of eight 16-byte blocks (8 token slots each); the
+// block index is XOR-swizzled with bits 3..5 of the row so that the transposing 16-bit writes
+// of one wavefront spread over the banks while operand reads stay aligned 128-bit loads.
+__device__ __forceinline__ int vt_offset(int row, int pos) {
+  return row * kVtStride + ((((pos >> 3) ^ (row >> 3)) & 7) << 3) + (pos & 7);
+}
 constexpr float kSqrt2 = 1.4142135623730951f;
 
 // Position of chunk-relative token tau inside a V^T row / inside the contraction slots:
@@ -116,46 +128,59 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
   const bf16x8 ones_op = __builtin_bit_cast(bf16x8, u32x4{one2, one2, one2, one2});
   const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
 
+  // Global loads of a chunk, issued one phase ahead of their use (the wavefront is alone on its
+  // SIMD, so nothing else hides HBM latency).  q, k: 64 rows x 32 B, lane <-> row.  v: 64 rows x
+  // 128 B, pass i: lane <-> (token 8 i + lane/8, channels 8 (lane%8) ..+8).
+  u32x4 pf_q[2], pf_k[2];
+  bf16x8 pf_v[8];
+  auto issue_loads = [&](int t0) {
+    const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
+    const u32x4 z4 = {0, 0, 0, 0};
+    pf_q[0] = pf_q[1] = pf_k[0] = pf_k[1] = z4;
+    if (lane < ntok) {
+      const u32x4* qs = reinterpret_cast<const u32x4*>(q + (long)(t0 + lane) * q_sl);
+      const u32x4* ks = reinterpret_cast<const u32x4*>(k + (long)(t0 + lane) * k_sl);
+      pf_q[0] = qs[0]; pf_q[1] = qs[1]; pf_k[0] = ks[0]; pf_k[1] = ks[1];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int tau = 8 * i + (lane >> 3);
+      bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (lane & 7));
+      pf_v[i] = x;
+    }
+  };
+  if (L > 0) issue_loads(0);
+
   for (int t0 = 0; t0 < L; t0 += kChunk) {
     const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
 
     // ---------------- stage the chunk: q, k row-major, v transposed, into LDS ----------------
     {
-      // q, k: 64 rows x 32 B; lane <-> row
-      u32x4 qa = {0, 0, 0, 0}, qb = {0, 0, 0, 0}, ka = {0, 0, 0, 0}, kb = {0, 0, 0, 0};
-      if (lane < ntok) {
-        const u32x4* qs = reinterpret_cast<const u32x4*>(q + (long)(t0 + lane) * q_sl);
-        const u32x4* ks = reinterpret_cast<const u32x4*>(k + (long)(t0 + lane) * k_sl);
-        qa = qs[0]; qb = qs[1]; ka = ks[0]; kb = ks[1];
-      }
       u32x4* dq = reinterpret_cast<u32x4*>(s_q + lane * kFeat);
       u32x4* dk = reinterpret_cast<u32x4*>(s_k + lane * kFeat);
-      dq[0] = qa; dq[1] = qb; dk[0] = ka; dk[1] = kb;
-      // v: 64 rows x 128 B; pass i: lane <-> (token 8 i + lane/8, channels 8 (lane%8) ..+8)
-      bf16x8 vv[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int tau = 8 * i + (lane >> 3);
-        bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (lane & 7));
-        vv[i] = x;
-      }
+      dq[0] = pf_q[0]; dq[1] = pf_q[1]; dk[0] = pf_k[0]; dk[1] = pf_k[1];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int pos = token_slot(8 * i + (lane >> 3));
 #pragma unroll
-        for (int c = 0; c < 8; ++c) s_vt[(8 * (lane & 7) + c) * kVtStride + pos] = vv[i][c];
+        for (int c = 0; c < 8; ++c) {
+#ifdef BASED_EXP_NO_LDSW
+          if (c > 0) continue;
+#endif
+          s_vt[vt_offset(8 * (lane & 7) + c, pos)] = pf_v[i][c];
+        }
       }
     }
     __syncthreads();
 
-    // V^T operand tiles: lane <-> channel 16 et + col, slots <-> tokens of slab s
-    bf16x8 vt[4][2];
-#pragma unroll
-    for (int et = 0; et < 4; ++et)
-#pragma unroll
-      for (int s = 0; s < 2; ++s)
-        vt[et][s] = *reinterpret_cast<const bf16x8*>(s_vt + (16 * et + col) * kVtStride + 32 * s + 8 * grp);
+    // V^T operand tiles: lane <-> channel 16 et + col, slots <-> tokens of slab s.  Loaded as a
+    // batch at the start of each phase that uses them (one LDS round trip per phase: the
+    // wavefront is alone on its SIMD, so every separate wait is exposed latency) and dropped
+    // during the register-hungry read-out phase in between.
+    auto load_vt = [&](int et, int s) -> bf16x8 {
+      return *reinterpret_cast<const bf16x8*>(s_vt + vt_offset(16 * et + col, 32 * s + 8 * grp));
+    };
 
     // output accumulators O^T[channel tile][token tile]: lane <-> token 16 nt + col, regs <-> channel
     f32x4 O[kETiles][4];
@@ -166,12 +191,16 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
 
     // ---------------- within the chunk: A^T = tril(1 + s + s^2/2)^T, O^T += V^T A^T ----------------
     {
-      bf16x8 kq_a[4], kq_b[4];  // K tiles (A operand, rows = keys), Q tiles (B operand, cols = queries)
+      // K tiles (A operand, rows = keys) and Q tiles (B operand, cols = queries); lane groups
+      // 2, 3 hold the zero padding of the K=32 contraction slots.
       const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+      bf16x8 kq_a[4], kq_b[4], vt[4][2];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         kq_a[i] = low_half ? *reinterpret_cast<const bf16x8*>(s_k + (16 * i + col) * kFeat + 8 * grp) : zero8;
         kq_b[i] = low_half ? *reinterpret_cast<const bf16x8*>(s_q + (16 * i + col) * kFeat + 8 * grp) : zero8;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) vt[i][s] = load_vt(i, s);
       }
       static_for<4>([&](auto NT) {
         constexpr int nt = decltype(NT)::value;
@@ -262,25 +291,33 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
         for (int et = 0; et < 4; ++et) {
           const uint32_t w0 = pack_bf16(O[et][nt][0] * inv, O[et][nt][1] * inv);
           const uint32_t w1 = pack_bf16(O[et][nt][2] * inv, O[et][nt][3] * inv);
+#ifdef BASED_EXP_NO_STORE
+          if (w0 != 0x12345678u) continue;
+#endif
           *reinterpret_cast<uint2*>(y + (long)(t0 + tau) * y_sl + 16 * et + 4 * grp) = make_uint2(w0, w1);
         }
       }
     }
 
+    // next chunk's loads fly during the state update (the phase with the fewest live registers)
+    if (t0 + kChunk < L) issue_loads(t0 + kChunk);
+
     // ---------------- state update: S += psi(k)^T V over the chunk's tokens ----------------
     {
       // lane <-> slot position j = col; registers <-> the 8 token slots of each slab
-      float kraw[2][8], k16[2][8], cst[2][8];
+      float kraw[2][8], k16[2][8];
+      bf16x8 vt[4][2];
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+      for (int s = 0; s < 2; ++s) {
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj) {
-          const int tau = slot_token(s, grp, jj);
-          const float x = to_f32(s_k[tau * kFeat + col]);
+          const float x = to_f32(s_k[slot_token(s, grp, jj) * kFeat + col]);
           kraw[s][jj] = x;
           k16[s][jj] = x * (1.0f / 16.0f);
-          cst[s][jj] = (col == 8 && tau < ntok) ? 1.0f : 0.0f;  // constant feature, real tokens only
         }
+#pragma unroll
+        for (int et = 0; et < 4; ++et) vt[et][s] = load_vt(et, s);
+      }
       static_for<kFTiles>([&](auto FT) {
         constexpr int t = decltype(FT)::value;
 #pragma unroll
@@ -294,7 +331,9 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
               f[jj] = row_ror<t>(kraw[s][jj]) * k16[s][jj];
             } else if constexpr (t == 8) {
               const float prod = row_ror<8>(kraw[s][jj]) * k16[s][jj];
-              f[jj] = col < 8 ? prod : cst[s][jj];
+              // position 8 is the constant feature (real tokens only), 9..15 are unused
+              const float cst = (col == 8 && slot_token(s, grp, jj) < ntok) ? 1.0f : 0.0f;
+              f[jj] = col < 8 ? prod : cst;
             } else {
               f[jj] = kraw[s][jj] * 0.25f;
             }
