@@ -28,9 +28,6 @@ FLAGS = [
     "-Wno-unused-command-line-argument",
     # packed-fp32 VALU forms are disabled for all device code built here
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # let MFMA results live in ordinary VGPRs as well as AccVGPRs: the prefill kernel keeps more
-    # than 256 accumulator registers, which the AccVGPR-only form cannot hold without scratch
-    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-I", INCLUDE,
     "-I", CSRC,
 ]

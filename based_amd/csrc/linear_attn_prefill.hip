@@ -63,48 +63,46 @@ __device__ __forceinline__ bf16x8 pack8(const float (&x)[8]) {
 }
 
 __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
-#ifdef BASED_EXP_NO_MFMA
-  asm volatile("" ::"v"(a), "v"(b));
-  return c;
-#else
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-#endif
 }
 
 constexpr int kChunk = 64;       // tokens per chunk
 constexpr int kFTiles = 10;      // 160 symmetric feature slots = 10 tiles of 16
 constexpr int kETiles = 5;       // 64 value channels + 1 normaliser channel (tile 4, column 0)
-constexpr int kVtStride = 72;    // bf16 per V^T row in LDS: 64 token slots + pad
-
-// V^T lives in LDS as 64 rows (channels) of eight 16-byte blocks (8 token slots each); the
-// block index is XOR-swizzled with bits 3..5 of the row so that the transposing 16-bit writes
-// of one wavefront spread over the banks while operand reads stay aligned 128-bit loads.
-__device__ __forceinline__ int vt_offset(int row, int pos) {
-  return row * kVtStride + ((((pos >> 3) ^ (row >> 3)) & 7) << 3) + (pos & 7);
-}
+constexpr int kVStride = 80;     // bf16 per V row in LDS (64 channels + pad): 160 B rows make the
+                                 // transposing reads below conflict-free
 constexpr float kSqrt2 = 1.4142135623730951f;
 
 // Position of chunk-relative token tau inside a V^T row / inside the contraction slots:
 // slab s = tau/32 holds, for lane group g, slots jj = 0..7 <-> tokens 32s + 16(jj/4) + 4g + jj%4,
 // which is the order in which accumulator rows (4g + r of tiles 2s, 2s+1) turn into operand slots.
-__device__ __forceinline__ int token_slot(int tau) {
-  const int s = tau >> 5, rem = tau & 31;
-  return 32 * s + 8 * ((rem & 15) >> 2) + 4 * (rem >> 4) + (rem & 3);
-}
 __device__ __forceinline__ int slot_token(int s, int g, int jj) {
   return 32 * s + 16 * (jj >> 2) + 4 * g + (jj & 3);
 }
 
-__global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
+constexpr int kWavesPerChain = 2;   // wavefronts cooperating on one (batch, head, channel block)
+constexpr int kOwnFT = kFTiles / kWavesPerChain;  // slot tiles of the state owned by a wavefront
+// Slot tiles owned by wavefront w: {0,1,2,3,8} and {4,5,6,7,9}.  Slabs (pairs of tiles 2s, 2s+1)
+// 0..3 then belong to one wavefront each, which publishes them with whole 16-byte writes; only
+// slab 4 is shared half and half.
+__host__ __device__ constexpr int own_tile(int wave, int i) { return i < 4 ? 4 * wave + i : 8 + wave; }
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+constexpr int kSbBytes = 5 * kETiles * 64 * 16;   // bf16 image of the state: [slab][channel tile][lane] x 16 B
+
+// The whole per-chain loop as seen by wavefront `wave` (a compile-time role: the two roles run
+// different instruction streams, chosen by one scalar branch at kernel entry, and meet only at
+// the workgroup barriers).
+template <int wave>
+__device__ __forceinline__ void lin_prefill_chain(
+    __bf16* s_q, __bf16* s_k, __bf16* s_v, unsigned char* s_sb,
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
     long v_sl, long y_sb, long y_sh, long y_sl, float eps) {
-  __shared__ __align__(16) __bf16 s_q[kChunk * kFeat];
-  __shared__ __align__(16) __bf16 s_k[kChunk * kFeat];
-  __shared__ __align__(16) __bf16 s_vt[64 * kVtStride];
-
-  const int lane = threadIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
   const long bh = blockIdx.x;
@@ -116,94 +114,111 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
   v += b * v_sb + h * v_sh + 64 * eb;
   y += b * y_sb + h * y_sh + 64 * eb;
 
-  // running state S[slot tile][channel tile]: lane <-> channel 16 et + col, regs <-> slots 4 grp + r
-  f32x4 S[kFTiles][kETiles];
+  // Division of labour between the two wavefronts of a chain:
+  //   read-out  (O^T = V^T A^T + S^T psi(q)^T)  split by TOKENS : wave 0 owns token tiles {0, 3},
+  //             wave 1 owns {1, 2} (equal causal work), each against the whole state;
+  //   update    (S += psi(k)^T V)               split by SLOTS  : wave w owns slot tiles 5w..5w+4.
+  // Each wavefront therefore generates every psi element exactly once, holds only its half of
+  // the fp32 state in accumulators, and publishes a bf16 image of that half in LDS once per
+  // chunk for the other's read-out.
+
+  // own half of the running state S[slot tile 5 wave + i][channel tile]:
+  // lane <-> channel 16 et + col, regs <-> slot positions 4 grp + r
+  f32x4 S[kOwnFT][kETiles];
 #pragma unroll
-  for (int ft = 0; ft < kFTiles; ++ft)
+  for (int i = 0; i < kOwnFT; ++i)
 #pragma unroll
-    for (int et = 0; et < kETiles; ++et) S[ft][et] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int et = 0; et < kETiles; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // operand of the normaliser channel: row/column 64 (col == 0) is all ones
   const uint32_t one2 = col == 0 ? 0x3F803F80u : 0u;
   const bf16x8 ones_op = __builtin_bit_cast(bf16x8, u32x4{one2, one2, one2, one2});
   const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
 
-  // Global loads of a chunk, issued one phase ahead of their use (the wavefront is alone on its
-  // SIMD, so nothing else hides HBM latency).  q, k: 64 rows x 32 B, lane <-> row.  v: 64 rows x
-  // 128 B, pass i: lane <-> (token 8 i + lane/8, channels 8 (lane%8) ..+8).
-  u32x4 pf_q[2], pf_k[2];
-  bf16x8 pf_v[8];
+  // Global loads of a chunk, issued one phase ahead of their use.  q (wave 0) / k (wave 1):
+  // 64 rows x 32 B, lane <-> row.  v: 64 rows x 128 B = 512 pieces of 16 B, four per thread:
+  // piece 128 i + tid <-> (token piece / 8, channels 8 (piece % 8) ..+8).
+  u32x4 pf_qk[2];
+  bf16x8 pf_v[4];
   auto issue_loads = [&](int t0) {
     const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
     const u32x4 z4 = {0, 0, 0, 0};
-    pf_q[0] = pf_q[1] = pf_k[0] = pf_k[1] = z4;
+    pf_qk[0] = pf_qk[1] = z4;
     if (lane < ntok) {
-      const u32x4* qs = reinterpret_cast<const u32x4*>(q + (long)(t0 + lane) * q_sl);
-      const u32x4* ks = reinterpret_cast<const u32x4*>(k + (long)(t0 + lane) * k_sl);
-      pf_q[0] = qs[0]; pf_q[1] = qs[1]; pf_k[0] = ks[0]; pf_k[1] = ks[1];
+      const __bf16* base = wave == 0 ? q + (long)(t0 + lane) * q_sl : k + (long)(t0 + lane) * k_sl;
+      const u32x4* src = reinterpret_cast<const u32x4*>(base);
+      pf_qk[0] = src[0];
+      pf_qk[1] = src[1];
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int tau = 8 * i + (lane >> 3);
+    for (int i = 0; i < 4; ++i) {
+      const int piece = 128 * i + tid;
+      const int tau = piece >> 3;
       bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (lane & 7));
+      if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (piece & 7));
       pf_v[i] = x;
     }
   };
   if (L > 0) issue_loads(0);
 
+  // V^T operand tile (lane <-> channel 16 et + col, slots jj <-> tokens 32 s + 16 (jj/4) + 4 grp + jj%4)
+  // straight from the row-major V chunk in LDS with the transposing 64-bit LDS read: inside
+  // each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
+  // loaded, so source lane 4j + a fetches channels 4a..4a+3 of token j of the group's four.
+  const __bf16* vt_base = s_v + (4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
+  auto load_vt = [&](int et, int s) -> bf16x8 {
+    const __bf16* p0 = vt_base + (32 * s) * kVStride + 16 * et;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kVStride));
+    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(bf16x8, both);
+  };
+
   for (int t0 = 0; t0 < L; t0 += kChunk) {
     const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
 
-    // ---------------- stage the chunk: q, k row-major, v transposed, into LDS ----------------
+    // ---------------- stage the chunk (q, k, v rows as they come) into LDS ----------------
     {
-      u32x4* dq = reinterpret_cast<u32x4*>(s_q + lane * kFeat);
-      u32x4* dk = reinterpret_cast<u32x4*>(s_k + lane * kFeat);
-      dq[0] = pf_q[0]; dq[1] = pf_q[1]; dk[0] = pf_k[0]; dk[1] = pf_k[1];
+      u32x4* dst = reinterpret_cast<u32x4*>((wave == 0 ? s_q : s_k) + lane * kFeat);
+      dst[0] = pf_qk[0];
+      dst[1] = pf_qk[1];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int pos = token_slot(8 * i + (lane >> 3));
-#pragma unroll
-        for (int c = 0; c < 8; ++c) {
-#ifdef BASED_EXP_NO_LDSW
-          if (c > 0) continue;
-#endif
-          s_vt[vt_offset(8 * (lane & 7) + c, pos)] = pf_v[i][c];
-        }
+      for (int i = 0; i < 4; ++i) {
+        const int piece = 128 * i + tid;
+        *reinterpret_cast<bf16x8*>(s_v + (piece >> 3) * kVStride + 8 * (piece & 7)) = pf_v[i];
       }
+    }
+    // ---------------- publish the bf16 image of the own half of the state ----------------
+    // s_sb[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes 0..7 come
+    // from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
+#pragma unroll
+    for (int et = 0; et < kETiles; ++et) {
+#pragma unroll
+      for (int sl = 0; sl < 2; ++sl) {  // the two whole slabs of this wavefront: tiles (2 sl, 2 sl + 1) of its four
+        const float x[8] = {S[2 * sl][et][0], S[2 * sl][et][1], S[2 * sl][et][2], S[2 * sl][et][3],
+                            S[2 * sl + 1][et][0], S[2 * sl + 1][et][1], S[2 * sl + 1][et][2], S[2 * sl + 1][et][3]};
+        *reinterpret_cast<bf16x8*>(s_sb + (((2 * wave + sl) * kETiles + et) * 64 + lane) * 16) = pack8(x);
+      }
+      // slab 4: tile 8 (wave 0) is its low half, tile 9 (wave 1) its high half
+      const uint2 w2 = make_uint2(pack_bf16(S[4][et][0], S[4][et][1]), pack_bf16(S[4][et][2], S[4][et][3]));
+      *reinterpret_cast<uint2*>(s_sb + ((4 * kETiles + et) * 64 + lane) * 16 + wave * 8) = w2;
     }
     __syncthreads();
 
-    // V^T operand tiles: lane <-> channel 16 et + col, slots <-> tokens of slab s.  Loaded as a
-    // batch at the start of each phase that uses them (one LDS round trip per phase: the
-    // wavefront is alone on its SIMD, so every separate wait is exposed latency) and dropped
-    // during the register-hungry read-out phase in between.
-    auto load_vt = [&](int et, int s) -> bf16x8 {
-      return *reinterpret_cast<const bf16x8*>(s_vt + vt_offset(16 * et + col, 32 * s + 8 * grp));
-    };
+    // ---------------- read-out of one own token tile: intra-chunk part, state part, store ----------------
+    auto readout = [&](auto NT) {
+      constexpr int nt = decltype(NT)::value;  // token tile within the chunk
+      // O^T[channel tile]: lane <-> token 16 nt + col, regs <-> channel 4 grp + r
+      f32x4 O[kETiles];
+#pragma unroll
+      for (int et = 0; et < kETiles; ++et) O[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // output accumulators O^T[channel tile][token tile]: lane <-> token 16 nt + col, regs <-> channel
-    f32x4 O[kETiles][4];
-#pragma unroll
-    for (int et = 0; et < kETiles; ++et)
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) O[et][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // ---------------- within the chunk: A^T = tril(1 + s + s^2/2)^T, O^T += V^T A^T ----------------
-    {
-      // K tiles (A operand, rows = keys) and Q tiles (B operand, cols = queries); lane groups
-      // 2, 3 hold the zero padding of the K=32 contraction slots.
-      const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-      bf16x8 kq_a[4], kq_b[4], vt[4][2];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        kq_a[i] = low_half ? *reinterpret_cast<const bf16x8*>(s_k + (16 * i + col) * kFeat + 8 * grp) : zero8;
-        kq_b[i] = low_half ? *reinterpret_cast<const bf16x8*>(s_q + (16 * i + col) * kFeat + 8 * grp) : zero8;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) vt[i][s] = load_vt(i, s);
-      }
-      static_for<4>([&](auto NT) {
-        constexpr int nt = decltype(NT)::value;
+      // within the chunk: A^T = tril(1 + s + s^2/2)^T from a K=16 product of raw q, k; O^T += V^T A^T.
+      // Lane groups 2, 3 hold the zero padding of the K=32 contraction slots.
+      {
+        const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+        const bf16x8 bq = low_half ? *reinterpret_cast<const bf16x8*>(s_q + (16 * nt + col) * kFeat + 8 * grp) : zero8;
         float p[4][4];  // [key tile][r]; tiles above the diagonal stay zero
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
@@ -211,7 +226,8 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
           for (int r = 0; r < 4; ++r) p[mt][r] = 0.f;
         static_for<nt + 1>([&](auto MT) {
           constexpr int mt = decltype(MT)::value;
-          const f32x4 a = mfma(kq_a[mt], kq_b[nt], f32x4{0.f, 0.f, 0.f, 0.f});
+          const bf16x8 ka = low_half ? *reinterpret_cast<const bf16x8*>(s_k + (16 * mt + col) * kFeat + 8 * grp) : zero8;
+          const f32x4 a = mfma(ka, bq, f32x4{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float pv = __builtin_fmaf(a[r], __builtin_fmaf(a[r], 1.0f / 32.0f, 0.25f), 1.0f);
@@ -225,49 +241,36 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
                                p[2 * s + 1][0], p[2 * s + 1][1], p[2 * s + 1][2], p[2 * s + 1][3]};
           const bf16x8 bp = pack8(pb);
 #pragma unroll
-          for (int et = 0; et < 4; ++et) O[et][nt] = mfma(vt[et][s], bp, O[et][nt]);
-          O[4][nt] = mfma(ones_op, bp, O[4][nt]);
+          for (int et = 0; et < 4; ++et) O[et] = mfma(load_vt(et, s), bp, O[et]);
+          O[4] = mfma(ones_op, bp, O[4]);
         });
-      });
-    }
+      }
 
-    // ---------------- across chunks: O^T += S^T psi(q)^T (state before this chunk) ----------------
-    {
-      // q of token 16 nt + col, rotated by 4 grp: qr[nt][r] = q[(4 grp + r) mod 16]
-      float qr[4][16];
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
+      // across chunks: O^T += S^T psi(q)^T with the state as it was before this chunk
+      {
+        // q of token 16 nt + col, rotated by 4 grp: qr[r] = q[(4 grp + r) mod 16]
+        float qr[16];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const bf16x4 x = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + ((4 * grp + 4 * i) & 15));
 #pragma unroll
-          for (int c = 0; c < 4; ++c) qr[nt][4 * i + c] = to_f32(x[c]);
+          for (int c = 0; c < 4; ++c) qr[4 * i + c] = to_f32(x[c]);
         }
-      const float fix8_0 = (grp == 2) ? 1.0f : 0.0f;  // slot (tile 8, position 8) = constant feature
-
-      static_for<5>([&](auto SG) {
-        constexpr int sg = decltype(SG)::value;  // slab of 32 slots = slot tiles 2 sg, 2 sg + 1
-        bf16x8 sa[kETiles];
-#pragma unroll
-        for (int et = 0; et < kETiles; ++et) {
-          const float x[8] = {S[2 * sg][et][0], S[2 * sg][et][1], S[2 * sg][et][2], S[2 * sg][et][3],
-                              S[2 * sg + 1][et][0], S[2 * sg + 1][et][1], S[2 * sg + 1][et][2], S[2 * sg + 1][et][3]};
-          sa[et] = pack8(x);
-        }
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt) {
+        const float fix8_0 = (grp == 2) ? 1.0f : 0.0f;  // slot (tile 8, position 8) = constant feature
+        static_for<5>([&](auto SG) {
+          constexpr int sg = decltype(SG)::value;  // slab of 32 slots = slot tiles 2 sg, 2 sg + 1
           float f[8];
           static_for<8>([&](auto JJ) {
             constexpr int jj = decltype(JJ)::value;
             constexpr int t = 2 * sg + jj / 4;  // slot tile
             constexpr int c = jj % 4;           // position 4 grp + c
-            const float own = qr[nt][c];
+            const float own = qr[c];
             if constexpr (t == 0) {
               f[jj] = own * own;
             } else if constexpr (t <= 7) {
-              f[jj] = own * qr[nt][(c - t) & 15];
+              f[jj] = own * qr[(c - t) & 15];
             } else if constexpr (t == 8) {
-              const float prod = own * qr[nt][(c - 8) & 15];
+              const float prod = own * qr[(c - 8) & 15];
               f[jj] = low_half ? prod : (c == 0 ? fix8_0 : 0.0f);
             } else {
               f[jj] = own;
@@ -275,75 +278,76 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
           });
           const bf16x8 bq = pack8(f);
 #pragma unroll
-          for (int et = 0; et < kETiles; ++et) O[et][nt] = mfma(sa[et], bq, O[et][nt]);
-        }
-      });
-    }
+          for (int et = 0; et < kETiles; ++et) {
+            const bf16x8 sa = *reinterpret_cast<const bf16x8*>(s_sb + ((sg * kETiles + et) * 64 + lane) * 16);
+            O[et] = mfma(sa, bq, O[et]);
+          }
+        });
+      }
 
-    // ---------------- normalise and store the chunk's outputs ----------------
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const float z = __shfl(O[4][nt][0], col, 64);  // denominator sits in lane group 0, register 0
+      // normalise and store: the denominator sits in lane group 0, register 0 of channel tile 4
+      const float z = __shfl(O[4][0], col, 64);
       const float inv = 1.0f / (z + eps);
       const int tau = 16 * nt + col;
       if (tau < ntok) {
 #pragma unroll
         for (int et = 0; et < 4; ++et) {
-          const uint32_t w0 = pack_bf16(O[et][nt][0] * inv, O[et][nt][1] * inv);
-          const uint32_t w1 = pack_bf16(O[et][nt][2] * inv, O[et][nt][3] * inv);
-#ifdef BASED_EXP_NO_STORE
-          if (w0 != 0x12345678u) continue;
-#endif
+          const uint32_t w0 = pack_bf16(O[et][0] * inv, O[et][1] * inv);
+          const uint32_t w1 = pack_bf16(O[et][2] * inv, O[et][3] * inv);
           *reinterpret_cast<uint2*>(y + (long)(t0 + tau) * y_sl + 16 * et + 4 * grp) = make_uint2(w0, w1);
         }
       }
-    }
+    };
+    readout(std::integral_constant<int, wave == 0 ? 0 : 1>{});
+    __builtin_amdgcn_sched_barrier(0);
+    readout(std::integral_constant<int, wave == 0 ? 3 : 2>{});
+    __builtin_amdgcn_sched_barrier(0);
 
-    // next chunk's loads fly during the state update (the phase with the fewest live registers)
+    // next chunk's loads fly during the state update
     if (t0 + kChunk < L) issue_loads(t0 + kChunk);
 
-    // ---------------- state update: S += psi(k)^T V over the chunk's tokens ----------------
+    // ---------------- state update: S += psi(k)^T V for the own slot tiles ----------------
     {
-      // lane <-> slot position j = col; registers <-> the 8 token slots of each slab
-      float kraw[2][8], k16[2][8];
-      bf16x8 vt[4][2];
+      // lane <-> slot position j = col; registers <-> the 8 token slots of a slab.  One slab of
+      // 32 tokens at a time, so that only its k values and V^T tiles are live.
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
+        float kraw[8], k16[8];
+        bf16x8 vt[4];
 #pragma unroll
         for (int jj = 0; jj < 8; ++jj) {
           const float x = to_f32(s_k[slot_token(s, grp, jj) * kFeat + col]);
-          kraw[s][jj] = x;
-          k16[s][jj] = x * (1.0f / 16.0f);
+          kraw[jj] = x;
+          k16[jj] = x * (1.0f / 16.0f);
         }
 #pragma unroll
-        for (int et = 0; et < 4; ++et) vt[et][s] = load_vt(et, s);
-      }
-      static_for<kFTiles>([&](auto FT) {
-        constexpr int t = decltype(FT)::value;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
+        for (int et = 0; et < 4; ++et) vt[et] = load_vt(et, s);
+        static_for<kOwnFT>([&](auto II) {
+          constexpr int i = decltype(II)::value;
+          constexpr int t = own_tile(wave, i);  // slot tile
           float f[8];
 #pragma unroll
           for (int jj = 0; jj < 8; ++jj) {
             if constexpr (t == 0) {
-              f[jj] = kraw[s][jj] * k16[s][jj] * 0.5f;
+              f[jj] = kraw[jj] * k16[jj] * 0.5f;
             } else if constexpr (t <= 7) {
-              f[jj] = row_ror<t>(kraw[s][jj]) * k16[s][jj];
+              f[jj] = row_ror<t>(kraw[jj]) * k16[jj];
             } else if constexpr (t == 8) {
-              const float prod = row_ror<8>(kraw[s][jj]) * k16[s][jj];
+              const float prod = row_ror<8>(kraw[jj]) * k16[jj];
               // position 8 is the constant feature (real tokens only), 9..15 are unused
               const float cst = (col == 8 && slot_token(s, grp, jj) < ntok) ? 1.0f : 0.0f;
               f[jj] = col < 8 ? prod : cst;
             } else {
-              f[jj] = kraw[s][jj] * 0.25f;
+              f[jj] = kraw[jj] * 0.25f;
             }
           }
           const bf16x8 ak = pack8(f);
 #pragma unroll
-          for (int et = 0; et < 4; ++et) S[t][et] = mfma(ak, vt[et][s], S[t][et]);
-          S[t][4] = mfma(ak, ones_op, S[t][4]);
-        }
-      });
+          for (int et = 0; et < 4; ++et) S[i][et] = mfma(ak, vt[et], S[i][et]);
+          S[i][4] = mfma(ak, ones_op, S[i][4]);
+        });
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     __syncthreads();  // LDS is overwritten by the next chunk
   }
@@ -351,44 +355,65 @@ __global__ __launch_bounds__(64, 1) void lin_prefill_mfma_kernel(
   // ---------------- expand the 160-slot state into the (dv, 273) decode layout ----------------
   if (kv_state != nullptr) {
     float* ks_row = k_state + bh * kExp;
-    static_for<kFTiles>([&](auto FT) {
-      constexpr int t = decltype(FT)::value;
+    auto expand = [&]() {
+      static_for<kOwnFT>([&](auto II) {
+        constexpr int i = decltype(II)::value;
+        constexpr int t = own_tile(wave, i);
 #pragma unroll
-      for (int et = 0; et < kETiles; ++et) {
-        float* row;
-        bool live;
-        if (et < 4) {
-          row = kv_state + (bh * dv + 64 * eb + 16 * et + col) * kExp;
-          live = true;
-        } else {
-          row = ks_row;
-          live = (col == 0) && (eb == 0);
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int j = 4 * grp + r;
-          const float x = S[t][et][r];
-          if (!live) continue;
-          if constexpr (t == 0) {
-            row[1 + kFeat + 17 * j] = x * (4.0f * kSqrt2);
-          } else if constexpr (t <= 7) {
-            const int pj = (j - t) & 15;
-            row[1 + kFeat + 16 * j + pj] = x * (2.0f * kSqrt2);
-            row[1 + kFeat + 16 * pj + j] = x * (2.0f * kSqrt2);
-          } else if constexpr (t == 8) {
-            if (j < 8) {
-              row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
-              row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
-            } else if (j == 8) {
-              row[0] = x;
-            }
+        for (int et = 0; et < kETiles; ++et) {
+          float* row;
+          bool live;
+          if (et < 4) {
+            row = kv_state + (bh * dv + 64 * eb + 16 * et + col) * kExp;
+            live = true;
           } else {
-            row[1 + j] = x * 2.0f;
+            row = ks_row;
+            live = (col == 0) && (eb == 0);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = 4 * grp + r;
+            const float x = S[i][et][r];
+            if (!live) continue;
+            if constexpr (t == 0) {
+              row[1 + kFeat + 17 * j] = x * (4.0f * kSqrt2);
+            } else if constexpr (t <= 7) {
+              const int pj = (j - t) & 15;
+              row[1 + kFeat + 16 * j + pj] = x * (2.0f * kSqrt2);
+              row[1 + kFeat + 16 * pj + j] = x * (2.0f * kSqrt2);
+            } else if constexpr (t == 8) {
+              if (j < 8) {
+                row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
+                row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
+              } else if (j == 8) {
+                row[0] = x;
+              }
+            } else {
+              row[1 + j] = x * 2.0f;
+            }
           }
         }
-      }
-    });
+      });
+    };
+    expand();
   }
+}
+
+__global__ __launch_bounds__(64 * kWavesPerChain, 2) void lin_prefill_mfma_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
+    __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
+    int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
+    long v_sl, long y_sb, long y_sh, long y_sl, float eps) {
+  __shared__ __align__(16) __bf16 s_q[kChunk * kFeat];
+  __shared__ __align__(16) __bf16 s_k[kChunk * kFeat];
+  __shared__ __align__(16) __bf16 s_v[kChunk * kVStride];
+  __shared__ __align__(16) unsigned char s_sb[kSbBytes];
+  if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0)
+    lin_prefill_chain<0>(s_q, s_k, s_v, s_sb, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb,
+                         k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
+  else
+    lin_prefill_chain<1>(s_q, s_k, s_v, s_sb, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb,
+                         k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -529,7 +554,7 @@ extern "C" BASED_API int based_linear_attn_prefill(
                     "linear_attn_prefill: bf16 strides must be multiples of 8 elements (16 bytes)");
     BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
                   "linear_attn_prefill: tensors must be 16-byte aligned");
-    dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(64);
+    dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(64 * kWavesPerChain);
     hipLaunchKernelGGL(lin_prefill_mfma_kernel, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
                        q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
