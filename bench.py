@@ -34,10 +34,11 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 D_EXP = 273
 
-# HBM traffic per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); None until a counter run for that kernel has been committed.
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what
+# the same counter reads for a plain copy of known size (the summaries and the commands that
+# produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": None,
+    "lin_step_kernel": 293097062,   # B=128, H=16, dv=64: fetch 146,863,104 + write 146,233,958
     "lin_prefill_mfma_kernel": None,
     "swa_prefill_kernel": None,
 }
@@ -178,7 +179,9 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["decode", "prefill", "swa"], default=None)
+    ap.add_argument("--only", choices=["decode", "prefill", "swa", "copy"], default=None,
+                    help="one workload only; 'copy' is a plain 256 MiB device copy used to calibrate the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     ap.add_argument("--prefill-batch", type=int, default=8)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -192,6 +195,15 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     from based_amd import ops
+
+    if args.only == "copy":
+        n = 256 * 1024 * 1024
+        src = torch.empty(n, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        ms, _ = _events_ms(torch, lambda: dst.copy_(src), args.steps, args.warmup)
+        print(json.dumps({"workload": "plain device copy", "bytes_read": n, "bytes_written": n, "ms": round(ms, 5),
+                          "GBps": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
+        return
 
     out = {
         "metric": "prefill tok/s @L=4096 + decode tok/s @B=128, Based-360m mixers, 1 GPU",
