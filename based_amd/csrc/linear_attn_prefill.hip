@@ -67,10 +67,11 @@ __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 }
 
 constexpr int kChunk = 64;       // tokens per chunk
-constexpr int kFTiles = 10;      // 160 symmetric feature slots = 10 tiles of 16
+constexpr int kFTiles = 10;      // 160 symmetric feature slots = 10 tiles of 16 (see own_tile)
 constexpr int kETiles = 5;       // 64 value channels + 1 normaliser channel (tile 4, column 0)
 constexpr int kVStride = 80;     // bf16 per V row in LDS (64 channels + pad): 160 B rows make the
                                  // transposing reads below conflict-free
+constexpr int kOStride = 72;     // bf16 per row of the output staging tile (64 channels + pad, 144 B)
 constexpr float kSqrt2 = 1.4142135623730951f;
 
 // Position of chunk-relative token tau inside a V^T row / inside the contraction slots:
@@ -80,23 +81,24 @@ __device__ __forceinline__ int slot_token(int s, int g, int jj) {
   return 32 * s + 16 * (jj >> 2) + 4 * g + (jj & 3);
 }
 
-constexpr int kWavesPerChain = 2;   // wavefronts cooperating on one (batch, head, channel block)
-constexpr int kOwnFT = kFTiles / kWavesPerChain;  // slot tiles of the state owned by a wavefront
-// Slot tiles owned by wavefront w: {0,1,2,3,8} and {4,5,6,7,9}.  Slabs (pairs of tiles 2s, 2s+1)
-// 0..3 then belong to one wavefront each, which publishes them with whole 16-byte writes; only
-// slab 4 is shared half and half.
-__host__ __device__ constexpr int own_tile(int wave, int i) { return i < 4 ? 4 * wave + i : 8 + wave; }
+constexpr int kWavesPerChain = 4;   // wavefronts cooperating on one (batch, head, channel block)
+// Slot tiles of the state owned by wavefront w: {0,1,2}, {3,4,5}, {6,7}, {8,9}.  The wavefronts
+// with fewer slot tiles own the token tiles with more causal work (see the kernel), which
+// balances the MFMA count per wavefront to 58..62 per chunk.
+__host__ __device__ constexpr int own_count(int wave) { return wave < 2 ? 3 : 2; }
+__host__ __device__ constexpr int own_tile(int wave, int i) { return (wave < 2 ? 3 * wave : 2 * wave + 2) + i; }
+static_assert(own_tile(3, own_count(3) - 1) == kFTiles - 1, "slot tiles must be covered exactly");
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 constexpr int kSbBytes = 5 * kETiles * 64 * 16;   // bf16 image of the state: [slab][channel tile][lane] x 16 B
 
-// The whole per-chain loop as seen by wavefront `wave` (a compile-time role: the two roles run
-// different instruction streams, chosen by one scalar branch at kernel entry, and meet only at
+// The whole per-chain loop as seen by wavefront `wave` (a compile-time role: the four roles run
+// different instruction streams, chosen by a scalar branch at kernel entry, and meet only at
 // the workgroup barriers).
 template <int wave>
 __device__ __forceinline__ void lin_prefill_chain(
-    __bf16* s_q, __bf16* s_k, __bf16* s_v, unsigned char* s_sb,
+    __bf16* s_q, __bf16* s_k, __bf16* s_v, unsigned char* s_sb, __bf16* s_o,
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
@@ -105,7 +107,14 @@ __device__ __forceinline__ void lin_prefill_chain(
   const int lane = tid & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
-  const long bh = blockIdx.x;
+  // Workgroups are dealt to the 8 XCDs round-robin by workgroup id.  Chains whose q/k rows share
+  // cache lines (neighbouring heads of one batch entry: 32-byte rows, 512 bytes apart) should
+  // sit behind the same L2, so consecutive chain numbers are laid along one XCD:
+  // chain = (id mod 8) * ceil(n / 8) + id / 8 when that stays in range.
+  const long n_chain = gridDim.x;
+  const long per_xcd = (n_chain + 7) / 8;
+  long bh = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (n_chain % 8 != 0) bh = blockIdx.x;  // irregular grids keep the identity mapping
   const int eb = blockIdx.y;  // 64-channel block of the value dimension
   const int b = (int)(bh / H), h = (int)(bh % H);
 
@@ -114,19 +123,20 @@ __device__ __forceinline__ void lin_prefill_chain(
   v += b * v_sb + h * v_sh + 64 * eb;
   y += b * y_sb + h * y_sh + 64 * eb;
 
-  // Division of labour between the two wavefronts of a chain:
-  //   read-out  (O^T = V^T A^T + S^T psi(q)^T)  split by TOKENS : wave 0 owns token tiles {0, 3},
-  //             wave 1 owns {1, 2} (equal causal work), each against the whole state;
-  //   update    (S += psi(k)^T V)               split by SLOTS  : wave w owns slot tiles 5w..5w+4.
-  // Each wavefront therefore generates every psi element exactly once, holds only its half of
-  // the fp32 state in accumulators, and publishes a bf16 image of that half in LDS once per
-  // chunk for the other's read-out.
+  // Division of labour between the four wavefronts of a chain:
+  //   read-out  (O^T = V^T A^T + S^T psi(q)^T)  split by TOKENS : wave w owns token tile w of the
+  //             chunk and contracts it against the whole state;
+  //   update    (S += psi(k)^T V)               split by SLOTS  : wave w owns slot tiles own_tile(w, .).
+  // Each wavefront therefore generates every psi element exactly once, holds only its share of
+  // the fp32 state in accumulators, and publishes a bf16 image of that share in LDS once per
+  // chunk for the others' read-out.
+  constexpr int kOwn = own_count(wave);
 
-  // own half of the running state S[slot tile 5 wave + i][channel tile]:
+  // own share of the running state S[i <-> slot tile own_tile(wave, i)][channel tile]:
   // lane <-> channel 16 et + col, regs <-> slot positions 4 grp + r
-  f32x4 S[kOwnFT][kETiles];
+  f32x4 S[kOwn][kETiles];
 #pragma unroll
-  for (int i = 0; i < kOwnFT; ++i)
+  for (int i = 0; i < kOwn; ++i)
 #pragma unroll
     for (int et = 0; et < kETiles; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -136,23 +146,25 @@ __device__ __forceinline__ void lin_prefill_chain(
   const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
 
   // Global loads of a chunk, issued one phase ahead of their use.  q (wave 0) / k (wave 1):
-  // 64 rows x 32 B, lane <-> row.  v: 64 rows x 128 B = 512 pieces of 16 B, four per thread:
-  // piece 128 i + tid <-> (token piece / 8, channels 8 (piece % 8) ..+8).
+  // 64 rows x 32 B, lane <-> row.  v: 64 rows x 128 B = 512 pieces of 16 B, two per thread:
+  // piece 256 i + tid <-> (token piece / 8, channels 8 (piece % 8) ..+8).
   u32x4 pf_qk[2];
-  bf16x8 pf_v[4];
+  bf16x8 pf_v[2];
   auto issue_loads = [&](int t0) {
     const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
-    const u32x4 z4 = {0, 0, 0, 0};
-    pf_qk[0] = pf_qk[1] = z4;
-    if (lane < ntok) {
-      const __bf16* base = wave == 0 ? q + (long)(t0 + lane) * q_sl : k + (long)(t0 + lane) * k_sl;
-      const u32x4* src = reinterpret_cast<const u32x4*>(base);
-      pf_qk[0] = src[0];
-      pf_qk[1] = src[1];
+    if constexpr (wave < 2) {
+      const u32x4 z4 = {0, 0, 0, 0};
+      pf_qk[0] = pf_qk[1] = z4;
+      if (lane < ntok) {
+        const __bf16* base = wave == 0 ? q + (long)(t0 + lane) * q_sl : k + (long)(t0 + lane) * k_sl;
+        const u32x4* src = reinterpret_cast<const u32x4*>(base);
+        pf_qk[0] = src[0];
+        pf_qk[1] = src[1];
+      }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int piece = 128 * i + tid;
+    for (int i = 0; i < 2; ++i) {
+      const int piece = 256 * i + tid;
       const int tau = piece >> 3;
       bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
       if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (piece & 7));
@@ -180,31 +192,34 @@ __device__ __forceinline__ void lin_prefill_chain(
 
     // ---------------- stage the chunk (q, k, v rows as they come) into LDS ----------------
     {
-      u32x4* dst = reinterpret_cast<u32x4*>((wave == 0 ? s_q : s_k) + lane * kFeat);
-      dst[0] = pf_qk[0];
-      dst[1] = pf_qk[1];
+      if constexpr (wave < 2) {
+        u32x4* dst = reinterpret_cast<u32x4*>((wave == 0 ? s_q : s_k) + lane * kFeat);
+        dst[0] = pf_qk[0];
+        dst[1] = pf_qk[1];
+      }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int piece = 128 * i + tid;
+      for (int i = 0; i < 2; ++i) {
+        const int piece = 256 * i + tid;
         *reinterpret_cast<bf16x8*>(s_v + (piece >> 3) * kVStride + 8 * (piece & 7)) = pf_v[i];
       }
     }
-    // ---------------- publish the bf16 image of the own half of the state ----------------
+    // ---------------- publish the bf16 image of the own share of the state ----------------
     // s_sb[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes 0..7 come
     // from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
 #pragma unroll
-    for (int et = 0; et < kETiles; ++et) {
+    for (int i = 0; i < kOwn; ++i) {
+      constexpr int kBase = own_tile(wave, 0);
+      const int t = kBase + i;
 #pragma unroll
-      for (int sl = 0; sl < 2; ++sl) {  // the two whole slabs of this wavefront: tiles (2 sl, 2 sl + 1) of its four
-        const float x[8] = {S[2 * sl][et][0], S[2 * sl][et][1], S[2 * sl][et][2], S[2 * sl][et][3],
-                            S[2 * sl + 1][et][0], S[2 * sl + 1][et][1], S[2 * sl + 1][et][2], S[2 * sl + 1][et][3]};
-        *reinterpret_cast<bf16x8*>(s_sb + (((2 * wave + sl) * kETiles + et) * 64 + lane) * 16) = pack8(x);
+      for (int et = 0; et < kETiles; ++et) {
+        const uint2 w2 = make_uint2(pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]));
+        *reinterpret_cast<uint2*>(s_sb + (((t >> 1) * kETiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
       }
-      // slab 4: tile 8 (wave 0) is its low half, tile 9 (wave 1) its high half
-      const uint2 w2 = make_uint2(pack_bf16(S[4][et][0], S[4][et][1]), pack_bf16(S[4][et][2], S[4][et][3]));
-      *reinterpret_cast<uint2*>(s_sb + ((4 * kETiles + et) * 64 + lane) * 16 + wave * 8) = w2;
     }
     __syncthreads();
+
+    // next chunk's global loads are in flight for the whole of this chunk's compute
+    if (t0 + kChunk < L) issue_loads(t0 + kChunk);
 
     // ---------------- read-out of one own token tile: intra-chunk part, state part, store ----------------
     auto readout = [&](auto NT) {
@@ -285,26 +300,29 @@ __device__ __forceinline__ void lin_prefill_chain(
         });
       }
 
-      // normalise and store: the denominator sits in lane group 0, register 0 of channel tile 4
+      // normalise: the denominator sits in lane group 0, register 0 of channel tile 4
       const float z = __shfl(O[4][0], col, 64);
       const float inv = 1.0f / (z + eps);
-      const int tau = 16 * nt + col;
-      if (tau < ntok) {
+      // store: the 16 x 64 output tile goes through a wave-private LDS tile so that each lane
+      // writes 16 contiguous bytes and 8 lanes cover one 128-byte row (8-byte scattered stores
+      // cost four times the L2 write requests)
+      __bf16* so = s_o + wave * (16 * kOStride);
 #pragma unroll
-        for (int et = 0; et < 4; ++et) {
-          const uint32_t w0 = pack_bf16(O[et][0] * inv, O[et][1] * inv);
-          const uint32_t w1 = pack_bf16(O[et][2] * inv, O[et][3] * inv);
-          *reinterpret_cast<uint2*>(y + (long)(t0 + tau) * y_sl + 16 * et + 4 * grp) = make_uint2(w0, w1);
-        }
+      for (int et = 0; et < 4; ++et) {
+        const uint32_t w0 = pack_bf16(O[et][0] * inv, O[et][1] * inv);
+        const uint32_t w1 = pack_bf16(O[et][2] * inv, O[et][3] * inv);
+        *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
+      }
+#pragma unroll
+      for (int hlf = 0; hlf < 2; ++hlf) {
+        const int row = 8 * hlf + (lane >> 3);
+        const u32x4 w4 = *reinterpret_cast<const u32x4*>(so + row * kOStride + 8 * (lane & 7));
+        const int tau = 16 * nt + row;
+        if (tau < ntok) *reinterpret_cast<u32x4*>(y + (long)(t0 + tau) * y_sl + 8 * (lane & 7)) = w4;
       }
     };
-    readout(std::integral_constant<int, wave == 0 ? 0 : 1>{});
+    readout(std::integral_constant<int, wave>{});
     __builtin_amdgcn_sched_barrier(0);
-    readout(std::integral_constant<int, wave == 0 ? 3 : 2>{});
-    __builtin_amdgcn_sched_barrier(0);
-
-    // next chunk's loads fly during the state update
-    if (t0 + kChunk < L) issue_loads(t0 + kChunk);
 
     // ---------------- state update: S += psi(k)^T V for the own slot tiles ----------------
     {
@@ -322,7 +340,7 @@ __device__ __forceinline__ void lin_prefill_chain(
         }
 #pragma unroll
         for (int et = 0; et < 4; ++et) vt[et] = load_vt(et, s);
-        static_for<kOwnFT>([&](auto II) {
+        static_for<kOwn>([&](auto II) {
           constexpr int i = decltype(II)::value;
           constexpr int t = own_tile(wave, i);  // slot tile
           float f[8];
@@ -356,7 +374,7 @@ __device__ __forceinline__ void lin_prefill_chain(
   if (kv_state != nullptr) {
     float* ks_row = k_state + bh * kExp;
     auto expand = [&]() {
-      static_for<kOwnFT>([&](auto II) {
+      static_for<kOwn>([&](auto II) {
         constexpr int i = decltype(II)::value;
         constexpr int t = own_tile(wave, i);
 #pragma unroll
@@ -399,7 +417,7 @@ __device__ __forceinline__ void lin_prefill_chain(
   }
 }
 
-__global__ __launch_bounds__(64 * kWavesPerChain, 2) void lin_prefill_mfma_kernel(
+__global__ __launch_bounds__(64 * kWavesPerChain, 3) void lin_prefill_mfma_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
@@ -408,12 +426,16 @@ __global__ __launch_bounds__(64 * kWavesPerChain, 2) void lin_prefill_mfma_kerne
   __shared__ __align__(16) __bf16 s_k[kChunk * kFeat];
   __shared__ __align__(16) __bf16 s_v[kChunk * kVStride];
   __shared__ __align__(16) unsigned char s_sb[kSbBytes];
-  if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0)
-    lin_prefill_chain<0>(s_q, s_k, s_v, s_sb, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb,
-                         k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
-  else
-    lin_prefill_chain<1>(s_q, s_k, s_v, s_sb, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb,
-                         k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
+  __shared__ __align__(16) __bf16 s_o[kWavesPerChain * 16 * kOStride];
+#define BASED_CHAIN_ARGS s_q, s_k, s_v, s_sb, s_o, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh, \
+                         k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps
+  switch (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) {
+    case 0: lin_prefill_chain<0>(BASED_CHAIN_ARGS); break;
+    case 1: lin_prefill_chain<1>(BASED_CHAIN_ARGS); break;
+    case 2: lin_prefill_chain<2>(BASED_CHAIN_ARGS); break;
+    default: lin_prefill_chain<3>(BASED_CHAIN_ARGS); break;
+  }
+#undef BASED_CHAIN_ARGS
 }
 
 // ------------------------------------------------------------------------------------------

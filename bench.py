@@ -217,7 +217,7 @@ def main():
                     "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
                     "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5)})
     if args.only in (None, "prefill"):
-        pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({1, args.prefill_batch, 64})]
+        pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({1, args.prefill_batch, 48, 96})]
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
     if args.only in (None, "swa"):
         s = bench_swa(torch, ops, 20, 3)
