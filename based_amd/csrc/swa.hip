@@ -3,15 +3,15 @@
 // Prefill.  One workgroup of four wavefronts covers 64 consecutive queries of one
 // (batch, head); wavefront w owns queries [q0+16w, q0+16w+16) and the 80 keys
 // [n0-64, n0+16) they can see (window <= 64 to the left plus the causal diagonal).
-//   S^T = K Q^T   : 5 key tiles x 2 MFMA 16x16x32 (head dim 64), operands loaded straight
-//                   from global memory (a lane's 8 consecutive bf16 of one row = 16 bytes).
+//   S^T = K Q^T   : 5 key tiles x 2 MFMA 16x16x32 (head dim 64); the workgroup's 128 K rows are
+//                   staged once in LDS (a lane's operand = 8 consecutive bf16 of one row).
 //   softmax       : S^T leaves the MFMA with lane <-> query and registers <-> keys, so the
 //                   row max / row sum are in-lane loops plus two cross-lane steps.
 //   O^T = V^T P^T : the accumulator layout of S^T is already the B-operand layout for a
 //                   product contracted over keys, so P never leaves registers.  V^T (lane
 //                   <-> channel, registers <-> keys) is the one operand that needs a
-//                   transpose; the workgroup stages its 128 keys of V through LDS,
-//                   transposed on the way in.
+//                   transpose: V rows are staged as they come and read with the transposing
+//                   LDS load.  Outputs leave through LDS as full 128-byte rows.
 // Whole-window softmax in one pass: 80 keys fit in registers, so no online rescaling.
 //
 // Decode.  One wavefront per (batch, head): lane <-> key for the scores, lane <-> channel
@@ -22,44 +22,69 @@ namespace based {
 
 constexpr int kHeadDim = 64;
 constexpr int kQTile = 64;          // queries per workgroup
-constexpr int kVtStride = 136;      // bf16 elements per V^T row in LDS (128 + pad)
+constexpr int kKeysWG = 128;        // keys staged per workgroup: [q0-64, q0+64)
+constexpr int kKStride = 72;        // bf16 per K row in LDS (144 B: 16 rows x 16 B reads hit 64 distinct banks)
+constexpr int kVStride = 80;        // bf16 per V row in LDS (160 B: conflict-free transposing reads)
+constexpr int kOStride = 72;        // bf16 per row of a wavefront's output staging tile
+
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 __global__ __launch_bounds__(256) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
-    __bf16* __restrict__ o, int L, long q_sb, long q_sl, long q_sh, long k_sb, long k_sl,
-    long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh, int w_left,
-    float scale_log2e) {
-  __shared__ __align__(16) __bf16 s_vt[kHeadDim * kVtStride];
+    __bf16* __restrict__ o, int H, int L, int n_tiles, long q_sb, long q_sl, long q_sh, long k_sb,
+    long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
+    int w_left, float scale_log2e) {
+  __shared__ __align__(16) __bf16 s_k[kKeysWG * kKStride];
+  __shared__ __align__(16) __bf16 s_v[kKeysWG * kVStride];
+  __shared__ __align__(16) __bf16 s_o[4 * 16 * kOStride];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 15;   // query (B operand / accumulator column), or row of an A tile
   const int grp = lane >> 4;   // 0..3: which 8 contraction slots / which 4 accumulator rows
-  const int q0 = blockIdx.x * kQTile;
-  const int h = blockIdx.y, b = blockIdx.z;
+
+  // Workgroups are dealt to the 8 XCDs round-robin by id.  Neighbouring query tiles of one
+  // (batch, head) read overlapping K/V rows (a 64-row halo), so consecutive tiles are laid along
+  // one XCD and the halo is an L2 hit: item = (id mod 8) * ceil(n / 8) + id / 8.
+  const long n_items = gridDim.x;
+  long item = blockIdx.x;
+  if (n_items % 8 == 0) item = (item % 8) * (n_items / 8) + item / 8;
+  const int tile = (int)(item % n_tiles);
+  const long bh = item / n_tiles;
+  const int h = (int)(bh % H), b = (int)(bh / H);
+  const int q0 = tile * kQTile;
 
   q += b * q_sb + h * q_sh;
   k += b * k_sb + h * k_sh;
   v += b * v_sb + h * v_sh;
   o += b * o_sb + h * o_sh;
 
-  // ---- stage V^T for keys [q0-64, q0+64): thread t -> key t/2, channels 32*(t%2)..+32 ----
+  // ---- stage K and V rows of keys [q0-64, q0+64) as they come: 1024 pieces of 16 B each ----
   {
-    const int kk = tid >> 1, half = tid & 1;
-    const int key = q0 - 64 + kk;
-    const bool ok = key >= 0 && key < L;
-    const bf16x8* src = reinterpret_cast<const bf16x8*>(v + (long)key * v_sl + 32 * half);
+    u32x4 kp[4], vp[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (ok) x = src[c];
+    for (int i = 0; i < 4; ++i) {
+      const int piece = 256 * i + tid;
+      const int key = q0 - 64 + (piece >> 3);
+      const u32x4 z4 = {0, 0, 0, 0};
+      kp[i] = vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
+      if (key >= 0 && key < L) {
+        kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + 8 * (piece & 7));
+        vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + 8 * (piece & 7));
+      }
+    }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) s_vt[(32 * half + 8 * c + i) * kVtStride + kk] = x[i];
+    for (int i = 0; i < 4; ++i) {
+      const int piece = 256 * i + tid;
+      *reinterpret_cast<u32x4*>(s_k + (piece >> 3) * kKStride + 8 * (piece & 7)) = kp[i];
+      *reinterpret_cast<u32x4*>(s_v + (piece >> 3) * kVStride + 8 * (piece & 7)) = vp[i];
     }
   }
 
-  // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
+  // ---- Q operand of this wavefront's 16 queries, straight from global memory ----
   const int n0 = q0 + 16 * wave;            // first query of this wavefront
   const int n = n0 + col;                   // this lane's query
   bf16x8 bq[2];
@@ -69,18 +94,18 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
     if (n < L) x = *reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp);
     bq[ds] = x;
   }
+  __syncthreads();
+
+  // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
+  // wavefront w sees staged keys 16 w .. 16 w + 79 (tile i = keys 16 w + 16 i ..)
   f32x4 st[5];
 #pragma unroll
   for (int i = 0; i < 5; ++i) {
-    const int key = n0 - 64 + 16 * i + col;  // A-tile row = key
+    const __bf16* row = s_k + (16 * wave + 16 * i + col) * kKStride + 8 * grp;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ds = 0; ds < 2; ++ds) {
-      bf16x8 a = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (key >= 0 && key < L)
-        a = *reinterpret_cast<const bf16x8*>(k + (long)key * k_sl + 32 * ds + 8 * grp);
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bq[ds], acc, 0, 0, 0);
-    }
+    for (int ds = 0; ds < 2; ++ds)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(row + 32 * ds), bq[ds], acc, 0, 0, 0);
     st[i] = acc;
   }
 
@@ -92,9 +117,9 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
     for (int r = 0; r < 4; ++r) {
       const int key = n0 - 64 + 16 * i + 4 * grp + r;
       const bool keep = key >= 0 && key <= n && key >= n - w_left;
-      const float s = keep ? st[i][r] * scale_log2e : -INFINITY;
-      st[i][r] = s;
-      mx = fmaxf(mx, s);
+      const float sc = keep ? st[i][r] * scale_log2e : -INFINITY;
+      st[i][r] = sc;
+      mx = fmaxf(mx, sc);
     }
   mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -110,16 +135,18 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
   sum += __shfl_xor(sum, 16, 64);
   sum += __shfl_xor(sum, 32, 64);
 
-  __syncthreads();  // V^T staged
-
   // ---- O^T = V^T P^T: 4 channel tiles x 3 key slabs of 32 (last slab half empty) ----
+  // V^T operand tiles come from the row-major V rows with the transposing 64-bit LDS read:
+  // in each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
+  // loaded, so source lane 4j + a fetches channels 4a..4a+3 of key j of the group's four.
+  const __bf16* vt_base = s_v + (16 * wave + 4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
   f32x4 ot[4];
 #pragma unroll
   for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int s = 0; s < 3; ++s) {
     // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent for s = 2)
-    uint32_t pb[4];
+    u32x4 pb;
     pb[0] = pack_bf16(st[2 * s][0], st[2 * s][1]);
     pb[1] = pack_bf16(st[2 * s][2], st[2 * s][3]);
     if (s < 2) {
@@ -129,29 +156,33 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
       pb[2] = 0u;
       pb[3] = 0u;
     }
-    const bf16x8 bp = __builtin_bit_cast(bf16x8, *reinterpret_cast<const __attribute__((ext_vector_type(4))) uint32_t*>(pb));
-    const int kk0 = 16 * wave + 32 * s + 4 * grp;  // LDS key slot of operand slot 0
+    const bf16x8 bp = __builtin_bit_cast(bf16x8, pb);
 #pragma unroll
     for (int et = 0; et < 4; ++et) {
-      const __bf16* row = s_vt + (16 * et + col) * kVtStride;
-      bf16x4 lo = *reinterpret_cast<const bf16x4*>(row + kk0);
-      bf16x4 hi = {0, 0, 0, 0};
-      if (s < 2) hi = *reinterpret_cast<const bf16x4*>(row + kk0 + 16);
-      const bf16x8 a = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, bp, ot[et], 0, 0, 0);
+      const __bf16* p0 = vt_base + (32 * s) * kVStride + 16 * et;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
+      s16x4 hi = {0, 0, 0, 0};
+      if (s < 2)
+        hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kVStride));
+      const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
     }
   }
 
-  // ---- normalise and store: lane holds channels 16 et + 4 grp + r of query n ----
-  if (n < L) {
-    const float inv = 1.0f / sum;
+  // ---- normalise; stage the 16 x 64 tile in LDS so each lane stores 16 contiguous bytes ----
+  const float inv = 1.0f / sum;
+  __bf16* so = s_o + wave * (16 * kOStride);
 #pragma unroll
-    for (int et = 0; et < 4; ++et) {
-      uint32_t w2[2];
-      w2[0] = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
-      w2[1] = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
-      *reinterpret_cast<uint2*>(o + (long)n * o_sl + 16 * et + 4 * grp) = make_uint2(w2[0], w2[1]);
-    }
+  for (int et = 0; et < 4; ++et) {
+    const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
+    const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
+    *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
+  }
+#pragma unroll
+  for (int hlf = 0; hlf < 2; ++hlf) {
+    const int row = 8 * hlf + (lane >> 3);
+    const u32x4 w4 = *reinterpret_cast<const u32x4*>(so + row * kOStride + 8 * (lane & 7));
+    if (n0 + row < L) *reinterpret_cast<u32x4*>(o + (long)(n0 + row) * o_sl + 8 * (lane & 7)) = w4;
   }
 }
 
@@ -258,11 +289,13 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(o), BASED_ERR_ALIGN,
                 "swa_prefill: tensors must be 16-byte aligned");
   if (B == 0 || L == 0) return BASED_OK;
-  dim3 grid((unsigned)((L + kQTile - 1) / kQTile), (unsigned)H, (unsigned)B), block(256);
+  const int64_t n_tiles = (L + kQTile - 1) / kQTile;
+  BASED_REQUIRE(B * H * n_tiles < (1ll << 31), BASED_ERR_SHAPE, "swa_prefill: grid too large");
+  dim3 grid((unsigned)(B * H * n_tiles)), block(256);
   hipLaunchKernelGGL(swa_prefill_kernel, grid, block, 0, static_cast<hipStream_t>(stream),
-                     (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o, (int)L, q_sb,
-                     q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh, w_left,
-                     scale * 1.4426950408889634f);
+                     (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o, (int)H, (int)L,
+                     (int)n_tiles, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh,
+                     w_left, scale * 1.4426950408889634f);
   return check_launch("swa_prefill");
 }
 
