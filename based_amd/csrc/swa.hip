@@ -38,7 +38,8 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
     int w_left, float scale_log2e) {
   __shared__ __align__(16) __bf16 s_k[kKeysWG * kKStride];
   __shared__ __align__(16) __bf16 s_v[kKeysWG * kVStride];
-  __shared__ __align__(16) __bf16 s_o[4 * 16 * kOStride];
+  // the output staging tiles reuse the K rows once every wavefront is done with them
+  static_assert(4 * 16 * kOStride <= kKeysWG * kKStride, "output staging must fit in the K region");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -171,7 +172,8 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
 
   // ---- normalise; stage the 16 x 64 tile in LDS so each lane stores 16 contiguous bytes ----
   const float inv = 1.0f / sum;
-  __bf16* so = s_o + wave * (16 * kOStride);
+  __syncthreads();  // all S^T products have consumed the K rows
+  __bf16* so = s_k + wave * (16 * kOStride);
 #pragma unroll
   for (int et = 0; et < 4; ++et) {
     const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
