@@ -31,6 +31,14 @@ SIGNATURES = {
         C.c_int,
         [_P, _P, _P, _P, _P, _P] + [_I64] * 4 + [_I64] * 12 + [C.c_float, C.c_int, _P],
     ),
+    "based_linear_attn_prefill_plan": (
+        C.c_int,
+        [_I64] * 4 + [C.c_int, C.POINTER(_I64), C.POINTER(_I64)],
+    ),
+    "based_linear_attn_prefill_split": (
+        C.c_int,
+        [_P, _P, _P, _P, _P, _P] + [_I64] * 4 + [_I64] * 12 + [C.c_float, C.c_int, _I64, _P, _I64, _P],
+    ),
     "based_swa_prefill": (
         C.c_int,
         [_P, _P, _P, _P] + [_I64] * 3 + [_I64] * 12 + [C.c_int, C.c_float, C.c_int, _P],

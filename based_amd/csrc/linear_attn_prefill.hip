@@ -96,13 +96,24 @@ constexpr int kSbBytes = 5 * kETiles * 64 * 16;   // bf16 image of the state: [s
 // The whole per-chain loop as seen by wavefront `wave` (a compile-time role: the four roles run
 // different instruction streams, chosen by a scalar branch at kernel entry, and meet only at
 // the workgroup barriers).
-template <int wave>
+//
+// MODE selects how much of a sequence one workgroup scans (small batches split each sequence
+// into segments so that the whole GPU has work; see based_linear_attn_prefill_split):
+//   kModeFull   the whole sequence, state starting at zero;
+//   kModeDelta  tokens [t_begin, t_end) only, state update only (no outputs), state starting at
+//               zero and dumped to the workspace at the end (the segment's contribution);
+//   kModeFrom   tokens [t_begin, t_end) in full, state starting from the workspace entry (the
+//               exclusive prefix over the earlier segments).
+constexpr int kModeFull = 0, kModeDelta = 1, kModeFrom = 2;
+constexpr int kSegStateFloats = kFTiles * kETiles * 64 * 4;  // accumulator image of one chain's state
+
+template <int wave, int MODE>
 __device__ __forceinline__ void lin_prefill_chain(
     __bf16* s_q, __bf16* s_k, __bf16* s_v, unsigned char* s_sb, __bf16* s_o,
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
-    long v_sl, long y_sb, long y_sh, long y_sl, float eps) {
+    long v_sl, long y_sb, long y_sh, long y_sl, float eps, float* __restrict__ ws, int seg_tokens, int n_seg) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int col = lane & 15;
@@ -140,6 +151,22 @@ __device__ __forceinline__ void lin_prefill_chain(
 #pragma unroll
     for (int et = 0; et < kETiles; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // token range of this workgroup and its slot in the workspace
+  const int seg = blockIdx.z;
+  const int t_begin = MODE == kModeFull ? 0 : seg * seg_tokens;
+  const int t_end = MODE == kModeFull ? L : (t_begin + seg_tokens < L ? t_begin + seg_tokens : L);
+  const bool last_seg = MODE == kModeFull || seg == n_seg - 1;
+  float* ws_mine = nullptr;
+  if constexpr (MODE != kModeFull)
+    ws_mine = ws + (((long)bh * gridDim.y + eb) * n_seg + seg) * (long)kSegStateFloats;
+  if constexpr (MODE == kModeFrom) {
+#pragma unroll
+    for (int i = 0; i < kOwn; ++i)
+#pragma unroll
+      for (int et = 0; et < kETiles; ++et)
+        S[i][et] = *reinterpret_cast<const f32x4*>(ws_mine + ((own_tile(wave, i) * kETiles + et) * 64 + lane) * 4);
+  }
+
   // operand of the normaliser channel: row/column 64 (col == 0) is all ones
   const uint32_t one2 = col == 0 ? 0x3F803F80u : 0u;
   const bf16x8 ones_op = __builtin_bit_cast(bf16x8, u32x4{one2, one2, one2, one2});
@@ -151,8 +178,8 @@ __device__ __forceinline__ void lin_prefill_chain(
   u32x4 pf_qk[2];
   bf16x8 pf_v[2];
   auto issue_loads = [&](int t0) {
-    const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
-    if constexpr (wave < 2) {
+    const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
+    if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
       const u32x4 z4 = {0, 0, 0, 0};
       pf_qk[0] = pf_qk[1] = z4;
       if (lane < ntok) {
@@ -171,7 +198,7 @@ __device__ __forceinline__ void lin_prefill_chain(
       pf_v[i] = x;
     }
   };
-  if (L > 0) issue_loads(0);
+  if (t_begin < t_end) issue_loads(t_begin);
 
   // V^T operand tile (lane <-> channel 16 et + col, slots jj <-> tokens 32 s + 16 (jj/4) + 4 grp + jj%4)
   // straight from the row-major V chunk in LDS with the transposing 64-bit LDS read: inside
@@ -187,12 +214,12 @@ __device__ __forceinline__ void lin_prefill_chain(
     return __builtin_bit_cast(bf16x8, both);
   };
 
-  for (int t0 = 0; t0 < L; t0 += kChunk) {
-    const int ntok = L - t0 < kChunk ? L - t0 : kChunk;
+  for (int t0 = t_begin; t0 < t_end; t0 += kChunk) {
+    const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
 
     // ---------------- stage the chunk (q, k, v rows as they come) into LDS ----------------
     {
-      if constexpr (wave < 2) {
+      if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
         u32x4* dst = reinterpret_cast<u32x4*>((wave == 0 ? s_q : s_k) + lane * kFeat);
         dst[0] = pf_qk[0];
         dst[1] = pf_qk[1];
@@ -207,7 +234,7 @@ __device__ __forceinline__ void lin_prefill_chain(
     // s_sb[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes 0..7 come
     // from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
 #pragma unroll
-    for (int i = 0; i < kOwn; ++i) {
+    for (int i = 0; i < (MODE == kModeDelta ? 0 : kOwn); ++i) {
       constexpr int kBase = own_tile(wave, 0);
       const int t = kBase + i;
 #pragma unroll
@@ -219,7 +246,7 @@ __device__ __forceinline__ void lin_prefill_chain(
     __syncthreads();
 
     // next chunk's global loads are in flight for the whole of this chunk's compute
-    if (t0 + kChunk < L) issue_loads(t0 + kChunk);
+    if (t0 + kChunk < t_end) issue_loads(t0 + kChunk);
 
     // ---------------- read-out of one own token tile: intra-chunk part, state part, store ----------------
     auto readout = [&](auto NT) {
@@ -321,7 +348,7 @@ __device__ __forceinline__ void lin_prefill_chain(
         if (tau < ntok) *reinterpret_cast<u32x4*>(y + (long)(t0 + tau) * y_sl + 8 * (lane & 7)) = w4;
       }
     };
-    readout(std::integral_constant<int, wave>{});
+    if constexpr (MODE != kModeDelta) readout(std::integral_constant<int, wave>{});
     __builtin_amdgcn_sched_barrier(0);
 
     // ---------------- state update: S += psi(k)^T V for the own slot tiles ----------------
@@ -370,8 +397,18 @@ __device__ __forceinline__ void lin_prefill_chain(
     __syncthreads();  // LDS is overwritten by the next chunk
   }
 
+  // ---------------- a segment's contribution goes to the workspace as it sits in registers ----------------
+  if constexpr (MODE == kModeDelta) {
+#pragma unroll
+    for (int i = 0; i < kOwn; ++i)
+#pragma unroll
+      for (int et = 0; et < kETiles; ++et)
+        *reinterpret_cast<f32x4*>(ws_mine + ((own_tile(wave, i) * kETiles + et) * 64 + lane) * 4) = S[i][et];
+    return;
+  }
+
   // ---------------- expand the 160-slot state into the (dv, 273) decode layout ----------------
-  if (kv_state != nullptr) {
+  if (kv_state != nullptr && last_seg) {
     float* ks_row = k_state + bh * kExp;
     auto expand = [&]() {
       static_for<kOwn>([&](auto II) {
@@ -417,25 +454,42 @@ __device__ __forceinline__ void lin_prefill_chain(
   }
 }
 
+template <int MODE>
 __global__ __launch_bounds__(64 * kWavesPerChain, 3) void lin_prefill_mfma_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
-    long v_sl, long y_sb, long y_sh, long y_sl, float eps) {
+    long v_sl, long y_sb, long y_sh, long y_sl, float eps, float* __restrict__ ws, int seg_tokens, int n_seg) {
   __shared__ __align__(16) __bf16 s_q[kChunk * kFeat];
   __shared__ __align__(16) __bf16 s_k[kChunk * kFeat];
   __shared__ __align__(16) __bf16 s_v[kChunk * kVStride];
   __shared__ __align__(16) unsigned char s_sb[kSbBytes];
   __shared__ __align__(16) __bf16 s_o[kWavesPerChain * 16 * kOStride];
 #define BASED_CHAIN_ARGS s_q, s_k, s_v, s_sb, s_o, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh, \
-                         k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps
+                         k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, ws, seg_tokens, n_seg
   switch (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) {
-    case 0: lin_prefill_chain<0>(BASED_CHAIN_ARGS); break;
-    case 1: lin_prefill_chain<1>(BASED_CHAIN_ARGS); break;
-    case 2: lin_prefill_chain<2>(BASED_CHAIN_ARGS); break;
-    default: lin_prefill_chain<3>(BASED_CHAIN_ARGS); break;
+    case 0: lin_prefill_chain<0, MODE>(BASED_CHAIN_ARGS); break;
+    case 1: lin_prefill_chain<1, MODE>(BASED_CHAIN_ARGS); break;
+    case 2: lin_prefill_chain<2, MODE>(BASED_CHAIN_ARGS); break;
+    default: lin_prefill_chain<3, MODE>(BASED_CHAIN_ARGS); break;
   }
 #undef BASED_CHAIN_ARGS
+}
+
+// In-place exclusive prefix over the segments of each chain: ws[c][s] <- sum_{s' < s} ws[c][s'].
+// The last segment's entry is never produced by the delta pass and is treated as zero.
+__global__ __launch_bounds__(256) void lin_prefill_prefix_kernel(float* __restrict__ ws, int n_seg) {
+  float* base = ws + (long)blockIdx.x * n_seg * kSegStateFloats;
+  const int idx = blockIdx.y * blockDim.x + threadIdx.x;  // one float4 of the state image per thread
+  if (idx >= kSegStateFloats / 4) return;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < n_seg; ++s) {
+    f32x4* p = reinterpret_cast<f32x4*>(base + (long)s * kSegStateFloats) + idx;
+    f32x4 cur = {0.f, 0.f, 0.f, 0.f};
+    if (s < n_seg - 1) cur = *p;
+    *p = acc;
+    acc += cur;
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -577,9 +631,9 @@ extern "C" BASED_API int based_linear_attn_prefill(
     BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
                   "linear_attn_prefill: tensors must be 16-byte aligned");
     dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(64 * kWavesPerChain);
-    hipLaunchKernelGGL(lin_prefill_mfma_kernel, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
+    hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFull>, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
-                       q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
+                       q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, (float*)nullptr, 0, 1);
     return check_launch("linear_attn_prefill");
   }
   BASED_REQUIRE(dv >= 1 && dv <= 1024, BASED_ERR_SHAPE, "linear_attn_prefill: head dim %ld unsupported",
@@ -595,4 +649,83 @@ extern "C" BASED_API int based_linear_attn_prefill(
                        (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps);
   }
   return check_launch("linear_attn_prefill");
+}
+
+// Workgroup slots of one full wave of the MFMA prefill kernel on MI355X (256 CUs x 3 resident
+// workgroups); segment counts are chosen to fill about one such wave.
+static constexpr int64_t kPrefillSlots = 768;
+
+extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, int64_t L, int64_t dv,
+                                                        int io_dtype, int64_t* n_seg,
+                                                        int64_t* workspace_bytes) {
+  using namespace based;
+  BASED_REQUIRE(n_seg && workspace_bytes, BASED_ERR_ARG, "linear_attn_prefill_plan: null output pointer");
+  *n_seg = 1;
+  *workspace_bytes = 0;
+  if (io_dtype != BASED_BF16 || (dv != 64 && dv != 128) || B <= 0 || H <= 0 || L <= 0) return BASED_OK;
+  const int64_t chains = B * H * (dv / 64);
+  const int64_t chunks = (L + kChunk - 1) / kChunk;
+  if (chains * 3 >= kPrefillSlots * 2 || chunks < 2) return BASED_OK;  // enough chains already
+  int64_t want = (kPrefillSlots + chains - 1) / chains;
+  if (want > chunks) want = chunks;
+  const int64_t seg_chunks = (chunks + want - 1) / want;
+  const int64_t segs = (chunks + seg_chunks - 1) / seg_chunks;
+  if (segs < 2) return BASED_OK;
+  *n_seg = segs;
+  *workspace_bytes = chains * segs * (int64_t)kSegStateFloats * 4;
+  return BASED_OK;
+}
+
+extern "C" BASED_API int based_linear_attn_prefill_split(
+    const void* q, const void* k, const void* v, void* y, float* kv_state, float* k_state, int64_t B,
+    int64_t H, int64_t L, int64_t dv, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+    int64_t k_sh, int64_t k_sl, int64_t v_sb, int64_t v_sh, int64_t v_sl, int64_t y_sb, int64_t y_sh,
+    int64_t y_sl, float eps, int io_dtype, int64_t n_seg, void* workspace, int64_t workspace_bytes,
+    void* stream) {
+  using namespace based;
+  if (n_seg <= 1)
+    return based_linear_attn_prefill(q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh,
+                                     k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype, stream);
+  BASED_REQUIRE(q && k && v && y && workspace, BASED_ERR_ARG, "linear_attn_prefill_split: null pointer argument");
+  BASED_REQUIRE((kv_state == nullptr) == (k_state == nullptr), BASED_ERR_ARG,
+                "linear_attn_prefill_split: kv_state and k_state must both be given or both be NULL");
+  BASED_REQUIRE(io_dtype == BASED_BF16 && (dv == 64 || dv == 128), BASED_ERR_SHAPE,
+                "linear_attn_prefill_split: only the bf16 MFMA path (dv 64 or 128) can be split");
+  BASED_REQUIRE(B > 0 && H > 0 && L > 0 && B * H < (1ll << 31) && L < (1ll << 31), BASED_ERR_ARG,
+                "linear_attn_prefill_split: bad sizes");
+  const int64_t chunks = (L + kChunk - 1) / kChunk;
+  BASED_REQUIRE(n_seg <= chunks && n_seg < 65536, BASED_ERR_ARG,
+                "linear_attn_prefill_split: %ld segments for %ld chunks", (long)n_seg, (long)chunks);
+  const int64_t seg_chunks = (chunks + n_seg - 1) / n_seg;
+  BASED_REQUIRE((n_seg - 1) * seg_chunks < chunks, BASED_ERR_ARG,
+                "linear_attn_prefill_split: segment count %ld leaves empty segments (use the plan)", (long)n_seg);
+  const int64_t chains = B * H * (dv / 64);
+  BASED_REQUIRE(workspace_bytes >= chains * n_seg * (int64_t)kSegStateFloats * 4, BASED_ERR_ARG,
+                "linear_attn_prefill_split: workspace too small");
+  const int64_t strides[] = {q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl};
+  for (int64_t st : strides)
+    BASED_REQUIRE(st % 8 == 0, BASED_ERR_ALIGN,
+                  "linear_attn_prefill_split: bf16 strides must be multiples of 8 elements (16 bytes)");
+  BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y) && aligned16(workspace),
+                BASED_ERR_ALIGN, "linear_attn_prefill_split: tensors must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  const int seg_tokens = (int)(seg_chunks * kChunk);
+  dim3 block(64 * kWavesPerChain);
+  // pass 1: every segment but the last accumulates its own contribution to the state
+  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)(n_seg - 1)),
+                     block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
+                     k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
+                     y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
+  int rc = check_launch("linear_attn_prefill_split (delta)");
+  if (rc) return rc;
+  hipLaunchKernelGGL(lin_prefill_prefix_kernel, dim3((unsigned)chains, (kSegStateFloats / 4 + 255) / 256), dim3(256), 0, s,
+                     ws, (int)n_seg);
+  rc = check_launch("linear_attn_prefill_split (prefix)");
+  if (rc) return rc;
+  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)n_seg),
+                     block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
+                     k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
+                     y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
+  return check_launch("linear_attn_prefill_split (read-out)");
 }

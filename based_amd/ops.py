@@ -2,6 +2,7 @@
 current stream.  PyTorch is used for device memory and streams only."""
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Optional, Tuple
 
@@ -121,14 +122,17 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
     return o
 
 
-def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False
+def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False, split=None
                         ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
     """Causal Taylor linear attention.  q, k: (B, H, L, 16) raw; v: (B, H, L, dv); any strides
     with the last dim contiguous (e.g. `(B, L, H, d).transpose(1, 2)` views).
 
     Returns (y, kv_state, k_state): y (B, H, L, dv) in q's dtype, stored so that
     `y.transpose(1, 2).reshape(B, L, H*dv)` is a free view; states are fp32
-    (B, H, 1, dv, 273) / (B, H, 1, 1, 273), or None unless return_state."""
+    (B, H, 1, dv, 273) / (B, H, 1, 1, 273), or None unless return_state.
+
+    split: None = let the library decide whether to scan each sequence in concurrent segments
+    (small batches); False = never; an int > 1 = that many segments."""
     _require_cuda(q, k, v)
     B, H, L, d = q.shape
     dv = v.shape[-1]
@@ -144,12 +148,26 @@ def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False
     if return_state:
         kv_state = torch.empty(B, H, 1, dv, EXPANDED_DIM, dtype=torch.float32, device=q.device)
         k_state = torch.empty(B, H, 1, 1, EXPANDED_DIM, dtype=torch.float32, device=q.device)
-    with torch.cuda.device(q.device):
-        _lib.check(_lib.lib().based_linear_attn_prefill(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
+    lib = _lib.lib()
+    n_seg, ws_bytes = ctypes.c_int64(1), ctypes.c_int64(0)
+    if split is not False:
+        _lib.check(lib.based_linear_attn_prefill_plan(B, H, L, dv, _dtype_code(q), ctypes.byref(n_seg),
+                                                      ctypes.byref(ws_bytes)))
+    if isinstance(split, int) and not isinstance(split, bool) and split > 1:
+        n_seg = ctypes.c_int64(split)  # explicit segment count (tests)
+        ws_bytes = ctypes.c_int64(B * H * (dv // 64) * split * 10 * 5 * 64 * 4 * 4)
+    args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
             kv_state.data_ptr() if return_state else None, k_state.data_ptr() if return_state else None,
             B, H, L, dv,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), y.stride(0), y.stride(1), y.stride(2),
-            float(eps), _dtype_code(q), _stream_ptr(q)))
+            float(eps), _dtype_code(q))
+    with torch.cuda.device(q.device):
+        if n_seg.value > 1:
+            # scratch for the per-segment states; torch's caching allocator makes this cheap
+            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q.device)
+            _lib.check(lib.based_linear_attn_prefill_split(*args, n_seg.value, ws.data_ptr(), ws_bytes.value,
+                                                           _stream_ptr(q)))
+        else:
+            _lib.check(lib.based_linear_attn_prefill(*args, _stream_ptr(q)))
     return y, kv_state, k_state

@@ -96,6 +96,32 @@ BASED_API int based_linear_attn_prefill(const void* q, const void* k, const void
                               float eps, int io_dtype, void* stream);
 
 /*
+ * Same computation as based_linear_attn_prefill for SMALL batches: each sequence is cut into
+ * n_seg segments of whole 64-token chunks that are scanned concurrently (every segment first
+ * accumulates its own contribution to the state, an exclusive prefix over segments follows,
+ * then every segment is read out from its prefix), so that B*H chains of a short batch can
+ * still fill the GPU.  Same reference lines as based_linear_attn_prefill; results agree with
+ * it to accumulation order.
+ *
+ * based_linear_attn_prefill_plan reports the segment count this library would use for a shape
+ * (1 = do not split) and the bytes of device workspace that count needs; the caller allocates
+ * the workspace (16-byte aligned; contents need no initialisation and are scratch afterwards)
+ * and passes both to based_linear_attn_prefill_split.  n_seg <= 1 forwards to the unsplit
+ * entry point.  bf16, dv in {64, 128} only.
+ */
+BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, int64_t L, int64_t dv, int io_dtype,
+                                             int64_t* n_seg, int64_t* workspace_bytes);
+BASED_API int based_linear_attn_prefill_split(const void* q, const void* k, const void* v, void* y,
+                              float* kv_state, float* k_state,
+                              int64_t B, int64_t H, int64_t L, int64_t dv,
+                              int64_t q_sb, int64_t q_sh, int64_t q_sl,
+                              int64_t k_sb, int64_t k_sh, int64_t k_sl,
+                              int64_t v_sb, int64_t v_sh, int64_t v_sl,
+                              int64_t y_sb, int64_t y_sh, int64_t y_sl,
+                              float eps, int io_dtype,
+                              int64_t n_seg, void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Sliding-window causal softmax attention over a whole sequence.
  * Replaces the flash-attn call behind FlashSelfAttention / FlashCrossAttention with
  * causal=True, window_size=(w_left, 0): based/models/mixers/slide_attention.py:100-106,

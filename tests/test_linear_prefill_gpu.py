@@ -121,3 +121,41 @@ def test_mfma_vs_fp32_kernel_long(dev):
     assert rel_l2(y1.float(), y2) < 1e-2
     assert rel_l2(kv1, kv2) < 5e-3
     assert rel_l2(ks1, ks2) < 5e-3
+
+
+@pytest.mark.parametrize("B,H,L,dv,split", [(1, 2, 1000, 64, 4), (1, 1, 128, 64, 2), (2, 2, 700, 128, 3),
+                                            (1, 3, 4096, 64, 64), (1, 16, 4096, 64, None)])
+def test_segmented_scan_matches_single_pass(dev, B, H, L, dv, split):
+    """Sequences scanned as concurrent segments (small-batch path) against the single-pass kernel
+    and the oracle, outputs and decode states; split=None lets the library plan the segments."""
+    from based_amd import ops
+
+    print(f"prefill split case B={B} H={H} L={L} dv={dv} split={split}", flush=True)
+    q, k, v = _qkv(B, H, L, dv, torch.bfloat16, seed=21)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y1, kv1, ks1 = ops.linear_attn_prefill(qd, kd, vd, return_state=True, split=False)
+    y2, kv2, ks2 = ops.linear_attn_prefill(qd, kd, vd, return_state=True, split=split)
+    torch.cuda.synchronize()
+    assert rel_l2(y2.float(), y1.float()) < 5e-3
+    assert rel_l2(kv2, kv1) < 2e-3 and rel_l2(ks2, ks1) < 2e-3
+    n = min(L, 1024)
+    y_ref = O.linear_attn_cumsum(q[:, :, :n].float(), k[:, :, :n].float(), v[:, :, :n].float())
+    assert rel_l2(y2[:, :, :n].float(), y_ref) < 1e-2
+    y3, _, _ = ops.linear_attn_prefill(qd, kd, vd, return_state=False, split=split)
+    assert torch.equal(y3, y2)  # deterministic, with or without the state outputs
+
+
+def test_split_plan(dev):
+    import ctypes
+    from based_amd import _lib
+
+    lib = _lib.lib()
+    n, w = ctypes.c_int64(), ctypes.c_int64()
+    assert lib.based_linear_attn_prefill_plan(64, 16, 4096, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 1 and w.value == 0                     # plenty of chains: single pass
+    assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert 2 <= n.value <= 64 and w.value == 16 * n.value * 12800 * 4
+    assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 64, 1, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 1                                      # fp32 path is never split
+    assert lib.based_linear_attn_prefill_plan(1, 16, 64, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 1                                      # a single chunk cannot be split
