@@ -483,12 +483,19 @@ __global__ __launch_bounds__(256) void lin_prefill_prefix_kernel(float* __restri
   const int idx = blockIdx.y * blockDim.x + threadIdx.x;  // one float4 of the state image per thread
   if (idx >= kSegStateFloats / 4) return;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < n_seg; ++s) {
-    f32x4* p = reinterpret_cast<f32x4*>(base + (long)s * kSegStateFloats) + idx;
-    f32x4 cur = {0.f, 0.f, 0.f, 0.f};
-    if (s < n_seg - 1) cur = *p;
-    *p = acc;
-    acc += cur;
+  // eight segments at a time: the loads are independent, only the running sum is sequential
+  for (int s0 = 0; s0 < n_seg; s0 += 8) {
+    f32x4 cur[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      cur[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (s0 + u < n_seg - 1) cur[u] = reinterpret_cast<const f32x4*>(base + (long)(s0 + u) * kSegStateFloats)[idx];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (s0 + u < n_seg) reinterpret_cast<f32x4*>(base + (long)(s0 + u) * kSegStateFloats)[idx] = acc;
+      acc += cur[u];
+    }
   }
 }
 

@@ -14,8 +14,8 @@
 //                   LDS load.  Outputs leave through LDS as full 128-byte rows.
 // Whole-window softmax in one pass: 80 keys fit in registers, so no online rescaling.
 //
-// Decode.  One wavefront per (batch, head): lane <-> key for the scores, lane <-> channel
-// for the output, against the last w_left+1 rows of a linear cache.
+// Decode.  One workgroup of four wavefronts per (batch, head) against the last w_left+1 rows of
+// a linear cache, with every load issued up front (one memory round trip per step).
 #include "common.hpp"
 
 namespace based {
@@ -188,82 +188,96 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
   }
 }
 
-// One wavefront per (b, h).  Keys lo..pos, lo = max(0, pos - w_left); at most 65.
-__global__ __launch_bounds__(64) void swa_step_kernel(
+// One workgroup of four wavefronts per (b, h).  Keys lo..pos, lo = max(0, pos - w_left): at most
+// 64 cached rows plus the new token.  Every global load of the step (K rows for the scores,
+// V rows for the output) is issued before anything is waited on, so the step costs one memory
+// round trip: thread t scores key t/4 over channels 16 (t%4)..+16, and accumulates channel t%64
+// over the keys congruent to t/64 mod 4.
+__global__ __launch_bounds__(256) void swa_step_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k_new, const __bf16* __restrict__ v_new,
     __bf16* __restrict__ kcache, __bf16* __restrict__ vcache, __bf16* __restrict__ o,
     const int32_t* __restrict__ cache_seqlens, int pos_host, int H, int max_seqlen, long q_sb,
     long q_sh, long kn_sb, long kn_sh, long vn_sb, long vn_sh, long o_sb, long o_sh, long c_sb,
     long c_st, long c_sh, int w_left, float scale_log2e) {
-  __shared__ float s_q[kHeadDim];
-  const int lane = threadIdx.x;
+  __shared__ float s_p[80];          // scores, then weights; entry 64 is the new token
+  __shared__ float s_part[4][kHeadDim];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bh = blockIdx.x;
   const int b = bh / H, h = bh % H;
   int pos = cache_seqlens ? cache_seqlens[b] : pos_host;
   pos = __builtin_amdgcn_readfirstlane(pos);
   if (pos < 0 || pos >= max_seqlen) return;  // out-of-range position: nothing to attend or write
 
-  const __bf16 kn = k_new[b * kn_sb + h * kn_sh + lane];
-  const __bf16 vn = v_new[b * vn_sb + h * vn_sh + lane];
   __bf16* kc = kcache + b * c_sb + h * c_sh;
   __bf16* vc = vcache + b * c_sb + h * c_sh;
-  kc[(long)pos * c_st + lane] = kn;
-  vc[(long)pos * c_st + lane] = vn;
-  s_q[lane] = to_f32(q[b * q_sb + h * q_sh + lane]);
+  const int lo = pos - w_left > 0 ? pos - w_left : 0;
+  const int ncached = pos - lo;  // 0..64 rows of the cache, then the new token itself
+
+  // ---- issue every load of the step ----
+  const int kj = tid >> 2, kq4 = tid & 3;  // key and channel quarter for the scores
+  bf16x8 kx[2] = {{0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0}};
+  if (kj < ncached) {
+    const bf16x8* row = reinterpret_cast<const bf16x8*>(kc + (long)(lo + kj) * c_st + 16 * kq4);
+    kx[0] = row[0];
+    kx[1] = row[1];
+  }
+  const bf16x8* qrow = reinterpret_cast<const bf16x8*>(q + b * q_sb + h * q_sh + 16 * kq4);
+  const bf16x8 qx[2] = {qrow[0], qrow[1]};
+  float vv[17];
+#pragma unroll
+  for (int u = 0; u < 17; ++u) {
+    const int j = 4 * u + wave;  // keys of this wavefront: j = wave, wave + 4, ...
+    vv[u] = j < ncached ? to_f32(vc[(long)(lo + j) * c_st + lane]) : 0.f;
+  }
+  const float kn = to_f32(k_new[b * kn_sb + h * kn_sh + lane]);
+  const float vn = to_f32(v_new[b * vn_sb + h * vn_sh + lane]);
+  const float ql = to_f32(q[b * q_sb + h * q_sh + lane]);
+  if (wave == 0) {  // the new token joins the cache (row pos)
+    kc[(long)pos * c_st + lane] = (__bf16)kn;
+    vc[(long)pos * c_st + lane] = (__bf16)vn;
+  }
+
+  // ---- scores ----
+  float part = 0.f;
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part = __builtin_fmaf(to_f32(kx[c][i]), to_f32(qx[c][i]), part);
+  part += __shfl_xor(part, 1, 64);
+  part += __shfl_xor(part, 2, 64);
+  if (kq4 == 0) s_p[kj] = kj < ncached ? part * scale_log2e : -INFINITY;
+  if (wave == 0) {
+    const float self = wave_sum(ql * kn);
+    if (lane == 0) s_p[64] = self * scale_log2e;
+  }
   __syncthreads();
 
-  const int lo = pos - w_left > 0 ? pos - w_left : 0;
-  const int nkeys = pos - lo + 1;  // 1..65, the last one is the new token itself
-
-  // scores: pass 0 -> key lo+lane, pass 1 -> key lo+64+lane (only lane 0 can be live)
-  float sc[2];
-#pragma unroll
-  for (int pass = 0; pass < 2; ++pass) {
-    const int j = 64 * pass + lane;
-    float s = -INFINITY;
-    if (j < nkeys) {
-      const __bf16* row = (j == nkeys - 1) ? (k_new + b * kn_sb + h * kn_sh) : (kc + (long)(lo + j) * c_st);
-      float acc = 0.f;
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const bf16x8 x = *reinterpret_cast<const bf16x8*>(row + 8 * c);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(to_f32(x[i]), s_q[8 * c + i], acc);
-      }
-      s = acc * scale_log2e;
-    }
-    sc[pass] = s;
-  }
-  float mx = fmaxf(sc[0], sc[1]);
+  // ---- softmax over the 65 entries (every wavefront redundantly: no second barrier) ----
+  const float s0 = s_p[lane];
+  const float s1 = s_p[64];
+  float mx = fmaxf(s0, s1);
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-  sc[0] = __builtin_amdgcn_exp2f(sc[0] - mx);
-  sc[1] = __builtin_amdgcn_exp2f(sc[1] - mx);
-  const float denom = wave_sum(sc[0] + sc[1]);
+  const float p0 = __builtin_amdgcn_exp2f(s0 - mx);
+  const float p1 = __builtin_amdgcn_exp2f(s1 - mx);
+  const float denom = wave_sum(p0) + p1;
 
-  // output channel = lane
-  float acc = 0.f;
-  const int ncached = nkeys - 1;
-  for (int j0 = 0; j0 < ncached; j0 += 8) {
-    float vv[8];
+  // ---- output: channel = lane, this wavefront's keys ----
+  float acc = wave == 0 ? p1 * vn : 0.f;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int j = j0 + u;
-      vv[u] = j < ncached ? to_f32(vc[(long)(lo + j) * c_st + lane]) : 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int j = j0 + u;
-      const float p = __shfl(sc[j >> 6], j & 63, 64);
-      acc = __builtin_fmaf(j < ncached ? p : 0.f, vv[u], acc);
-    }
+  for (int u = 0; u < 17; ++u) {
+    const int j = 4 * u + wave;
+    const float p = __shfl(p0, j & 63, 64);
+    acc = __builtin_fmaf(j < ncached ? p : 0.f, vv[u], acc);
   }
-  {
-    const int j = nkeys - 1;
-    const float p = __shfl(sc[j >> 6], j & 63, 64);
-    acc = __builtin_fmaf(p, to_f32(vn), acc);
+  s_part[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0) {
+    const float tot = s_part[0][lane] + s_part[1][lane] + s_part[2][lane] + s_part[3][lane];
+    o[b * o_sb + h * o_sh + lane] = (__bf16)(tot / denom);
   }
-  o[b * o_sb + h * o_sh + lane] = (__bf16)(acc / denom);
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -321,12 +335,12 @@ extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const 
     BASED_REQUIRE(pos_host >= 0 && pos_host < max_seqlen, BASED_ERR_ARG,
                   "swa_step: position %ld outside the cache (max_seqlen %ld)", (long)pos_host,
                   (long)max_seqlen);
-  BASED_REQUIRE(c_sb % 8 == 0 && c_st % 8 == 0 && c_sh % 8 == 0 && kn_sb % 8 == 0 && kn_sh % 8 == 0,
-                BASED_ERR_ALIGN, "swa_step: cache and k_new strides must be multiples of 8 elements");
-  BASED_REQUIRE(aligned16(kcache) && aligned16(k_new), BASED_ERR_ALIGN,
-                "swa_step: kcache and k_new must be 16-byte aligned");
+  BASED_REQUIRE(c_sb % 8 == 0 && c_st % 8 == 0 && c_sh % 8 == 0 && q_sb % 8 == 0 && q_sh % 8 == 0,
+                BASED_ERR_ALIGN, "swa_step: cache and q strides must be multiples of 8 elements");
+  BASED_REQUIRE(aligned16(kcache) && aligned16(q), BASED_ERR_ALIGN,
+                "swa_step: kcache and q must be 16-byte aligned");
   if (B == 0) return BASED_OK;
-  hipLaunchKernelGGL(swa_step_kernel, dim3((unsigned)(B * H)), dim3(64), 0,
+  hipLaunchKernelGGL(swa_step_kernel, dim3((unsigned)(B * H)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), (const __bf16*)q, (const __bf16*)k_new,
                      (const __bf16*)v_new, (__bf16*)kcache, (__bf16*)vcache, (__bf16*)o, cache_seqlens,
                      (int)pos_host, (int)H, (int)max_seqlen, q_sb, q_sh, kn_sb, kn_sh, vn_sb, vn_sh,

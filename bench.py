@@ -39,8 +39,8 @@ D_EXP = 273
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
     "lin_step_kernel": 293097062,   # B=128, H=16, dv=64: fetch 146,863,104 + write 146,233,958
-    "lin_prefill_mfma_kernel": None,
-    "swa_prefill_kernel": None,
+    "lin_prefill_mfma_kernel": {96: 2253223000},  # B=96, L=4096, dv=64, states written; keyed by batch
+    "swa_prefill_kernel": 268549364,   # B=8, H=16, L=4096: fetch 201,440,500 + write 67,108,864
 }
 
 
@@ -121,7 +121,7 @@ def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
         "tok_s": B * L / (ms * 1e-3), "ms": ms, "B": B, "L": L, "dv": dv,
         "roofline": {"kernel": "lin_prefill_mfma_kernel", "bound": "mfma", "achieved": round(tf, 2),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["lin_prefill_mfma_kernel"],
+                     "traffic": MEASURED_TRAFFIC_BYTES["lin_prefill_mfma_kernel"].get(B),
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": byts,
                      "hbm_gbs": round(byts / (ms * 1e-3) / 1e9, 1)},
     }
