@@ -408,49 +408,52 @@ __device__ __forceinline__ void lin_prefill_chain(
   }
 
   // ---------------- expand the 160-slot state into the (dv, 273) decode layout ----------------
+  // Sixteen channels at a time: the four wavefronts scatter their slot tiles of one channel
+  // tile into a 16 x 273 fp32 block in LDS (each cross slot lands on both (i, j) and (j, i),
+  // with the factor that undoes the packing weights), and the block, which is contiguous in
+  // the decode state, leaves with coalesced 16-byte stores.
   if (kv_state != nullptr && last_seg) {
-    float* ks_row = k_state + bh * kExp;
-    auto expand = [&]() {
+    float* blk = reinterpret_cast<float*>(s_sb);
+    static_assert(16 * kExp * 4 <= kSbBytes, "expansion block must fit in the state image buffer");
+    static_for<kETiles>([&](auto ET) {
+      constexpr int et = decltype(ET)::value;
+      __syncthreads();  // the buffer is free (main loop done / previous block copied out)
+      float* row = blk + col * kExp;
       static_for<kOwn>([&](auto II) {
         constexpr int i = decltype(II)::value;
         constexpr int t = own_tile(wave, i);
 #pragma unroll
-        for (int et = 0; et < kETiles; ++et) {
-          float* row;
-          bool live;
-          if (et < 4) {
-            row = kv_state + (bh * dv + 64 * eb + 16 * et + col) * kExp;
-            live = true;
-          } else {
-            row = ks_row;
-            live = (col == 0) && (eb == 0);
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int j = 4 * grp + r;
-            const float x = S[i][et][r];
-            if (!live) continue;
-            if constexpr (t == 0) {
-              row[1 + kFeat + 17 * j] = x * (4.0f * kSqrt2);
-            } else if constexpr (t <= 7) {
-              const int pj = (j - t) & 15;
-              row[1 + kFeat + 16 * j + pj] = x * (2.0f * kSqrt2);
-              row[1 + kFeat + 16 * pj + j] = x * (2.0f * kSqrt2);
-            } else if constexpr (t == 8) {
-              if (j < 8) {
-                row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
-                row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
-              } else if (j == 8) {
-                row[0] = x;
-              }
-            } else {
-              row[1 + j] = x * 2.0f;
+        for (int r = 0; r < 4; ++r) {
+          const int j = 4 * grp + r;
+          const float x = S[i][et][r];
+          if constexpr (t == 0) {
+            row[1 + kFeat + 17 * j] = x * (4.0f * kSqrt2);
+          } else if constexpr (t <= 7) {
+            const int pj = (j - t) & 15;
+            row[1 + kFeat + 16 * j + pj] = x * (2.0f * kSqrt2);
+            row[1 + kFeat + 16 * pj + j] = x * (2.0f * kSqrt2);
+          } else if constexpr (t == 8) {
+            if (j < 8) {
+              row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
+              row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
+            } else if (j == 8) {
+              row[0] = x;
             }
+          } else {
+            row[1 + j] = x * 2.0f;
           }
         }
       });
-    };
-    expand();
+      __syncthreads();
+      if constexpr (et < 4) {
+        f32x4* dst = reinterpret_cast<f32x4*>(kv_state + (bh * dv + 64 * eb + 16 * et) * kExp);
+        const f32x4* src = reinterpret_cast<const f32x4*>(blk);
+        for (int idx = tid; idx < 16 * kExp / 4; idx += 64 * kWavesPerChain) dst[idx] = src[idx];
+      } else if (eb == 0) {
+        // channel tile 4 carries the normaliser state in its column 0 (= row 0 of the block)
+        for (int idx = tid; idx < kExp; idx += 64 * kWavesPerChain) k_state[bh * kExp + idx] = blk[idx];
+      }
+    });
   }
 }
 
