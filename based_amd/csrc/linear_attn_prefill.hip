@@ -205,6 +205,7 @@ __device__ __forceinline__ void lin_prefill_chain(
   // each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
   // loaded, so source lane 4j + a fetches channels 4a..4a+3 of token j of the group's four.
   const __bf16* vt_base = s_v + (4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
+  const __bf16* kt_base = s_k + (4 * grp + (col >> 2)) * kFeat + 4 * (col & 3);
   auto load_vt = [&](int et, int s) -> bf16x8 {
     const __bf16* p0 = vt_base + (32 * s) * kVStride + 16 * et;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
@@ -233,15 +234,28 @@ __device__ __forceinline__ void lin_prefill_chain(
     // ---------------- publish the bf16 image of the own share of the state ----------------
     // s_sb[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes 0..7 come
     // from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
+    // A wavefront that owns both slot tiles of a slab writes the operand in one 16-byte piece.
+    if constexpr (MODE != kModeDelta) {
+      static_for<kOwn>([&](auto II) {
+        constexpr int i = decltype(II)::value;
+        constexpr int t = own_tile(wave, i);
+        constexpr bool pair_lo = (t % 2 == 0) && (i + 1 < kOwn);
+        constexpr bool pair_hi = (t % 2 == 1) && (i > 0);
+        if constexpr (pair_lo) {
 #pragma unroll
-    for (int i = 0; i < (MODE == kModeDelta ? 0 : kOwn); ++i) {
-      constexpr int kBase = own_tile(wave, 0);
-      const int t = kBase + i;
+          for (int et = 0; et < kETiles; ++et) {
+            const u32x4 w4 = {pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]),
+                              pack_bf16(S[i + 1][et][0], S[i + 1][et][1]), pack_bf16(S[i + 1][et][2], S[i + 1][et][3])};
+            *reinterpret_cast<u32x4*>(s_sb + (((t >> 1) * kETiles + et) * 64 + lane) * 16) = w4;
+          }
+        } else if constexpr (!pair_hi) {
 #pragma unroll
-      for (int et = 0; et < kETiles; ++et) {
-        const uint2 w2 = make_uint2(pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]));
-        *reinterpret_cast<uint2*>(s_sb + (((t >> 1) * kETiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
-      }
+          for (int et = 0; et < kETiles; ++et) {
+            const uint2 w2 = make_uint2(pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]));
+            *reinterpret_cast<uint2*>(s_sb + (((t >> 1) * kETiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
+          }
+        }
+      });
     }
     __syncthreads();
 
@@ -359,11 +373,19 @@ __device__ __forceinline__ void lin_prefill_chain(
       for (int s = 0; s < 2; ++s) {
         float kraw[8], k16[8];
         bf16x8 vt[4];
+        {
+          // k^T (lane <-> feature col, slots <-> tokens) with the same transposing read as V^T
+          const __bf16* p0 = kt_base + (32 * s) * kFeat;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kFeat));
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-          const float x = to_f32(s_k[slot_token(s, grp, jj) * kFeat + col]);
-          kraw[jj] = x;
-          k16[jj] = x * (1.0f / 16.0f);
+          for (int jj = 0; jj < 8; ++jj) {
+            const uint32_t bits = (uint32_t)(uint16_t)(jj < 4 ? lo[jj & 3] : hi[jj & 3]) << 16;
+            const float x = __builtin_bit_cast(float, bits);
+            kraw[jj] = x;
+            k16[jj] = x * (1.0f / 16.0f);
+          }
         }
 #pragma unroll
         for (int et = 0; et < 4; ++et) vt[et] = load_vt(et, s);
