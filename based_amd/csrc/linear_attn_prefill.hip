@@ -171,6 +171,8 @@ __device__ __forceinline__ void lin_prefill_chain(
   const uint32_t one2 = col == 0 ? 0x3F803F80u : 0u;
   const bf16x8 ones_op = __builtin_bit_cast(bf16x8, u32x4{one2, one2, one2, one2});
   const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
+  const uint32_t t8_keep = col < 8 ? 0xFFFFFFFFu : 0u;      // slot tile 8: pair products live in positions 0..7,
+  const uint32_t t8_const = col == 8 ? 0x3F803F80u : 0u;    // the constant feature (bf16 1.0) in position 8
 
   // Global loads of a chunk, issued one phase ahead of their use.  q (wave 0) / k (wave 1):
   // 64 rows x 32 B, lane <-> row.  v: 64 rows x 128 B = 512 pieces of 16 B, two per thread:
@@ -400,15 +402,21 @@ __device__ __forceinline__ void lin_prefill_chain(
             } else if constexpr (t <= 7) {
               f[jj] = row_ror<t>(kraw[jj]) * k16[jj];
             } else if constexpr (t == 8) {
-              const float prod = row_ror<8>(kraw[jj]) * k16[jj];
-              // position 8 is the constant feature (real tokens only), 9..15 are unused
-              const float cst = (col == 8 && slot_token(s, grp, jj) < ntok) ? 1.0f : 0.0f;
-              f[jj] = col < 8 ? prod : cst;
+              f[jj] = row_ror<8>(kraw[jj]) * k16[jj];  // positions 8..15 are replaced below
             } else {
               f[jj] = kraw[jj] * 0.25f;
             }
           }
-          const bf16x8 ak = pack8(f);
+          bf16x8 ak = pack8(f);
+          if constexpr (t == 8) {
+            // position 8 is the constant feature, 9..15 are unused.  The constant is also set
+            // for the zero rows that pad the last chunk: their v is zero, and the count they
+            // add to the normaliser state is taken off when the state is written out.
+            u32x4 w = __builtin_bit_cast(u32x4, ak);
+#pragma unroll
+            for (int d = 0; d < 4; ++d) w[d] = (w[d] & t8_keep) | t8_const;
+            ak = __builtin_bit_cast(bf16x8, w);
+          }
 #pragma unroll
           for (int et = 0; et < 4; ++et) S[i][et] = mfma(ak, vt[et], S[i][et]);
           S[i][4] = mfma(ak, ones_op, S[i][4]);
@@ -435,6 +443,7 @@ __device__ __forceinline__ void lin_prefill_chain(
   // with the factor that undoes the packing weights), and the block, which is contiguous in
   // the decode state, leaves with coalesced 16-byte stores.
   if (kv_state != nullptr && last_seg) {
+    const int pad_tokens = (kChunk - (t_end - t_begin) % kChunk) % kChunk;
     float* blk = reinterpret_cast<float*>(s_sb);
     static_assert(16 * kExp * 4 <= kSbBytes, "expansion block must fit in the state image buffer");
     static_for<kETiles>([&](auto ET) {
@@ -459,7 +468,8 @@ __device__ __forceinline__ void lin_prefill_chain(
               row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
               row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
             } else if (j == 8) {
-              row[0] = x;
+              // constant feature; in the normaliser column it counted the padding rows too
+              row[0] = et == 4 ? x - (float)pad_tokens : x;
             }
           } else {
             row[1 + j] = x * 2.0f;

@@ -36,6 +36,8 @@ def _check(dev, q, k, v, dtype, with_state=True):
         stol = 5e-3 if dtype == torch.bfloat16 else 1e-5
         assert rel_l2(kv, kv_ref) < stol
         assert rel_l2(ks, ks_ref) < stol
+        # the constant feature's entry of the normaliser state counts the tokens exactly
+        assert torch.all(ks[..., 0] == q.shape[2])
     return y
 
 
