@@ -182,7 +182,8 @@ def main():
     ap.add_argument("--only", choices=["decode", "prefill", "swa", "copy"], default=None,
                     help="one workload only; 'copy' is a plain 256 MiB device copy used to calibrate the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
-    ap.add_argument("--prefill-batch", type=int, default=8)
+    ap.add_argument("--prefill-batches", default="1,8,48,96",
+                    help="comma-separated batch sizes of the L=4096 prefill lines")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU (every (batch, head) pair is independent; "
@@ -217,7 +218,7 @@ def main():
                     "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
                     "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5)})
     if args.only in (None, "prefill"):
-        pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({1, args.prefill_batch, 48, 96})]
+        pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
     if args.only in (None, "swa"):
         s = bench_swa(torch, ops, 20, 3)

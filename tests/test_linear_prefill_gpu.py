@@ -50,6 +50,24 @@ def test_bf16_mfma_matches_oracle(dev, B, H, L, dv):
     _check(dev, q, k, v, torch.bfloat16)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_golden_reference_causal_product(dev, dtype):
+    """Both prefill kernels against the committed output of the reference's compiled CPU causal
+    product (tests/golden/causal_dot_E273_M64.npz; inputs are bf16-representable)."""
+    import os
+
+    import numpy as np
+    from based_amd import ops
+
+    print(f"prefill golden case dtype={dtype}", flush=True)
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "causal_dot_E273_M64.npz"))
+    q, k, v = (torch.from_numpy(g[n]).to(dtype) for n in ("q", "k", "v"))
+    y_gold = torch.from_numpy(g["numerator"]) / (torch.from_numpy(g["normaliser"]) + 1e-12)
+    y, _, _ = ops.linear_attn_prefill(q.to(dev), k.to(dev), v.to(dev), return_state=False)
+    torch.cuda.synchronize()
+    assert rel_l2(y.float(), y_gold) < TOL[dtype]
+
+
 def test_bf16_small_qk_scale(dev):
     """q, k scaled by 1/sqrt(16) as in the reference's CPU-runnable configuration."""
     q, k, v = _qkv(1, 4, 512, 64, torch.bfloat16, seed=8, qk_scale=0.25)

@@ -111,6 +111,25 @@ def test_numerator_matches_reference_cpp():
         assert float((y - y_ref).norm() / y_ref.norm()) < 1e-5
 
 
+def test_golden_causal_product_fixture():
+    """Committed output of the reference's compiled CPU causal product (written by
+    tests/golden/make_causal_dot_golden.py): numerator and normaliser at E = 273, M = 64."""
+    import os
+
+    import numpy as np
+
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "causal_dot_E273_M64.npz"))
+    q, k, v = (torch.from_numpy(g[n]) for n in ("q", "k", "v"))
+    num, den = torch.from_numpy(g["numerator"]), torch.from_numpy(g["normaliser"])
+    y_gold = num / (den + 1e-12)
+    for y in (O.linear_attn_quadratic(q, k, v), O.linear_attn_cumsum(q, k, v)):
+        assert float((y - y_gold).norm() / y_gold.norm()) < 1e-5
+    # the normaliser alone pins the closed form 1 + s + s^2/2 summed over the causal prefix
+    s_ = torch.einsum("bhid,bhjd->bhij", q, k) / 4.0
+    den_closed = torch.tril(1 + s_ + s_ * s_ / 2).sum(-1, keepdim=True)
+    assert float((den - den_closed).norm() / den_closed.norm()) < 1e-5
+
+
 def test_smoke_script_formulation():
     """The comparison the reference's causal-product smoke script makes (positive q, k, v;
     cumulative-sum form), whose recorded difference is 7.4e-05 in bf16: here in fp64 on the
