@@ -22,7 +22,6 @@ namespace based {
 
 constexpr int kHeadDim = 64;
 constexpr int kQTile = 64;          // queries per workgroup
-constexpr int kKeysWG = 128;        // keys staged per workgroup: [q0-64, q0+64)
 constexpr int kKStride = 72;        // bf16 per K row in LDS (144 B: 16 rows x 16 B reads hit 64 distinct banks)
 constexpr int kVStride = 80;        // bf16 per V row in LDS (160 B: conflict-free transposing reads)
 constexpr int kOStride = 72;        // bf16 per row of a wavefront's output staging tile
@@ -33,13 +32,15 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 __global__ __launch_bounds__(256) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
-    __bf16* __restrict__ o, int H, int L, int n_tiles, long q_sb, long q_sl, long q_sh, long k_sb,
-    long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
+    __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
+    long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
     int w_left, float scale_log2e) {
-  __shared__ __align__(16) __bf16 s_k[kKeysWG * kKStride];
-  __shared__ __align__(16) __bf16 s_v[kKeysWG * kVStride];
-  // the output staging tiles reuse the K rows once every wavefront is done with them
-  static_assert(4 * 16 * kOStride <= kKeysWG * kKStride, "output staging must fit in the K region");
+  // Two blocks of 64 K rows and 64 V rows: one holds the current tile's own keys, the other the
+  // 64 keys to its left.  Moving on by one tile, "own" becomes "left" without a copy and the
+  // old left block takes the next tile's rows.
+  __shared__ __align__(16) __bf16 s_k[2 * kQTile * kKStride];
+  __shared__ __align__(16) __bf16 s_v[2 * kQTile * kVStride];
+  static_assert(kOStride == kKStride, "output staging reuses whole K rows of the left block");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -47,144 +48,181 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
   const int col = lane & 15;   // query (B operand / accumulator column), or row of an A tile
   const int grp = lane >> 4;   // 0..3: which 8 contraction slots / which 4 accumulator rows
 
-  // Workgroups are dealt to the 8 XCDs round-robin by id.  Neighbouring query tiles of one
-  // (batch, head) read overlapping K/V rows (a 64-row halo), so consecutive tiles are laid along
-  // one XCD and the halo is an L2 hit: item = (id mod 8) * ceil(n / 8) + id / 8.
-  const long n_items = gridDim.x;
-  long item = blockIdx.x;
-  if (n_items % 8 == 0) item = (item % 8) * (n_items / 8) + item / 8;
-  const int tile = (int)(item % n_tiles);
-  const long bh = item / n_tiles;
+  // work item: a run of up to run_tiles consecutive query tiles of one (batch, head)
+  const int runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
+  const int run = (int)(blockIdx.x % runs_per_seq);
+  const long bh = blockIdx.x / runs_per_seq;
   const int h = (int)(bh % H), b = (int)(bh / H);
-  const int q0 = tile * kQTile;
+  const int tile_begin = run * run_tiles;
+  const int tile_end = tile_begin + run_tiles < n_tiles ? tile_begin + run_tiles : n_tiles;
 
   q += b * q_sb + h * q_sh;
   k += b * k_sb + h * k_sh;
   v += b * v_sb + h * v_sh;
   o += b * o_sb + h * o_sh;
 
-  // ---- stage K and V rows of keys [q0-64, q0+64) as they come: 1024 pieces of 16 B each ----
-  {
-    u32x4 kp[4], vp[4];
+  // Rows of a 64-row block moved by this thread: 16 wave + 8 i + lane / 8 (i = 0, 1), 16 bytes at
+  // channel 8 (lane % 8).  A wavefront only ever writes block rows 16 wave .. 16 wave + 15,
+  // the rows that double as its output staging tile.
+  const int my_row = 16 * wave + (lane >> 3);
+  const int my_seg = 8 * (lane & 7);
+  auto load_rows = [&](int key0, u32x4 (&kp)[2], u32x4 (&vp)[2]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int piece = 256 * i + tid;
-      const int key = q0 - 64 + (piece >> 3);
+    for (int i = 0; i < 2; ++i) {
+      const int key = key0 + my_row + 8 * i;
       const u32x4 z4 = {0, 0, 0, 0};
       kp[i] = vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
       if (key >= 0 && key < L) {
-        kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + 8 * (piece & 7));
-        vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + 8 * (piece & 7));
+        kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + my_seg);
+        vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + my_seg);
       }
     }
+  };
+  auto store_rows = [&](int blk, const u32x4 (&kp)[2], const u32x4 (&vp)[2]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int piece = 256 * i + tid;
-      *reinterpret_cast<u32x4*>(s_k + (piece >> 3) * kKStride + 8 * (piece & 7)) = kp[i];
-      *reinterpret_cast<u32x4*>(s_v + (piece >> 3) * kVStride + 8 * (piece & 7)) = vp[i];
+    for (int i = 0; i < 2; ++i) {
+      const int row = blk * kQTile + my_row + 8 * i;
+      *reinterpret_cast<u32x4*>(s_k + row * kKStride + my_seg) = kp[i];
+      *reinterpret_cast<u32x4*>(s_v + row * kVStride + my_seg) = vp[i];
     }
+  };
+  // Q operand of this wavefront's 16 queries, straight from global memory
+  auto load_q = [&](int q0, bf16x8 (&bq)[2]) {
+    const int n = q0 + 16 * wave + col;
+#pragma unroll
+    for (int ds = 0; ds < 2; ++ds) {
+      bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (n < L) x = *reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp);
+      bq[ds] = x;
+    }
+  };
+
+  int q0 = tile_begin * kQTile;
+  u32x4 kp[2], vp[2];
+  bf16x8 bq[2], bq_next[2];
+  {
+    // first tile: own rows in block 0, the 64 keys to the left in block 1 (one round trip)
+    u32x4 kl[2], vl[2];
+    load_rows(q0 - kQTile, kl, vl);
+    load_rows(q0, kp, vp);
+    load_q(q0, bq);
+    store_rows(1, kl, vl);
+    store_rows(0, kp, vp);
+  }
+  if (tile_begin + 1 < tile_end) {  // the next tile's rows travel while this one is computed
+    load_rows(q0 + kQTile, kp, vp);
+    load_q(q0 + kQTile, bq_next);
   }
 
-  // ---- Q operand of this wavefront's 16 queries, straight from global memory ----
-  const int n0 = q0 + 16 * wave;            // first query of this wavefront
-  const int n = n0 + col;                   // this lane's query
-  bf16x8 bq[2];
-#pragma unroll
-  for (int ds = 0; ds < 2; ++ds) {
-    bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-    if (n < L) x = *reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp);
-    bq[ds] = x;
-  }
-  __syncthreads();
+  for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile) {
+    const int own = (tile - tile_begin) & 1;  // block with keys [q0, q0+64); 1 - own has [q0-64, q0)
+    const int n0 = q0 + 16 * wave;            // first query of this wavefront
+    const int n = n0 + col;                   // this lane's query
+    // staged key index x (0..127 <-> key q0 - 64 + x) -> row of the ring
+    auto ring_row = [&](int x) { return ((x < kQTile ? 1 - own : own) * kQTile) + (x & (kQTile - 1)); };
+    __syncthreads();  // the staged rows are visible
 
-  // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
-  // wavefront w sees staged keys 16 w .. 16 w + 79 (tile i = keys 16 w + 16 i ..)
-  f32x4 st[5];
+    // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
+    // wavefront w sees staged keys 16 w .. 16 w + 79 (tile i = keys 16 w + 16 i ..)
+    f32x4 st[5];
 #pragma unroll
-  for (int i = 0; i < 5; ++i) {
-    const __bf16* row = s_k + (16 * wave + 16 * i + col) * kKStride + 8 * grp;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < 5; ++i) {
+      const __bf16* row = s_k + (ring_row(16 * wave + 16 * i) + col) * kKStride + 8 * grp;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ds = 0; ds < 2; ++ds)
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(row + 32 * ds), bq[ds], acc, 0, 0, 0);
-    st[i] = acc;
-  }
+      for (int ds = 0; ds < 2; ++ds)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(row + 32 * ds), bq[ds], acc, 0, 0, 0);
+      st[i] = acc;
+    }
 
-  // ---- masked softmax over keys; lane holds keys 16 i + 4 grp + r of query n ----
-  float mx = -INFINITY;
+    // ---- masked softmax over keys; lane holds keys 16 i + 4 grp + r of query n ----
+    float mx = -INFINITY;
 #pragma unroll
-  for (int i = 0; i < 5; ++i)
+    for (int i = 0; i < 5; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int key = n0 - 64 + 16 * i + 4 * grp + r;
-      const bool keep = key >= 0 && key <= n && key >= n - w_left;
-      const float sc = keep ? st[i][r] * scale_log2e : -INFINITY;
-      st[i][r] = sc;
-      mx = fmaxf(mx, sc);
-    }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  float sum = 0.f;
+      for (int r = 0; r < 4; ++r) {
+        const int key = n0 - 64 + 16 * i + 4 * grp + r;
+        const bool keep = key >= 0 && key <= n && key >= n - w_left;
+        const float sc = keep ? st[i][r] * scale_log2e : -INFINITY;
+        st[i][r] = sc;
+        mx = fmaxf(mx, sc);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float sum = 0.f;
 #pragma unroll
-  for (int i = 0; i < 5; ++i)
+    for (int i = 0; i < 5; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float p = __builtin_amdgcn_exp2f(st[i][r] - mx);  // exp2(-inf) = 0 for masked keys
-      st[i][r] = p;
-      sum += p;
-    }
-  sum += __shfl_xor(sum, 16, 64);
-  sum += __shfl_xor(sum, 32, 64);
+      for (int r = 0; r < 4; ++r) {
+        const float p = __builtin_amdgcn_exp2f(st[i][r] - mx);  // exp2(-inf) = 0 for masked keys
+        st[i][r] = p;
+        sum += p;
+      }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
 
-  // ---- O^T = V^T P^T: 4 channel tiles x 3 key slabs of 32 (last slab half empty) ----
-  // V^T operand tiles come from the row-major V rows with the transposing 64-bit LDS read:
-  // in each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
-  // loaded, so source lane 4j + a fetches channels 4a..4a+3 of key j of the group's four.
-  const __bf16* vt_base = s_v + (16 * wave + 4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
-  f32x4 ot[4];
+    // ---- O^T = V^T P^T: 4 channel tiles x 3 key slabs of 32 (last slab half empty) ----
+    // V^T operand tiles come from the row-major V rows with the transposing 64-bit LDS read:
+    // in each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
+    // loaded, so source lane 4j + a fetches channels 4a..4a+3 of key j of the group's four.
+    const int vt_off = (4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
+    f32x4 ot[4];
 #pragma unroll
-  for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int s = 0; s < 3; ++s) {
-    // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent for s = 2)
-    u32x4 pb;
-    pb[0] = pack_bf16(st[2 * s][0], st[2 * s][1]);
-    pb[1] = pack_bf16(st[2 * s][2], st[2 * s][3]);
-    if (s < 2) {
-      pb[2] = pack_bf16(st[2 * s + 1][0], st[2 * s + 1][1]);
-      pb[3] = pack_bf16(st[2 * s + 1][2], st[2 * s + 1][3]);
-    } else {
-      pb[2] = 0u;
-      pb[3] = 0u;
+    for (int s = 0; s < 3; ++s) {
+      // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent for s = 2)
+      u32x4 pb;
+      pb[0] = pack_bf16(st[2 * s][0], st[2 * s][1]);
+      pb[1] = pack_bf16(st[2 * s][2], st[2 * s][3]);
+      if (s < 2) {
+        pb[2] = pack_bf16(st[2 * s + 1][0], st[2 * s + 1][1]);
+        pb[3] = pack_bf16(st[2 * s + 1][2], st[2 * s + 1][3]);
+      } else {
+        pb[2] = 0u;
+        pb[3] = 0u;
+      }
+      const bf16x8 bp = __builtin_bit_cast(bf16x8, pb);
+      const __bf16* lo_rows = s_v + ring_row(16 * wave + 32 * s) * kVStride + vt_off;
+      const __bf16* hi_rows = s_v + ring_row((16 * wave + 32 * s + 16) & (2 * kQTile - 1)) * kVStride + vt_off;
+#pragma unroll
+      for (int et = 0; et < 4; ++et) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + 16 * et));
+        s16x4 hi = {0, 0, 0, 0};
+        if (s < 2)
+          hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + 16 * et));
+        const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
+      }
     }
-    const bf16x8 bp = __builtin_bit_cast(bf16x8, pb);
+
+    // ---- normalise; stage the 16 x 64 tile in LDS so each lane stores 16 contiguous bytes ----
+    const float inv = 1.0f / sum;
+    __syncthreads();  // every wavefront is done with the left block
+    __bf16* so = s_k + ((1 - own) * kQTile + 16 * wave) * kKStride;
 #pragma unroll
     for (int et = 0; et < 4; ++et) {
-      const __bf16* p0 = vt_base + (32 * s) * kVStride + 16 * et;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
-      s16x4 hi = {0, 0, 0, 0};
-      if (s < 2)
-        hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kVStride));
-      const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
+      const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
+      const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
+      *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
     }
-  }
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+      const int row = 8 * hlf + (lane >> 3);
+      const u32x4 w4 = *reinterpret_cast<const u32x4*>(so + row * kOStride + 8 * (lane & 7));
+      if (n0 + row < L) *reinterpret_cast<u32x4*>(o + (long)(n0 + row) * o_sl + 8 * (lane & 7)) = w4;
+    }
 
-  // ---- normalise; stage the 16 x 64 tile in LDS so each lane stores 16 contiguous bytes ----
-  const float inv = 1.0f / sum;
-  __syncthreads();  // all S^T products have consumed the K rows
-  __bf16* so = s_k + wave * (16 * kOStride);
-#pragma unroll
-  for (int et = 0; et < 4; ++et) {
-    const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
-    const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
-    *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
-  }
-#pragma unroll
-  for (int hlf = 0; hlf < 2; ++hlf) {
-    const int row = 8 * hlf + (lane >> 3);
-    const u32x4 w4 = *reinterpret_cast<const u32x4*>(so + row * kOStride + 8 * (lane & 7));
-    if (n0 + row < L) *reinterpret_cast<u32x4*>(o + (long)(n0 + row) * o_sl + 8 * (lane & 7)) = w4;
+    // ---- the left block takes the next tile's rows (this wavefront's own 16 rows of it) ----
+    if (tile + 1 < tile_end) {
+      store_rows(1 - own, kp, vp);
+      bq[0] = bq_next[0];
+      bq[1] = bq_next[1];
+      if (tile + 2 < tile_end) {
+        load_rows(q0 + 2 * kQTile, kp, vp);
+        load_q(q0 + 2 * kQTile, bq_next);
+      }
+    }
   }
 }
 
@@ -307,10 +345,16 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   if (B == 0 || L == 0) return BASED_OK;
   const int64_t n_tiles = (L + kQTile - 1) / kQTile;
   BASED_REQUIRE(B * H * n_tiles < (1ll << 31), BASED_ERR_SHAPE, "swa_prefill: grid too large");
-  dim3 grid((unsigned)(B * H * n_tiles)), block(256);
+  // Consecutive query tiles of one (batch, head) are walked by one workgroup (the keys to the left
+  // of a tile are the previous tile's own keys, already staged); runs are as long as still
+  // leaves about four workgroups for each of the 256 compute units.
+  int64_t run_tiles = B * H * n_tiles / 1024;
+  run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
+  const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
+  dim3 grid((unsigned)(B * H * runs_per_seq)), block(256);
   hipLaunchKernelGGL(swa_prefill_kernel, grid, block, 0, static_cast<hipStream_t>(stream),
                      (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o, (int)H, (int)L,
-                     (int)n_tiles, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh,
+                     (int)n_tiles, (int)run_tiles, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh,
                      w_left, scale * 1.4426950408889634f);
   return check_launch("swa_prefill");
 }
