@@ -173,6 +173,52 @@ def cpu_baseline_decode(torch, B=128, H=16, dv=64, sample_steps=8):
             "host_cpu_count": os.cpu_count(), "ms_per_step": round(dt * 1e3, 2)}
 
 
+def cpu_baseline_prefill(torch, H=16, L=1024, dv=64, reps=3):
+    """configs[0] on the host: the quadratic causal form (the reference's default
+    parallel_forward), B=1, fp32, plus the compiled reference C++ causal product when present."""
+    from oracle import based_oracle as O
+    from oracle import ref_loader
+
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, H, L, 16, generator=g) * 0.25
+    k = torch.randn(1, H, L, 16, generator=g) * 0.25
+    v = torch.randn(1, H, L, dv, generator=g)
+    O.linear_attn_quadratic(q, k, v)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        O.linear_attn_quadratic(q, k, v)
+    dt = (time.perf_counter() - t0) / reps
+    out = {"value": round(L / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"configs[0]: B=1 H={H} L={L} dv={dv} fp32, oracle linear_attn_quadratic, {reps} passes",
+           "ms": round(dt * 1e3, 2)}
+    if ref_loader.available():
+        fq, fk = O.taylor_exp(q), O.taylor_exp(k)
+        ref_loader.causal_dot_product(fq, fk, v)
+        t0 = time.perf_counter()
+        ref_loader.causal_dot_product(fq, fk, v)
+        dt = time.perf_counter() - t0
+        out["reference_cpp"] = {"value": round(L / dt, 1), "unit": "tokens/s", "kind": "reference", "ms": round(dt * 1e3, 2),
+                                "sample": "same inputs, compiled causal_dot_product on precomputed 273-dim feature maps "
+                                          "(numerator only), 1 pass"}
+    return out
+
+
+def cpu_baseline_swa(torch, H=16, L=4096, reps=2):
+    """One batch entry of configs[2] on the host (masked-softmax statement of the window attention)."""
+    from oracle import based_oracle as O
+
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, L, H, 64, generator=g) for _ in range(3))
+    O.sliding_window_attn(q, k, v, w_left=64)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        O.sliding_window_attn(q, k, v, w_left=64)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(L / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"B=1 of configs[2]'s 8: H={H} L={L} window 64 fp32, oracle sliding_window_attn, {reps} passes",
+            "ms": round(dt * 1e3, 2)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -233,6 +279,9 @@ def main():
                     "roofline": out["swa"]["roofline"]})
     if not args.no_cpu and args.only in (None, "decode"):
         out["cpu_baseline"] = cpu_baseline_decode(torch)
+    if not args.no_cpu and args.only is None:
+        out["cpu_baseline_prefill"] = cpu_baseline_prefill(torch)
+        out["cpu_baseline_swa"] = cpu_baseline_swa(torch)
     print(json.dumps(out))
 
 
