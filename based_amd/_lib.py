@@ -43,6 +43,14 @@ SIGNATURES = {
         C.c_int,
         [_P, _P, _P, _P] + [_I64] * 3 + [_I64] * 12 + [C.c_int, C.c_float, C.c_int, _P],
     ),
+    "based_gated_conv_prefill": (
+        C.c_int,
+        [_P, _P, _P, _P, _P] + [_I64] * 3 + [C.c_int] + [_I64] * 4 + [C.c_int, C.c_int, _P],
+    ),
+    "based_gated_conv_step": (
+        C.c_int,
+        [_P, _P, _P, _P, _P] + [_I64] * 2 + [C.c_int] + [_I64] * 2 + [C.c_int, C.c_int, _P],
+    ),
     "based_swa_step": (
         C.c_int,
         [_P, _P, _P, _P, _P, _P, _P, _I64] + [_I64] * 3 + [_I64] * 8 + [_I64] * 3

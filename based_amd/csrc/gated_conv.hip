@@ -1,0 +1,246 @@
+// Gated short convolution of the Based stack for gfx950 (memory-bound, element-wise):
+//   y[b,l,c] = silu( sum_j w[c,j] * u1[b, l-K+1+j, c] (+ bias[c]) ) * u2[b,l,c]
+// with u = [u1 | u2] the (B, L, 2D) output of the block's input projection
+// (based/models/mixers/convolution.py:195-210: depthwise causal Conv1d, SiLU, gate), plus the
+// single-token form on a rolling (B, D, K) state (convolution.py:88-109).
+//
+// Prefill: a thread owns 16 bytes of channels (8 bf16 / 4 fp32) and walks kTokens consecutive
+// tokens with the last K-1 inputs kept in registers, so every u element is read once (plus a
+// K-1 row halo per token block) and every y element written once, all as 16-byte accesses that
+// a wavefront coalesces into full rows.
+#include "common.hpp"
+
+namespace based {
+
+constexpr int kConvTokens = 16;   // tokens per thread in the prefill kernel
+constexpr int kConvMaxK = 4;      // supported kernel sizes: 2..4
+
+template <typename T> struct Vec16;
+template <> struct Vec16<__bf16> {
+  static constexpr int kN = 8;
+  typedef bf16x8 type;
+};
+template <> struct Vec16<float> {
+  static constexpr int kN = 4;
+  typedef f32x4 type;
+};
+
+__device__ __forceinline__ float silu(float a) { return a / (1.0f + __expf(-a)); }
+
+template <typename T> __device__ __forceinline__ float load_as_f32(const void* p, long i) {
+  return to_f32(reinterpret_cast<const T*>(p)[i]);
+}
+__device__ __forceinline__ float load_dyn(const void* p, long i, int dtype) {
+  return dtype == BASED_BF16 ? load_as_f32<__bf16>(p, i) : load_as_f32<float>(p, i);
+}
+__device__ __forceinline__ void store_dyn(void* p, long i, int dtype, float x) {
+  if (dtype == BASED_BF16)
+    reinterpret_cast<__bf16*>(p)[i] = (__bf16)x;
+  else
+    reinterpret_cast<float*>(p)[i] = x;
+}
+
+template <typename T, int K>
+__global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
+    const T* __restrict__ u, const T* __restrict__ weight, const T* __restrict__ bias, T* __restrict__ y,
+    void* __restrict__ state, int L, int D, long u_sb, long u_sl, long y_sb, long y_sl, int state_dtype) {
+  constexpr int N = Vec16<T>::kN;
+  typedef typename Vec16<T>::type vec_t;
+  const int c0 = (blockIdx.x * 256 + threadIdx.x) * N;  // first channel of this thread
+  if (c0 >= D) return;
+  const int l0 = blockIdx.y * kConvTokens;
+  const int b = blockIdx.z;
+  const T* u1 = u + b * u_sb + c0;
+  const T* u2 = u1 + D;
+  T* yo = y + b * y_sb + c0;
+
+  float w[N][K], bs[N];
+#pragma unroll
+  for (int c = 0; c < N; ++c) {
+#pragma unroll
+    for (int j = 0; j < K; ++j) w[c][j] = to_f32(weight[(long)(c0 + c) * K + j]);
+    bs[c] = bias != nullptr ? to_f32(bias[c0 + c]) : 0.0f;
+  }
+
+  // the K-1 inputs before the block (zeros before the sequence start)
+  float win[K][N];
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) {
+    const int l = l0 - (K - 1) + j;
+    vec_t x = {};
+    if (l >= 0) x = *reinterpret_cast<const vec_t*>(u1 + (long)l * u_sl);
+#pragma unroll
+    for (int c = 0; c < N; ++c) win[j][c] = to_f32(x[c]);
+  }
+
+  const int ntok = L - l0 < kConvTokens ? L - l0 : kConvTokens;
+  constexpr int kBatch = 4;  // tokens whose loads are in flight together
+#pragma unroll
+  for (int t0 = 0; t0 < kConvTokens; t0 += kBatch) {
+    vec_t x1[kBatch], x2[kBatch];
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      x1[i] = vec_t{};
+      x2[i] = vec_t{};
+      if (t0 + i < ntok) {
+        x1[i] = *reinterpret_cast<const vec_t*>(u1 + (long)(l0 + t0 + i) * u_sl);
+        x2[i] = *reinterpret_cast<const vec_t*>(u2 + (long)(l0 + t0 + i) * u_sl);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kBatch; ++i) {
+      if (t0 + i < ntok) {
+        vec_t out;
+#pragma unroll
+        for (int c = 0; c < N; ++c) {
+          win[K - 1][c] = to_f32(x1[i][c]);
+          float acc = bs[c];
+#pragma unroll
+          for (int j = 0; j < K; ++j) acc = __builtin_fmaf(w[c][j], win[j][c], acc);
+          out[c] = from_f32<T>(silu(acc) * to_f32(x2[i][c]));
+#pragma unroll
+          for (int j = 0; j < K - 1; ++j) win[j][c] = win[j + 1][c];
+        }
+        *reinterpret_cast<vec_t*>(yo + (long)(l0 + t0 + i) * y_sl) = out;
+      }
+    }
+  }
+
+  // rolling state for decoding: the last K inputs of every channel, oldest first
+  if (state != nullptr && l0 + ntok == L) {
+#pragma unroll
+    for (int c = 0; c < N; ++c) {
+      const long base = ((long)b * D + c0 + c) * K;
+      // after the last token the window holds inputs L-K+1 .. L-1 in win[0..K-2]; input L-K is
+      // gone from it, so re-read it (it exists only if L >= K)
+      float oldest = 0.0f;
+      if (L - K >= 0) oldest = to_f32(u1[(long)(L - K) * u_sl + c]);
+      store_dyn(state, base, state_dtype, oldest);
+#pragma unroll
+      for (int j = 1; j < K; ++j) store_dyn(state, base + j, state_dtype, win[j - 1][c]);
+    }
+  }
+}
+
+template <typename T, int K>
+__global__ __launch_bounds__(256) void gated_conv_step_kernel(
+    const T* __restrict__ u, void* __restrict__ state, const T* __restrict__ weight, const T* __restrict__ bias,
+    T* __restrict__ y, int B, int D, long u_sb, long y_sb, int state_dtype) {
+  constexpr int N = Vec16<T>::kN;
+  typedef typename Vec16<T>::type vec_t;
+  const long item = (long)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = D / N;
+  if (item >= (long)B * per_row) return;
+  const int b = (int)(item / per_row);
+  const int c0 = (int)(item % per_row) * N;
+  const vec_t x1 = *reinterpret_cast<const vec_t*>(u + b * u_sb + c0);
+  const vec_t x2 = *reinterpret_cast<const vec_t*>(u + b * u_sb + D + c0);
+  vec_t out;
+#pragma unroll
+  for (int c = 0; c < N; ++c) {
+    const long base = ((long)b * D + c0 + c) * K;
+    float st[K];
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) st[j] = load_dyn(state, base + j + 1, state_dtype);  // roll by one
+    st[K - 1] = to_f32(x1[c]);
+    float acc = bias != nullptr ? to_f32(bias[c0 + c]) : 0.0f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      acc = __builtin_fmaf(to_f32(weight[(long)(c0 + c) * K + j]), st[j], acc);
+      store_dyn(state, base + j, state_dtype, st[j]);
+    }
+    out[c] = from_f32<T>(silu(acc) * to_f32(x2[c]));
+  }
+  *reinterpret_cast<vec_t*>(y + b * y_sb + c0) = out;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+template <typename T>
+int launch_gated_conv_prefill(const void* u, const void* weight, const void* bias, void* y, void* state,
+                              int64_t B, int64_t L, int64_t D, int K, int64_t u_sb, int64_t u_sl,
+                              int64_t y_sb, int64_t y_sl, int state_dtype, hipStream_t stream) {
+  constexpr int N = Vec16<T>::kN;
+  dim3 grid((unsigned)((D / N + 255) / 256), (unsigned)((L + kConvTokens - 1) / kConvTokens), (unsigned)B), block(256);
+#define BASED_CONV_CASE(KK)                                                                               \
+  case KK:                                                                                                \
+    hipLaunchKernelGGL((gated_conv_prefill_kernel<T, KK>), grid, block, 0, stream, (const T*)u,            \
+                       (const T*)weight, (const T*)bias, (T*)y, state, (int)L, (int)D, u_sb, u_sl, y_sb,   \
+                       y_sl, state_dtype);                                                                \
+    break;
+  switch (K) {
+    BASED_CONV_CASE(2)
+    BASED_CONV_CASE(3)
+    BASED_CONV_CASE(4)
+  }
+#undef BASED_CONV_CASE
+  return check_launch("gated_conv_prefill");
+}
+
+template <typename T>
+int launch_gated_conv_step(const void* u, void* state, const void* weight, const void* bias, void* y,
+                           int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb, int state_dtype,
+                           hipStream_t stream) {
+  constexpr int N = Vec16<T>::kN;
+  const int64_t items = B * (D / N);
+  dim3 grid((unsigned)((items + 255) / 256)), block(256);
+#define BASED_CONV_CASE(KK)                                                                             \
+  case KK:                                                                                              \
+    hipLaunchKernelGGL((gated_conv_step_kernel<T, KK>), grid, block, 0, stream, (const T*)u, state,      \
+                       (const T*)weight, (const T*)bias, (T*)y, (int)B, (int)D, u_sb, y_sb, state_dtype); \
+    break;
+  switch (K) {
+    BASED_CONV_CASE(2)
+    BASED_CONV_CASE(3)
+    BASED_CONV_CASE(4)
+  }
+#undef BASED_CONV_CASE
+  return check_launch("gated_conv_step");
+}
+
+}  // namespace based
+
+extern "C" BASED_API int based_gated_conv_prefill(const void* u, const void* weight, const void* bias, void* y,
+                                                  void* state, int64_t B, int64_t L, int64_t D, int K,
+                                                  int64_t u_sb, int64_t u_sl, int64_t y_sb, int64_t y_sl,
+                                                  int io_dtype, int state_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(u && weight && y, BASED_ERR_ARG, "gated_conv_prefill: null pointer argument");
+  BASED_REQUIRE(B >= 0 && L >= 0 && D > 0, BASED_ERR_ARG, "gated_conv_prefill: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_prefill: bad io dtype");
+  BASED_REQUIRE(state == nullptr || state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE,
+                "gated_conv_prefill: bad state dtype");
+  BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "gated_conv_prefill: kernel size %d unsupported (2..4)", K);
+  const int n = io_dtype == BASED_BF16 ? 8 : 4;
+  BASED_REQUIRE(D % n == 0, BASED_ERR_SHAPE, "gated_conv_prefill: channel count must be a multiple of %d", n);
+  BASED_REQUIRE(u_sb % n == 0 && u_sl % n == 0 && y_sb % n == 0 && y_sl % n == 0, BASED_ERR_ALIGN,
+                "gated_conv_prefill: strides must be multiples of %d elements", n);
+  BASED_REQUIRE(aligned16(u) && aligned16(y), BASED_ERR_ALIGN, "gated_conv_prefill: tensors must be 16-byte aligned");
+  BASED_REQUIRE(B < 65536 && (L + kConvTokens - 1) / kConvTokens < 65536, BASED_ERR_SHAPE,
+                "gated_conv_prefill: grid too large");
+  if (B == 0 || L == 0) return BASED_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return io_dtype == BASED_BF16
+             ? launch_gated_conv_prefill<__bf16>(u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl, state_dtype, s)
+             : launch_gated_conv_prefill<float>(u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl, state_dtype, s);
+}
+
+extern "C" BASED_API int based_gated_conv_step(const void* u, void* state, const void* weight, const void* bias,
+                                               void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
+                                               int io_dtype, int state_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(u && state && weight && y, BASED_ERR_ARG, "gated_conv_step: null pointer argument");
+  BASED_REQUIRE(B >= 0 && D > 0, BASED_ERR_ARG, "gated_conv_step: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_step: bad io dtype");
+  BASED_REQUIRE(state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_step: bad state dtype");
+  BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "gated_conv_step: kernel size %d unsupported (2..4)", K);
+  const int n = io_dtype == BASED_BF16 ? 8 : 4;
+  BASED_REQUIRE(D % n == 0, BASED_ERR_SHAPE, "gated_conv_step: channel count must be a multiple of %d", n);
+  BASED_REQUIRE(u_sb % n == 0 && y_sb % n == 0, BASED_ERR_ALIGN, "gated_conv_step: strides must be multiples of %d elements", n);
+  BASED_REQUIRE(aligned16(u) && aligned16(y), BASED_ERR_ALIGN, "gated_conv_step: tensors must be 16-byte aligned");
+  BASED_REQUIRE(B * (D / n) < (1ll << 39), BASED_ERR_SHAPE, "gated_conv_step: grid too large");
+  if (B == 0) return BASED_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return io_dtype == BASED_BF16 ? launch_gated_conv_step<__bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, state_dtype, s)
+                                : launch_gated_conv_step<float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, state_dtype, s);
+}

@@ -1,7 +1,8 @@
-"""Gated short convolution mixer (plain PyTorch).  Filler so that the 27-layer Based stack can
-be assembled around the HIP mixers; mirrors based/models/mixers/convolution.py:16-218
-(non-CUDA branch): depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a
-rolling (B, D, K) state for decoding."""
+"""Gated short convolution mixer; mirrors based/models/mixers/convolution.py:16-218 (non-CUDA
+branch): depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a rolling (B, D, K)
+state for decoding.  On a HIP device everything between the two projections is one kernel
+(`ops.gated_conv_prefill` / `ops.gated_conv_step`); host tensors take the literal torch
+statement of the same arithmetic, which is what the module-level CPU tests exercise."""
 from __future__ import annotations
 
 import torch
@@ -81,9 +82,25 @@ class BaseConv(nn.Module):
 
     def forward(self, u, position_ids=None, inference_params=None, *args, **kwargs):
         u = self.in_proj(u)
+        if u.is_cuda:
+            return self.out_proj(self._gated_conv_hip(u, inference_params))
         u1, u2 = torch.split(u, self.d_inner, dim=-1)
         u_conv = F.silu(self.conv(u1, inference_params=inference_params))
         return self.out_proj(u_conv * u2)
+
+    def _gated_conv_hip(self, u, inference_params):
+        """silu(conv(u1)) * u2 and the state handling of ShortConvolution.forward/step in one launch."""
+        from .. import ops
+
+        weight, bias = self.conv.conv.weight, self.conv.conv.bias
+        if inference_params is None:
+            return ops.gated_conv_prefill(u, weight, bias)
+        if inference_params.seqlen_offset > 0:
+            state = self.conv._get_state(inference_params)
+            return ops.gated_conv_step(u, state[: u.shape[0]], weight, bias)
+        self.conv._init_state(inference_params)
+        state = self.conv._get_state(inference_params)
+        return ops.gated_conv_prefill(u, weight, bias, state=state[: u.shape[0]])
 
     def allocate_inference_cache(self, batch_size: int, max_seqlen: int, dtype=None, **kwargs):
         return {"conv": self.conv.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)}

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Based sequence-mixer hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|copy]
 
 Headline workload (`value`): the recurrent decode step of Taylor linear attention at
 B=128, H=16, dv=64 — fp32 kv_state (128,16,1,64,273) + k_state, initialised from a seeded
@@ -153,6 +153,26 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256):
     }
 
 
+def bench_conv(torch, ops, steps, warmup, B=4, L=2048, D=2048, K=3, decode_B=128):
+    """Gated short convolution at the shape of the 27-layer configuration (d_inner = 2048)."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(2)
+    u = torch.randn(B, L, 2 * D, generator=g).bfloat16().to(dev)
+    w = (torch.randn(D, 1, K, generator=g) * 0.5).bfloat16().to(dev)
+    ms, _ = _events_ms(torch, lambda: ops.gated_conv_prefill(u, w), steps, warmup)
+    byts = B * L * D * 3 * 2
+    state = torch.zeros(decode_B, D, K, dtype=torch.bfloat16, device=dev)
+    u1 = torch.randn(decode_B, 1, 2 * D, generator=g).bfloat16().to(dev)
+    dms, _ = _events_ms(torch, lambda: ops.gated_conv_step(u1, state, w), 64, 8)
+    return {
+        "prefill_tok_s": B * L / (ms * 1e-3), "prefill_ms": ms, "B": B, "L": L, "D": D, "K": K,
+        "decode_tok_s": decode_B / (dms * 1e-3), "decode_us": dms * 1e3, "decode_B": decode_B,
+        "roofline": {"kernel": "gated_conv_prefill_kernel", "bound": "hbm", "achieved": round(byts / (ms * 1e-3) / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes_per_launch": byts},
+    }
+
+
 def cpu_baseline_decode(torch, B=128, H=16, dv=64, sample_steps=8):
     """The oracle's recurrent step on the host: `sample_steps` of the 256 steps at full batch."""
     from oracle import based_oracle as O
@@ -225,7 +245,7 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["decode", "prefill", "swa", "copy"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "copy"], default=None,
                     help="one workload only; 'copy' is a plain 256 MiB device copy used to calibrate the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     ap.add_argument("--prefill-batches", default="1,8,48,96",
@@ -269,6 +289,13 @@ def main():
     if args.only in (None, "swa"):
         s = bench_swa(torch, ops, 20, 3)
         out["swa"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in s.items()}
+    if args.only in (None, "conv"):
+        c = bench_conv(torch, ops, 20, 3)
+        out["conv"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in c.items()}
+    if args.only == "conv":
+        out.update({"value": round(out["conv"]["prefill_tok_s"], 1), "ms_per_step": out["conv"]["prefill_ms"], "dtype": "bf16",
+                    "config": {"workload": "gated short convolution prefill B=4 L=2048 D=2048 K=3"},
+                    "roofline": out["conv"]["roofline"]})
     if args.only == "prefill":
         p = out["prefill"][-1]
         out.update({"value": round(p["tok_s"], 1), "ms_per_step": p["ms"], "dtype": "bf16",

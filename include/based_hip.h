@@ -162,6 +162,40 @@ BASED_API int based_swa_step(const void* q, const void* k_new, const void* v_new
                    int64_t c_sb, int64_t c_st, int64_t c_sh,
                    int w_left, float scale, int io_dtype, void* stream);
 
+/*
+ * Gated short convolution of the Based stack (the mixer of 17 of the 27 layers of the 360m
+ * configuration), prefill form.  Replaces, in based/models/mixers/convolution.py, the body of
+ * BaseConv.forward between the two projections (:201-208: split, ShortConvolution.forward
+ * :47-86 = depthwise causal nn.Conv1d with padding K-1 truncated to L, SiLU, gate) and the state
+ * initialisation of ShortConvolution.forward (:62-68).
+ *
+ *   u      : (B, L, 2D): u1 = u[..., :D] is convolved, u2 = u[..., D:] gates; element (b,l,c) at
+ *            u[b*u_sb + l*u_sl + c]
+ *   weight : (D, 1, K) contiguous, same dtype as u (the nn.Conv1d weight); K in 2..4
+ *   bias   : (D) or NULL (the conv bias)
+ *   y      : (B, L, D), y = silu(conv(u1) + bias) * u2; element (b,l,c) at y[b*y_sb + l*y_sl + c]
+ *   state  : NULL, or (B, D, K) contiguous of dtype state_dtype, overwritten with the last K
+ *            inputs u1 of every channel, oldest first, zero-filled on the left when L < K
+ * D must be a multiple of 8 (bf16) / 4 (fp32); strides likewise; u, y 16-byte aligned.
+ */
+BASED_API int based_gated_conv_prefill(const void* u, const void* weight, const void* bias, void* y,
+                             void* state, int64_t B, int64_t L, int64_t D, int K,
+                             int64_t u_sb, int64_t u_sl, int64_t y_sb, int64_t y_sl,
+                             int io_dtype, int state_dtype, void* stream);
+
+/*
+ * Single-token form on the rolling state.  Replaces ShortConvolution.step
+ * (convolution.py:104-108: roll the (B, D, K) state left by one, append the input, contract with
+ * the conv weight) together with BaseConv.forward's SiLU and gate (:204-207).
+ *
+ *   u     : (B, 2D) rows at u[b*u_sb + c]     y : (B, D) rows at y[b*y_sb + c]
+ *   state : (B, D, K) contiguous, updated in place
+ *   bias  : (D) or NULL
+ */
+BASED_API int based_gated_conv_step(const void* u, void* state, const void* weight, const void* bias,
+                          void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
+                          int io_dtype, int state_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,8 @@ tests/test_oracle.py):
   sliding_window_step     decode == prefill invariant                     -> pinned (same caveat)
   rms_norm / swiglu_mlp / short_conv(_step)
                           closed forms + F.conv1d + step == parallel      -> pinned
+  gated_short_conv(_step) F.conv1d(groups=D, padding=K-1)[..., :L] + F.silu, per-element
+                          brute force, step == parallel                   -> pinned
 """
 from __future__ import annotations
 
@@ -207,3 +209,24 @@ def short_conv_step(x, state, weight):
     state.copy_(torch.roll(state, shifts=-1, dims=-1))
     state[:, :, -1] = x[:, 0]
     return torch.einsum("bck,ck->bc", state, weight).to(x.dtype).unsqueeze(1)
+
+
+def gated_short_conv(u, weight, bias=None):
+    """BaseConv between its projections (convolution.py:201-208, non-CUDA branch): split
+    u (B, L, 2D) into u1 | u2, y = silu(short_conv(u1) + bias) * u2.  weight: (D, K)."""
+    D = u.shape[-1] // 2
+    u1, u2 = u[..., :D].float(), u[..., D:].float()
+    c = short_conv(u1, weight.float())
+    if bias is not None:
+        c = c + bias.float()
+    return (F.silu(c) * u2).to(u.dtype)
+
+
+def gated_short_conv_step(u, state, weight, bias=None):
+    """Single-token form (convolution.py:104-108 + :204-207): roll the (B, D, K) state, append
+    u1, contract with the weight, SiLU, gate.  u: (B, 1, 2D).  The state is updated in place."""
+    D = u.shape[-1] // 2
+    c = short_conv_step(u[..., :D].float(), state, weight.float())
+    if bias is not None:
+        c = c + bias.float()
+    return (F.silu(c.float()) * u[..., D:].float()).to(u.dtype)

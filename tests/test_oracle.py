@@ -230,3 +230,32 @@ def test_rms_norm_swiglu_conv():
     for t in range(5):
         y = O.short_conv_step(x[:, t:t + 1], state, cw)
         assert torch.allclose(y, ref[:, t:t + 1], atol=1e-6)
+
+
+def test_gated_short_conv_against_library_and_brute_force():
+    """Gated short convolution: F.conv1d(groups=D, padding=K-1) truncated to L (the module form
+    the reference uses), F.silu, per-element brute force on a tiny case, and step == parallel."""
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(5)
+    B, L, D, K = 2, 11, 6, 3
+    u = torch.randn(B, L, 2 * D, generator=g)
+    w = torch.randn(D, K, generator=g)
+    bias = torch.randn(D, generator=g)
+    for b_ in (None, bias):
+        y = O.gated_short_conv(u, w, b_)
+        conv = F.conv1d(u[..., :D].transpose(1, 2), w[:, None, :], bias=b_, groups=D, padding=K - 1)[..., :L].transpose(1, 2)
+        assert torch.allclose(y, F.silu(conv) * u[..., D:], atol=1e-6)
+    # brute force: y[b,l,c] = silu(sum_j w[c,j] u1[b,l-K+1+j,c]) * u2[b,l,c]
+    y = O.gated_short_conv(u, w)
+    for (b, l, c) in [(0, 0, 0), (1, 1, 3), (0, 7, 5), (1, 10, 2)]:
+        acc = sum(float(w[c, j]) * float(u[b, l - K + 1 + j, c]) for j in range(K) if l - K + 1 + j >= 0)
+        ref = acc / (1 + math.exp(-acc)) * float(u[b, l, D + c])
+        assert abs(float(y[b, l, c]) - ref) < 1e-5
+    # step == parallel: prefix through the parallel form leaves the state, then single tokens
+    P = 7
+    state = torch.zeros(B, D, K)
+    state[..., -min(K, P):] = u[:, P - min(K, P):P, :D].transpose(1, 2)
+    for t in range(P, L):
+        yt = O.gated_short_conv_step(u[:, t:t + 1], state, w, bias)
+        assert torch.allclose(yt[:, 0], O.gated_short_conv(u, w, bias)[:, t], atol=1e-5)
