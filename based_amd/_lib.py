@@ -41,7 +41,8 @@ SIGNATURES = {
     ),
     "based_swa_prefill": (
         C.c_int,
-        [_P, _P, _P, _P] + [_I64] * 3 + [_I64] * 12 + [C.c_int, C.c_float, C.c_int, _P],
+        [_P, _P, _P, _P] + [_I64] * 3 + [_I64] * 12 + [C.c_int, C.c_float]
+        + [_P, _P, _I64] + [_P, _P] + [_I64] * 4 + [C.c_int, _P],
     ),
     "based_gated_conv_prefill": (
         C.c_int,
@@ -54,7 +55,7 @@ SIGNATURES = {
     "based_swa_step": (
         C.c_int,
         [_P, _P, _P, _P, _P, _P, _P, _I64] + [_I64] * 3 + [_I64] * 8 + [_I64] * 3
-        + [C.c_int, C.c_float, C.c_int, _P],
+        + [C.c_int, C.c_float] + [_P, _P, _I64] + [C.c_int, _P],
     ),
 }
 

@@ -30,16 +30,55 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
+// bf16 pair (x1 at channel c < 32, x2 at channel c + 32) -> rotated pair, rounded to bf16
+__device__ __forceinline__ void rope_rotate8(u32x4& lo, u32x4& hi, const f32x4 (&cs)[2], const f32x4 (&sn)[2]) {
+  u32x4 out_lo, out_hi;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    float o1[2], o2[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const int j = 2 * d + e;
+      const float x1 = bf16_bits_to_f32(e == 0 ? (lo[d] & 0xFFFFu) : (lo[d] >> 16));
+      const float x2 = bf16_bits_to_f32(e == 0 ? (hi[d] & 0xFFFFu) : (hi[d] >> 16));
+      const float c = cs[j >> 2][j & 3], sgn = sn[j >> 2][j & 3];
+      o1[e] = x1 * c - x2 * sgn;
+      o2[e] = x1 * sgn + x2 * c;
+    }
+    out_lo[d] = pack_bf16(o1[0], o1[1]);
+    out_hi[d] = pack_bf16(o2[0], o2[1]);
+  }
+  lo = out_lo;
+  hi = out_hi;
+}
+
+// One tile's worth of rows on their way from global memory to LDS (register prefetch).
+template <bool ROPE> struct SwaRows {
+  u32x4 kp[2], vp[2];
+};
+template <> struct SwaRows<true> {
+  u32x4 kp[2], vp[2], qp[2];
+  f32x4 cs[2], sn[2];
+};
+
+// ROPE: q and k are rotated on their way into LDS (non-interleaved rotary over the whole head,
+// cos/sin tables of 32 frequencies per position), as flash-attn's rotary layer does before the
+// attention of the reference (slide_attention.py:346-355,553-556).
+// kc_out / vc_out (optional): the (rotated) K rows and the V rows of this call are also written
+// to a KV cache, the job of _update_kv_cache (slide_attention.py:255-281).
+template <bool ROPE>
 __global__ __launch_bounds__(256) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
-    int w_left, float scale_log2e) {
+    int w_left, float scale_log2e, const float* __restrict__ rope_cos, const float* __restrict__ rope_sin,
+    __bf16* __restrict__ kc_out, __bf16* __restrict__ vc_out, long c_sb, long c_st, long c_sh) {
   // Two blocks of 64 K rows and 64 V rows: one holds the current tile's own keys, the other the
   // 64 keys to its left.  Moving on by one tile, "own" becomes "left" without a copy and the
   // old left block takes the next tile's rows.
   __shared__ __align__(16) __bf16 s_k[2 * kQTile * kKStride];
   __shared__ __align__(16) __bf16 s_v[2 * kQTile * kVStride];
+  __shared__ __align__(16) __bf16 s_q[ROPE ? kQTile * kKStride : 8];  // rotated queries (ROPE only)
   static_assert(kOStride == kKStride, "output staging reuses whole K rows of the left block");
 
   const int tid = threadIdx.x;
@@ -60,33 +99,68 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
   k += b * k_sb + h * k_sh;
   v += b * v_sb + h * v_sh;
   o += b * o_sb + h * o_sh;
+  if (kc_out != nullptr) {
+    kc_out += b * c_sb + h * c_sh;
+    vc_out += b * c_sb + h * c_sh;
+  }
 
-  // Rows of a 64-row block moved by this thread: 16 wave + 8 i + lane / 8 (i = 0, 1), 16 bytes at
-  // channel 8 (lane % 8).  A wavefront only ever writes block rows 16 wave .. 16 wave + 15,
-  // the rows that double as its output staging tile.
-  const int my_row = 16 * wave + (lane >> 3);
-  const int my_seg = 8 * (lane & 7);
-  auto load_rows = [&](int key0, u32x4 (&kp)[2], u32x4 (&vp)[2]) {
+  // Pieces (row of a 64-row block, first channel) moved by this thread, 16 bytes each.  A
+  // wavefront only ever writes block rows 16 wave .. 16 wave + 15, the rows that double as its
+  // output staging tile.  Plain: rows 16 wave + 8 i + lane / 8, channels 8 (lane % 8).
+  // ROPE: one row, 16 wave + lane / 4, and the two channel groups 8 (lane % 4) + 32 i that the
+  // rotation pairs up.
+  auto piece_row = [&](int i) { return ROPE ? 16 * wave + (lane >> 2) : 16 * wave + 8 * i + (lane >> 3); };
+  auto piece_ch = [&](int i) { return ROPE ? 8 * (lane & 3) + 32 * i : 8 * (lane & 7); };
+  auto load_rows = [&](int key0, SwaRows<ROPE>& r, bool with_q) {
+    const u32x4 z4 = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int key = key0 + my_row + 8 * i;
-      const u32x4 z4 = {0, 0, 0, 0};
-      kp[i] = vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
+      const int key = key0 + piece_row(i);
+      r.kp[i] = r.vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
+      if constexpr (ROPE) r.qp[i] = z4;
       if (key >= 0 && key < L) {
-        kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + my_seg);
-        vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + my_seg);
+        r.kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + piece_ch(i));
+        r.vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + piece_ch(i));
+        if constexpr (ROPE)
+          if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q + (long)key * q_sl + piece_ch(i));
+      }
+    }
+    if constexpr (ROPE) {
+      const int key = key0 + piece_row(0);
+      const f32x4 one4 = {1.f, 1.f, 1.f, 1.f}, zero4 = {0.f, 0.f, 0.f, 0.f};
+      r.cs[0] = r.cs[1] = one4;
+      r.sn[0] = r.sn[1] = zero4;
+      if (key >= 0 && key < L) {
+        const f32x4* c4 = reinterpret_cast<const f32x4*>(rope_cos + (long)key * (kHeadDim / 2) + 8 * (lane & 3));
+        const f32x4* s4 = reinterpret_cast<const f32x4*>(rope_sin + (long)key * (kHeadDim / 2) + 8 * (lane & 3));
+        r.cs[0] = c4[0];
+        r.cs[1] = c4[1];
+        r.sn[0] = s4[0];
+        r.sn[1] = s4[1];
       }
     }
   };
-  auto store_rows = [&](int blk, const u32x4 (&kp)[2], const u32x4 (&vp)[2]) {
+  // own_rows: the rows are the tile's own keys (they also carry its queries and go to the cache)
+  auto store_rows = [&](int blk, int key0, SwaRows<ROPE>& r, bool own_rows) {
+    if constexpr (ROPE) {
+      rope_rotate8(r.kp[0], r.kp[1], r.cs, r.sn);
+      if (own_rows) rope_rotate8(r.qp[0], r.qp[1], r.cs, r.sn);
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int row = blk * kQTile + my_row + 8 * i;
-      *reinterpret_cast<u32x4*>(s_k + row * kKStride + my_seg) = kp[i];
-      *reinterpret_cast<u32x4*>(s_v + row * kVStride + my_seg) = vp[i];
+      const int row = blk * kQTile + piece_row(i);
+      *reinterpret_cast<u32x4*>(s_k + row * kKStride + piece_ch(i)) = r.kp[i];
+      *reinterpret_cast<u32x4*>(s_v + row * kVStride + piece_ch(i)) = r.vp[i];
+      if constexpr (ROPE)
+        if (own_rows) *reinterpret_cast<u32x4*>(s_q + piece_row(i) * kKStride + piece_ch(i)) = r.qp[i];
+      const int key = key0 + piece_row(i);
+      if (own_rows && kc_out != nullptr && key < L) {
+        *reinterpret_cast<u32x4*>(kc_out + (long)key * c_st + piece_ch(i)) = r.kp[i];
+        *reinterpret_cast<u32x4*>(vc_out + (long)key * c_st + piece_ch(i)) = r.vp[i];
+      }
     }
   };
-  // Q operand of this wavefront's 16 queries, straight from global memory
+  // Q operand of this wavefront's 16 queries, straight from global memory (plain variant)
   auto load_q = [&](int q0, bf16x8 (&bq)[2]) {
     const int n = q0 + 16 * wave + col;
 #pragma unroll
@@ -98,20 +172,20 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
   };
 
   int q0 = tile_begin * kQTile;
-  u32x4 kp[2], vp[2];
+  SwaRows<ROPE> pre;
   bf16x8 bq[2], bq_next[2];
   {
     // first tile: own rows in block 0, the 64 keys to the left in block 1 (one round trip)
-    u32x4 kl[2], vl[2];
-    load_rows(q0 - kQTile, kl, vl);
-    load_rows(q0, kp, vp);
-    load_q(q0, bq);
-    store_rows(1, kl, vl);
-    store_rows(0, kp, vp);
+    SwaRows<ROPE> left;
+    load_rows(q0 - kQTile, left, false);
+    load_rows(q0, pre, true);
+    if constexpr (!ROPE) load_q(q0, bq);
+    store_rows(1, q0 - kQTile, left, false);
+    store_rows(0, q0, pre, true);
   }
   if (tile_begin + 1 < tile_end) {  // the next tile's rows travel while this one is computed
-    load_rows(q0 + kQTile, kp, vp);
-    load_q(q0 + kQTile, bq_next);
+    load_rows(q0 + kQTile, pre, true);
+    if constexpr (!ROPE) load_q(q0 + kQTile, bq_next);
   }
 
   for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile) {
@@ -121,6 +195,11 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
     // staged key index x (0..127 <-> key q0 - 64 + x) -> row of the ring
     auto ring_row = [&](int x) { return ((x < kQTile ? 1 - own : own) * kQTile) + (x & (kQTile - 1)); };
     __syncthreads();  // the staged rows are visible
+    if constexpr (ROPE) {
+#pragma unroll
+      for (int ds = 0; ds < 2; ++ds)
+        bq[ds] = *reinterpret_cast<const bf16x8*>(s_q + (16 * wave + col) * kKStride + 32 * ds + 8 * grp);
+    }
 
     // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
     // wavefront w sees staged keys 16 w .. 16 w + 79 (tile i = keys 16 w + 16 i ..)
@@ -215,12 +294,14 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
 
     // ---- the left block takes the next tile's rows (this wavefront's own 16 rows of it) ----
     if (tile + 1 < tile_end) {
-      store_rows(1 - own, kp, vp);
-      bq[0] = bq_next[0];
-      bq[1] = bq_next[1];
+      store_rows(1 - own, q0 + kQTile, pre, true);
+      if constexpr (!ROPE) {
+        bq[0] = bq_next[0];
+        bq[1] = bq_next[1];
+      }
       if (tile + 2 < tile_end) {
-        load_rows(q0 + 2 * kQTile, kp, vp);
-        load_q(q0 + 2 * kQTile, bq_next);
+        load_rows(q0 + 2 * kQTile, pre, true);
+        if constexpr (!ROPE) load_q(q0 + 2 * kQTile, bq_next);
       }
     }
   }
@@ -236,9 +317,11 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
     __bf16* __restrict__ kcache, __bf16* __restrict__ vcache, __bf16* __restrict__ o,
     const int32_t* __restrict__ cache_seqlens, int pos_host, int H, int max_seqlen, long q_sb,
     long q_sh, long kn_sb, long kn_sh, long vn_sb, long vn_sh, long o_sb, long o_sh, long c_sb,
-    long c_st, long c_sh, int w_left, float scale_log2e) {
+    long c_st, long c_sh, int w_left, float scale_log2e, const float* __restrict__ rope_cos,
+    const float* __restrict__ rope_sin, int rope_len) {
   __shared__ float s_p[80];          // scores, then weights; entry 64 is the new token
   __shared__ float s_part[4][kHeadDim];
+  __shared__ __align__(16) float s_qrot[4][kHeadDim];  // rotated query, one private copy per wavefront
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -247,6 +330,7 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
   int pos = cache_seqlens ? cache_seqlens[b] : pos_host;
   pos = __builtin_amdgcn_readfirstlane(pos);
   if (pos < 0 || pos >= max_seqlen) return;  // out-of-range position: nothing to attend or write
+  if (rope_cos != nullptr && pos >= rope_len) return;
 
   __bf16* kc = kcache + b * c_sb + h * c_sh;
   __bf16* vc = vcache + b * c_sb + h * c_sh;
@@ -263,15 +347,46 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
   }
   const bf16x8* qrow = reinterpret_cast<const bf16x8*>(q + b * q_sb + h * q_sh + 16 * kq4);
   const bf16x8 qx[2] = {qrow[0], qrow[1]};
+  float cs = 1.0f, sn = 0.0f;  // rotary factors of channel `lane` at this position
+  if (rope_cos != nullptr) {
+    cs = rope_cos[(long)pos * (kHeadDim / 2) + (lane & 31)];
+    sn = rope_sin[(long)pos * (kHeadDim / 2) + (lane & 31)];
+  }
   float vv[17];
 #pragma unroll
   for (int u = 0; u < 17; ++u) {
     const int j = 4 * u + wave;  // keys of this wavefront: j = wave, wave + 4, ...
     vv[u] = j < ncached ? to_f32(vc[(long)(lo + j) * c_st + lane]) : 0.f;
   }
-  const float kn = to_f32(k_new[b * kn_sb + h * kn_sh + lane]);
+  float kn = to_f32(k_new[b * kn_sb + h * kn_sh + lane]);
   const float vn = to_f32(v_new[b * vn_sb + h * vn_sh + lane]);
-  const float ql = to_f32(q[b * q_sb + h * q_sh + lane]);
+  float ql = to_f32(q[b * q_sb + h * q_sh + lane]);
+  // this wavefront's slice of the query for the scores: 16 channels from 16 kq4
+  float qf[16];
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[8 * c + i] = to_f32(qx[c][i]);
+  if (rope_cos != nullptr) {
+    // Non-interleaved rotary over the whole head: channel c pairs with c +- 32,
+    //   out[c] = x[c] cos - x[c+32] sin (c < 32),  out[c] = x[c] cos + x[c-32] sin (c >= 32),
+    // rounded to bf16 like the rotated tensors of the prefill.  Every wavefront rotates the
+    // query for itself (lane <-> channel) and hands the slices round through its own LDS row.
+    const float sgn = lane < 32 ? -1.0f : 1.0f;
+    ql = to_f32((__bf16)__builtin_fmaf(ql, cs, sgn * __shfl_xor(ql, 32, 64) * sn));
+    kn = to_f32((__bf16)__builtin_fmaf(kn, cs, sgn * __shfl_xor(kn, 32, 64) * sn));
+    s_qrot[wave][lane] = ql;
+    __builtin_amdgcn_wave_barrier();
+    const f32x4* src = reinterpret_cast<const f32x4*>(&s_qrot[wave][16 * kq4]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const f32x4 x = src[i];
+      qf[4 * i + 0] = x[0];
+      qf[4 * i + 1] = x[1];
+      qf[4 * i + 2] = x[2];
+      qf[4 * i + 3] = x[3];
+    }
+  }
   if (wave == 0) {  // the new token joins the cache (row pos)
     kc[(long)pos * c_st + lane] = (__bf16)kn;
     vc[(long)pos * c_st + lane] = (__bf16)vn;
@@ -282,7 +397,7 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
 #pragma unroll
   for (int c = 0; c < 2; ++c)
 #pragma unroll
-    for (int i = 0; i < 8; ++i) part = __builtin_fmaf(to_f32(kx[c][i]), to_f32(qx[c][i]), part);
+    for (int i = 0; i < 8; ++i) part = __builtin_fmaf(to_f32(kx[c][i]), qf[8 * c + i], part);
   part += __shfl_xor(part, 1, 64);
   part += __shfl_xor(part, 2, 64);
   if (kq4 == 0) s_p[kj] = kj < ncached ? part * scale_log2e : -INFINITY;
@@ -328,9 +443,28 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
                                            int64_t k_sb, int64_t k_sl, int64_t k_sh,
                                            int64_t v_sb, int64_t v_sl, int64_t v_sh,
                                            int64_t o_sb, int64_t o_sl, int64_t o_sh,
-                                           int w_left, float scale, int io_dtype, void* stream) {
+                                           int w_left, float scale,
+                                           const float* rope_cos, const float* rope_sin, int64_t rope_len,
+                                           void* kcache_out, void* vcache_out,
+                                           int64_t c_sb, int64_t c_st, int64_t c_sh, int64_t max_seqlen,
+                                           int io_dtype, void* stream) {
   using namespace based;
   BASED_REQUIRE(q && k && v && o, BASED_ERR_ARG, "swa_prefill: null pointer argument");
+  BASED_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), BASED_ERR_ARG,
+                "swa_prefill: rotary tables must be given together");
+  if (rope_cos)
+    BASED_REQUIRE(rope_len >= L, BASED_ERR_ARG, "swa_prefill: rotary tables hold %ld positions, need %ld",
+                  (long)rope_len, (long)L);
+  BASED_REQUIRE((kcache_out == nullptr) == (vcache_out == nullptr), BASED_ERR_ARG,
+                "swa_prefill: cache outputs must be given together");
+  if (kcache_out) {
+    BASED_REQUIRE(L <= max_seqlen, BASED_ERR_SHAPE, "swa_prefill: %ld tokens do not fit a cache of %ld rows",
+                  (long)L, (long)max_seqlen);
+    BASED_REQUIRE(c_sb % 8 == 0 && c_st % 8 == 0 && c_sh % 8 == 0, BASED_ERR_ALIGN,
+                  "swa_prefill: cache strides must be multiples of 8 elements");
+    BASED_REQUIRE(aligned16(kcache_out) && aligned16(vcache_out), BASED_ERR_ALIGN,
+                  "swa_prefill: caches must be 16-byte aligned");
+  }
   BASED_REQUIRE(B >= 0 && H > 0 && L >= 0, BASED_ERR_ARG, "swa_prefill: bad sizes");
   BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_prefill: only bf16 is supported");
   BASED_REQUIRE(w_left >= 0 && w_left <= 64, BASED_ERR_SHAPE,
@@ -352,10 +486,12 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
   const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
   dim3 grid((unsigned)(B * H * runs_per_seq)), block(256);
-  hipLaunchKernelGGL(swa_prefill_kernel, grid, block, 0, static_cast<hipStream_t>(stream),
+  auto kern = rope_cos ? swa_prefill_kernel<true> : swa_prefill_kernel<false>;
+  hipLaunchKernelGGL(kern, grid, block, 0, static_cast<hipStream_t>(stream),
                      (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o, (int)H, (int)L,
-                     (int)n_tiles, (int)run_tiles, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh,
-                     w_left, scale * 1.4426950408889634f);
+                     (int)n_tiles, (int)run_tiles, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb,
+                     o_sl, o_sh, w_left, scale * 1.4426950408889634f, rope_cos, rope_sin,
+                     (__bf16*)kcache_out, (__bf16*)vcache_out, c_sb, c_st, c_sh);
   return check_launch("swa_prefill");
 }
 
@@ -366,10 +502,20 @@ extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const 
                                         int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
                                         int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
                                         int64_t c_sb, int64_t c_st, int64_t c_sh,
-                                        int w_left, float scale, int io_dtype, void* stream) {
+                                        int w_left, float scale,
+                                        const float* rope_cos, const float* rope_sin, int64_t rope_len,
+                                        int io_dtype, void* stream) {
   using namespace based;
   BASED_REQUIRE(q && k_new && v_new && kcache && vcache && o, BASED_ERR_ARG,
                 "swa_step: null pointer argument");
+  BASED_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), BASED_ERR_ARG,
+                "swa_step: rotary tables must be given together");
+  if (rope_cos) {
+    BASED_REQUIRE(rope_len > 0 && rope_len < (1ll << 31), BASED_ERR_ARG, "swa_step: bad rotary table length");
+    if (!cache_seqlens)
+      BASED_REQUIRE(pos_host < rope_len, BASED_ERR_ARG, "swa_step: position %ld beyond the rotary table (%ld rows)",
+                    (long)pos_host, (long)rope_len);
+  }
   BASED_REQUIRE(B >= 0 && H > 0 && max_seqlen > 0, BASED_ERR_ARG, "swa_step: bad sizes");
   BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_step: only bf16 is supported");
   BASED_REQUIRE(w_left >= 0 && w_left <= 64, BASED_ERR_SHAPE,
@@ -388,6 +534,7 @@ extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const 
                      static_cast<hipStream_t>(stream), (const __bf16*)q, (const __bf16*)k_new,
                      (const __bf16*)v_new, (__bf16*)kcache, (__bf16*)vcache, (__bf16*)o, cache_seqlens,
                      (int)pos_host, (int)H, (int)max_seqlen, q_sb, q_sh, kn_sb, kn_sh, vn_sb, vn_sh,
-                     o_sb, o_sh, c_sb, c_st, c_sh, w_left, scale * 1.4426950408889634f);
+                     o_sb, o_sh, c_sb, c_st, c_sh, w_left, scale * 1.4426950408889634f, rope_cos, rope_sin,
+                     (int)rope_len);
   return check_launch("swa_step");
 }

@@ -36,6 +36,15 @@ class RotaryEmbedding(nn.Module):
         freqs = torch.outer(positions.float(), self.inv_freq.to(positions.device))
         return freqs.cos(), freqs.sin()
 
+    def tables(self, n_pos: int, device):
+        """(cos, sin) fp32 (>= n_pos, dim/2) tables for the kernels' in-flight rotation; grown on
+        demand and kept (a captured decode graph holds their addresses)."""
+        cached = getattr(self, "_tables", None)
+        if cached is None or cached[0].shape[0] < n_pos or cached[0].device != device:
+            cos, sin = self._cos_sin(torch.arange(n_pos, device=device))
+            self._tables = (cos.contiguous(), sin.contiguous())
+        return self._tables
+
     def _rotate(self, x, cos, sin):
         # x: (B, L, H, D); cos/sin: (L, dim/2)
         ro = x[..., : self.dim].float()
@@ -148,18 +157,28 @@ class SlidingAttention(nn.Module):
         if qkv.dtype != torch.bfloat16:
             qkv = qkv.to(torch.bfloat16)
         offset = 0 if inference_params is None else inference_params.seqlen_offset
+        # Rotary over the whole head, non-interleaved (the released configurations), happens inside
+        # the kernels; other rotary shapes are applied here with torch ops at host-known positions.
+        rope = None
         if self.rotary_emb_dim > 0:
-            qkv = self.rotary_emb(qkv, seqlen_offset=offset)
+            if self.rotary_emb_dim == self.head_dim and not self.rotary_emb.interleaved:
+                n_pos = seqlen if inference_params is None else max(inference_params.max_seqlen, offset + seqlen)
+                rope = self.rotary_emb.tables(n_pos, qkv.device)
+            else:
+                if inference_params is not None and inference_params.lengths_per_sample is not None:
+                    raise NotImplementedError("per-sample positions need the in-kernel rotary (full head, non-interleaved)")
+                qkv = self.rotary_emb(qkv, seqlen_offset=offset)
         q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
 
         if inference_params is None:
-            context = ops.swa_prefill(q, k, v, w_left=self.window[0], scale=self.softmax_scale)
+            context = ops.swa_prefill(q, k, v, w_left=self.window[0], scale=self.softmax_scale, rope=rope)
         elif offset == 0:
             cache = self._cache(inference_params, qkv)
             b0 = inference_params.batch_size_offset
             assert b0 + batch <= cache.shape[0] and seqlen <= cache.shape[1]
-            cache[b0:b0 + batch, :seqlen] = qkv[:, :, 1:]
-            context = ops.swa_prefill(q, k, v, w_left=self.window[0], scale=self.softmax_scale)
+            # the kernel also files the (rotated) k and the v rows in the cache
+            context = ops.swa_prefill(q, k, v, w_left=self.window[0], scale=self.softmax_scale, rope=rope,
+                                      kv_cache=cache[b0:b0 + batch])
         else:
             assert seqlen == 1, "decoding feeds one token at a time"
             cache = self._cache(inference_params, qkv)
@@ -168,6 +187,6 @@ class SlidingAttention(nn.Module):
             if inference_params.lengths_per_sample is not None:
                 pos = inference_params.lengths_per_sample[b0:b0 + batch]
             context = ops.swa_step(q, k, v, cache[b0:b0 + batch], pos, w_left=self.window[0],
-                                   scale=self.softmax_scale)
+                                   scale=self.softmax_scale, rope=rope)
         out = self.out_proj(context.reshape(batch, seqlen, self.embed_dim).to(in_dtype))
         return out if not self.return_residual else (out, x)

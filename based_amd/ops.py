@@ -66,9 +66,27 @@ def linear_attn_step(q, k, v, kv_state, k_state, eps: float = 1e-12) -> torch.Te
     return y
 
 
-def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None) -> torch.Tensor:
+def _rope_tables(rope, device, need_rows):
+    """(cos, sin) fp32 (n_pos, 32) contiguous device tables -> (cos_ptr, sin_ptr, n_pos) or Nones."""
+    if rope is None:
+        return None, None, 0
+    cos, sin = rope
+    for t in (cos, sin):
+        if (not t.is_cuda or t.device != device or t.dtype != torch.float32 or t.dim() != 2
+                or t.shape[1] != 32 or not t.is_contiguous()):
+            raise ValueError("rotary tables must be contiguous fp32 (n_pos, 32) tensors on the device of q")
+    if cos.shape != sin.shape or cos.shape[0] < need_rows:
+        raise ValueError(f"rotary tables hold {cos.shape[0]} positions, need {need_rows}")
+    return cos.data_ptr(), sin.data_ptr(), cos.shape[0]
+
+
+def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=None, kv_cache=None) -> torch.Tensor:
     """Sliding-window causal attention.  q, k, v: (B, L, H, 64) bf16 (any strides with the
-    last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i]."""
+    last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i].
+    rope: None or (cos, sin) fp32 (n_pos >= L, 32) tables; q and k are then rotated in the kernel
+    (non-interleaved rotary over the whole head, positions 0..L-1).
+    kv_cache: None or a (B, max_seqlen >= L, 2, H, 64) bf16 cache whose rows 0..L-1 receive the
+    (rotated) k and v."""
     _require_cuda(q, k, v)
     B, L, H, D = q.shape
     if D != 64 or k.shape != q.shape or v.shape != q.shape:
@@ -77,20 +95,33 @@ def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None) -> tor
         if t.stride(-1) != 1:
             raise ValueError("innermost dimension must be contiguous")
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, L)
+    kc_ptr = vc_ptr = None
+    c_strides, max_seqlen = (0, 0, 0), 0
+    if kv_cache is not None:
+        _require_cuda(q, kv_cache)
+        if (kv_cache.dim() != 5 or kv_cache.shape[0] != B or kv_cache.shape[2] != 2
+                or tuple(kv_cache.shape[3:]) != (H, D) or kv_cache.dtype != q.dtype or kv_cache.stride(-1) != 1):
+            raise ValueError(f"bad cache {tuple(kv_cache.shape)} {kv_cache.dtype}")
+        kc, vc = kv_cache[:, :, 0], kv_cache[:, :, 1]
+        kc_ptr, vc_ptr = kc.data_ptr(), vc.data_ptr()
+        c_strides, max_seqlen = (kc.stride(0), kc.stride(1), kc.stride(2)), kv_cache.shape[1]
     o = torch.empty(B, L, H, D, dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
         _lib.check(_lib.lib().based_swa_prefill(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
-            int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
+            int(w_left), scale, cos_ptr, sin_ptr, n_pos, kc_ptr, vc_ptr, *c_strides, max_seqlen,
+            _dtype_code(q), _stream_ptr(q)))
     return o
 
 
-def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None) -> torch.Tensor:
+def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None, rope=None) -> torch.Tensor:
     """Decode step.  q, k_new, v_new: (B, 1, H, 64) bf16; kv_cache (B, max_seqlen, 2, H, 64)
     bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.
-    pos: int (same for the whole batch) or an int32 device tensor of B positions."""
+    pos: int (same for the whole batch) or an int32 device tensor of B positions.
+    rope: None or (cos, sin) tables as for swa_prefill: q and k_new are rotated at `pos` first."""
     _require_cuda(q, k_new, v_new, kv_cache)
     B, one, H, D = q.shape
     if one != 1 or D != 64 or k_new.shape != q.shape or v_new.shape != q.shape:
@@ -107,8 +138,10 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
         if pos.dtype != torch.int32 or not pos.is_cuda or pos.numel() < B or not pos.is_contiguous():
             raise ValueError("cache_seqlens must be a contiguous int32 device tensor with B entries")
         seq_ptr, pos_host = pos.data_ptr(), 0
+        cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, 1)
     else:
         seq_ptr, pos_host = None, int(pos)
+        cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, pos_host + 1)
     o = torch.empty(B, 1, H, D, dtype=q.dtype, device=q.device)
     kc, vc = kv_cache[:, :, 0], kv_cache[:, :, 1]
     with torch.cuda.device(q.device):
@@ -118,7 +151,7 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
             q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
             v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
             kc.stride(0), kc.stride(1), kc.stride(2),
-            int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
+            int(w_left), scale, cos_ptr, sin_ptr, n_pos, _dtype_code(q), _stream_ptr(q)))
     return o
 
 

@@ -129,6 +129,15 @@ BASED_API int based_linear_attn_prefill_split(const void* q, const void* k, cons
  *
  * q, k, v, o : element (b,l,h,c) at p[b*sb + l*sl + h*sh + c], c < 64 contiguous.
  * head dim is 64; 0 <= w_left <= 64 (pass window_size // 2 of the module).  bf16 only.
+ *
+ * rope_cos, rope_sin : NULL, or fp32 tables (rope_len, 32) of cos / sin(position * inv_freq[i]):
+ *   q and k are rotated inside the kernel (non-interleaved rotary over the whole head:
+ *   channel c pairs with c + 32), the job of the rotary layer the reference applies to qkv
+ *   before the attention (slide_attention.py:346-355, 553-556).  Positions start at 0;
+ *   rope_len >= L.
+ * kcache_out, vcache_out : NULL, or a KV cache (element (b,t,h,c) at p[b*c_sb + t*c_st +
+ *   h*c_sh + c], max_seqlen >= L rows) that receives the (rotated) k rows and the v rows of
+ *   tokens 0..L-1: the copy _update_kv_cache makes at prefill (slide_attention.py:255-281).
  */
 BASED_API int based_swa_prefill(const void* q, const void* k, const void* v, void* o,
                       int64_t B, int64_t H, int64_t L,
@@ -136,7 +145,11 @@ BASED_API int based_swa_prefill(const void* q, const void* k, const void* v, voi
                       int64_t k_sb, int64_t k_sl, int64_t k_sh,
                       int64_t v_sb, int64_t v_sl, int64_t v_sh,
                       int64_t o_sb, int64_t o_sl, int64_t o_sh,
-                      int w_left, float scale, int io_dtype, void* stream);
+                      int w_left, float scale,
+                      const float* rope_cos, const float* rope_sin, int64_t rope_len,
+                      void* kcache_out, void* vcache_out,
+                      int64_t c_sb, int64_t c_st, int64_t c_sh, int64_t max_seqlen,
+                      int io_dtype, void* stream);
 
 /*
  * Sliding-window decode step against a linear KV cache.
@@ -152,6 +165,11 @@ BASED_API int based_swa_prefill(const void* q, const void* k, const void* v, voi
  * kcache, vcache : element (b,t,h,c) at p[b*c_sb + t*c_st + h*c_sh + c]; the reference's
  *   packed (B, max_seqlen, 2, H, 64) cache is passed as two pointers 1 plane apart.
  * q, k_new, v_new, o : element (b,h,c) at p[b*sb + h*sh + c].
+ * rope_cos, rope_sin : NULL, or the tables described at based_swa_prefill: q and k_new are
+ *   rotated at position pos before use (and the rotated k_new is what enters the cache), as
+ *   flash_attn_with_kvcache does with its rotary_cos / rotary_sin arguments
+ *   (slide_attention.py:400-427).  The position comes from the same place as the cache row,
+ *   so a captured graph needs no host-side position.
  */
 BASED_API int based_swa_step(const void* q, const void* k_new, const void* v_new,
                    void* kcache, void* vcache, void* o,
@@ -160,7 +178,9 @@ BASED_API int based_swa_step(const void* q, const void* k_new, const void* v_new
                    int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
                    int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
                    int64_t c_sb, int64_t c_st, int64_t c_sh,
-                   int w_left, float scale, int io_dtype, void* stream);
+                   int w_left, float scale,
+                   const float* rope_cos, const float* rope_sin, int64_t rope_len,
+                   int io_dtype, void* stream);
 
 /*
  * Gated short convolution of the Based stack (the mixer of 17 of the 27 layers of the 360m

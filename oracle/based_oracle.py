@@ -25,6 +25,12 @@ tests/test_oracle.py):
   sliding_window_step     decode == prefill invariant                     -> pinned (same caveat)
   rms_norm / swiglu_mlp / short_conv(_step)
                           closed forms + F.conv1d + step == parallel      -> pinned
+  rotary_embedding        position 0 == identity, norm preservation, relative-position
+                          property of the rotated dot product, complex-number brute
+                          force                                            -> pinned against
+                          the published RoPE formula (GPT-NeoX half-split layout); the
+                          reference takes it from flash-attn's rotary layer (absent), so
+                          agreement with THAT library is "parity unpinned".
   gated_short_conv(_step) F.conv1d(groups=D, padding=K-1)[..., :L] + F.silu, per-element
                           brute force, step == parallel                   -> pinned
 """
@@ -230,3 +236,18 @@ def gated_short_conv_step(u, state, weight, bias=None):
     if bias is not None:
         c = c + bias.float()
     return (F.silu(c.float()) * u[..., D:].float()).to(u.dtype)
+
+
+def rotary_embedding(x, positions, base: float = 10000.0):
+    """Rotary position embedding over the whole last dimension, non-interleaved ("half-split")
+    layout, as the reference applies to q and k of the sliding-window mixer through flash-attn's
+    RotaryEmbedding (slide_attention.py:346-355,553-556; rotary_emb_interleaved=False):
+        out[..., i]       = x[..., i] cos(p w_i) - x[..., i + D/2] sin(p w_i)
+        out[..., i + D/2] = x[..., i] sin(p w_i) + x[..., i + D/2] cos(p w_i),   w_i = base^(-2i/D).
+    x: (B, L, H, D); positions: (L,) integer tensor.  fp32 arithmetic, cast back to x.dtype."""
+    D = x.shape[-1]
+    inv_freq = 1.0 / (base ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = torch.outer(positions.float(), inv_freq)            # (L, D/2)
+    cos, sin = ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]
+    x1, x2 = x[..., : D // 2].float(), x[..., D // 2:].float()
+    return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)

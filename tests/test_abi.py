@@ -47,10 +47,10 @@ def test_argument_validation_without_gpu():
     rc = lib.based_linear_attn_step(p, p, p, p, p, p, 1, 1, 40, 0, 0, 0, 0, 0, 0, 0, 0, 1e-12, 0, None)
     assert rc == 1
     # window too wide -> BASED_ERR_SHAPE
-    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 65, 0.125, 0, None)
+    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 65, 0.125, None, None, 0, None, None, 0, 0, 0, 0, 0, None)
     assert rc == 1
     # fp32 is not a sliding-window element type -> BASED_ERR_DTYPE (2)
-    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 64, 0.125, 1, None)
+    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 64, 0.125, None, None, 0, None, None, 0, 0, 0, 0, 1, None)
     assert rc == 2
     # misaligned stride -> BASED_ERR_ALIGN (3)
     rc = lib.based_linear_attn_prefill(p, p, p, p, None, None, 1, 1, 8, 64, 0, 0, 20, 0, 0, 16, 0, 0, 64, 0, 0, 64, 1e-12, 0, None)
@@ -59,5 +59,11 @@ def test_argument_validation_without_gpu():
     rc = lib.based_linear_attn_prefill(p, p, p, p, p, None, 1, 1, 8, 64, 0, 0, 16, 0, 0, 16, 0, 0, 64, 0, 0, 64, 1e-12, 0, None)
     assert rc == 4
     # empty batch is a no-op success
-    rc = lib.based_swa_prefill(p, p, p, p, 0, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 64, 0.125, 0, None)
+    rc = lib.based_swa_prefill(p, p, p, p, 0, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 64, 0.125, None, None, 0, None, None, 0, 0, 0, 0, 0, None)
     assert rc == 0
+    # one rotary table without the other -> BASED_ERR_ARG
+    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 64, 0.125, p, None, 8, None, None, 0, 0, 0, 0, 0, None)
+    assert rc == 4
+    # gated convolution: kernel size outside 2..4 -> BASED_ERR_SHAPE
+    rc = lib.based_gated_conv_prefill(p, p, None, p, None, 1, 4, 8, 5, 64, 16, 32, 8, 0, 0, None)
+    assert rc == 1

@@ -259,3 +259,27 @@ def test_gated_short_conv_against_library_and_brute_force():
     for t in range(P, L):
         yt = O.gated_short_conv_step(u[:, t:t + 1], state, w, bias)
         assert torch.allclose(yt[:, 0], O.gated_short_conv(u, w, bias)[:, t], atol=1e-5)
+
+
+def test_rotary_embedding_properties():
+    """RoPE: identity at position 0, norm preservation, <R_m q, R_n k> depends on m - n only,
+    and a brute-force complex multiplication (x_i + i x_{i+D/2}) * exp(i p w_i)."""
+    g = torch.Generator().manual_seed(9)
+    B, L, H, D = 2, 12, 3, 64
+    x = torch.randn(B, L, H, D, generator=g)
+    y = torch.randn(B, L, H, D, generator=g)
+    pos = torch.arange(L)
+    rx = O.rotary_embedding(x, pos)
+    assert torch.allclose(rx[:, 0], x[:, 0], atol=1e-6)
+    assert torch.allclose(rx.norm(dim=-1), x.norm(dim=-1), rtol=1e-5)
+    # relative-position property: shift both positions by 5
+    ry = O.rotary_embedding(y, pos)
+    rx5, ry5 = O.rotary_embedding(x, pos + 5), O.rotary_embedding(y, pos + 5)
+    d0 = torch.einsum("bmhd,bnhd->bhmn", rx, ry)
+    d5 = torch.einsum("bmhd,bnhd->bhmn", rx5, ry5)
+    assert torch.allclose(d0, d5, atol=2e-4)
+    # complex brute force on a few entries
+    for (b, l, h, i) in [(0, 3, 1, 0), (1, 11, 2, 31), (0, 7, 0, 13)]:
+        w = 10000.0 ** (-2.0 * i / D)
+        z = complex(float(x[b, l, h, i]), float(x[b, l, h, i + D // 2])) * complex(math.cos(l * w), math.sin(l * w))
+        assert abs(float(rx[b, l, h, i]) - z.real) < 1e-5 and abs(float(rx[b, l, h, i + D // 2]) - z.imag) < 1e-5

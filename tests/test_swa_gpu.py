@@ -83,3 +83,67 @@ def test_rejects(dev):
     cache = torch.zeros(1, 8, 2, 2, 64, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         ops.swa_step(y[:, :1], y[:, :1], y[:, :1], cache, 8)  # position outside the cache
+
+
+def _rope_tables(n_pos, dev):
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, 64, 2, dtype=torch.float32) / 64))
+    ang = torch.outer(torch.arange(n_pos).float(), inv_freq)
+    return ang.cos().contiguous().to(dev), ang.sin().contiguous().to(dev)
+
+
+@pytest.mark.parametrize("B,L,H,w", [(2, 256, 3, 64), (1, 1, 2, 64), (1, 100, 2, 64), (1, 333, 4, 20), (1, 1024, 8, 64)])
+def test_prefill_with_rotary_and_cache_output(dev, B, L, H, w):
+    """Rotary inside the kernel == rotating q, k first (oracle RoPE, rounded to bf16 like the
+    reference's rotated tensors); the optional cache output holds the rotated k and v."""
+    from based_amd import ops
+
+    print(f"swa prefill rotary case B={B} L={L} H={H} w={w}", flush=True)
+    qkv = _qkv(B, L, H, seed=13)
+    pos = torch.arange(L)
+    q_r, k_r = O.rotary_embedding(qkv[:, :, 0], pos), O.rotary_embedding(qkv[:, :, 1], pos)
+    ref = O.sliding_window_attn(q_r, k_r, qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    rope = _rope_tables(L + 5, dev)
+    cache = torch.full((B, L + 2, 2, H, 64), 3.0, dtype=torch.bfloat16, device=dev)
+    out = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, rope=rope, kv_cache=cache)
+    torch.cuda.synchronize()
+    assert rel_l2(out.float(), ref.float()) < TOL
+    out2 = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, rope=rope)
+    assert torch.equal(out, out2)
+    # cache: v exact, rotated k to one bf16 rounding (fp32 contraction order may differ), rest untouched
+    c = cache.cpu()
+    assert torch.equal(c[:, :L, 1], qkv[:, :, 2])
+    assert rel_l2(c[:, :L, 0].float(), k_r.float()) < 3e-3
+    assert bool((c[:, L:] == 3.0).all())
+    # without rotary the cache receives k as it is
+    cache2 = torch.zeros_like(cache)
+    ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, kv_cache=cache2)
+    assert torch.equal(cache2.cpu()[:, :L], qkv[:, :, 1:])
+
+
+@pytest.mark.parametrize("P,T,w", [(0, 70, 64), (130, 6, 64), (10, 10, 7)])
+def test_decode_with_rotary_matches_parallel(dev, P, T, w):
+    """Prefill P tokens into the cache with in-kernel rotary, then rotary decode steps (host and
+    device positions): every step equals the parallel oracle on the rotated sequence."""
+    from based_amd import ops
+
+    B, H = 2, 3
+    L = P + T
+    qkv = _qkv(B, L, H, seed=17)
+    pos = torch.arange(L)
+    q_r, k_r = O.rotary_embedding(qkv[:, :, 0], pos), O.rotary_embedding(qkv[:, :, 1], pos)
+    ref = O.sliding_window_attn(q_r, k_r, qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    rope = _rope_tables(L, dev)
+    cache = torch.zeros(B, L, 2, H, 64, dtype=torch.bfloat16, device=dev)
+    if P > 0:
+        o0 = ops.swa_prefill(qd[:, :P, 0], qd[:, :P, 1], qd[:, :P, 2], w_left=w, rope=rope, kv_cache=cache)
+        assert rel_l2(o0.float(), ref[:, :P].float()) < TOL
+    for t in range(P, L):
+        print(f"swa rotary step case P={P} w={w} pos={t}", flush=True)
+        q, kn, vn = qd[:, t:t + 1, 0], qd[:, t:t + 1, 1], qd[:, t:t + 1, 2]
+        p = t if t % 2 == 0 else torch.full((B,), t, dtype=torch.int32, device=dev)
+        o = ops.swa_step(q, kn, vn, cache, p, w_left=w, rope=rope)
+        assert rel_l2(o.float(), ref[:, t:t + 1].float()) < TOL
+    assert rel_l2(cache[:, :, 0].float(), k_r.float()) < 3e-3
+    assert torch.equal(cache[:, :, 1].cpu(), qkv[:, :, 2])
