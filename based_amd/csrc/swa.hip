@@ -67,7 +67,7 @@ template <> struct SwaRows<true> {
 // kc_out / vc_out (optional): the (rotated) K rows and the V rows of this call are also written
 // to a KV cache, the job of _update_kv_cache (slide_attention.py:255-281).
 template <bool ROPE>
-__global__ __launch_bounds__(256) void swa_prefill_kernel(
+__global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
@@ -301,6 +301,12 @@ __global__ __launch_bounds__(256) void swa_prefill_kernel(
       }
       if (tile + 2 < tile_end) {
         load_rows(q0 + 2 * kQTile, pre, true);
+        // Measured: letting these loads overlap the next tile's compute is SLOWER (B=32:
+        // 264 us vs 247 us).  With 1024 workgroups resident, one more tile in flight per
+        // workgroup (24 MB in total) only lengthens the HBM queues; waiting here keeps the
+        // request stream of a workgroup in bursts of one tile, and the other workgroups of
+        // the compute unit cover the latency.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if constexpr (!ROPE) load_q(q0 + 2 * kQTile, bq_next);
       }
     }
