@@ -1,12 +1,18 @@
 """Generation runtime around the mixers: per-request cache bookkeeping and greedy / sampled
 decoding.  Host-side mirror of based/generation.py:18-35 (InferenceParams), :64-90 (sample),
-:93-204 (decode) and :558-578 (GenerationMixin) of the reference; the output container is a
-plain dataclass instead of the transformers classes.
+:93-204 (decode), :558-578 (GenerationMixin) and :601-739 (decode-step graph cache) of the
+reference; the output container is a plain dataclass instead of the transformers classes.
+
+The graph cache records one single-token forward of the whole stack as a HIP graph (through
+torch.cuda.CUDAGraph) and replays it per token: the kernels behind the mixers take their position
+from a device tensor (`lengths_per_sample`), allocate nothing outside torch's graph pool and read
+nothing on the host, so a replay is one launch instead of a few hundred.
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass, field
-from typing import Optional, Tuple
+from typing import Callable, Optional, Tuple
 
 import torch
 from torch import Tensor
@@ -67,14 +73,109 @@ def sample(logits: Tensor, top_k: int = 1, top_p: float = 0.0, temperature: floa
     return torch.multinomial(torch.softmax(logits_top, dim=-1), num_samples=1).squeeze(-1)
 
 
+@dataclass
+class DecodingGraphCache:
+    """Captured single-token graphs of one model, keyed by (batch_size, tokens per step), with the
+    pre-allocated per-layer caches they were recorded on (reference: DecodingCGCache, :601-610)."""
+
+    max_batch_size: int = 0
+    max_seqlen: int = 0
+    device: Optional[torch.device] = None
+    dtype: Optional[torch.dtype] = None
+    callables: dict = field(default_factory=dict)
+    mempool: Optional[tuple] = None
+    inference_params: Optional[InferenceParams] = None
+    run: Optional[Callable] = None
+
+
+@torch.inference_mode()
+def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, dtype=None, n_warmups=2):
+    """Returns a cache whose graphs fit (batch_size, max_seqlen); a larger batch, a longer
+    max_seqlen or another device/dtype throws the old graphs and caches away (reference
+    update_graph_cache, :613-680)."""
+    if cache is None:
+        cache = DecodingGraphCache()
+    param = next(iter(model.parameters()))
+    device = param.device
+    dtype = param.dtype if dtype is None else dtype
+    if ((device, dtype) != (cache.device, cache.dtype) or batch_size > cache.max_batch_size
+            or max_seqlen > cache.max_seqlen):
+        cache.callables = {}
+        cache.mempool = None
+        cache.inference_params = None
+        gc.collect()
+        cache.device, cache.dtype = device, dtype
+        cache.max_batch_size, cache.max_seqlen = batch_size, max_seqlen
+        inf_cache = model.allocate_inference_cache(batch_size, max_seqlen, dtype)
+        lengths = torch.full((batch_size,), seqlen_og, dtype=torch.int32, device=device)
+        cache.inference_params = InferenceParams(max_seqlen=max_seqlen, max_batch_size=batch_size,
+                                                 seqlen_offset=seqlen_og, key_value_memory_dict=inf_cache,
+                                                 lengths_per_sample=lengths)
+        cache.mempool = torch.cuda.graphs.graph_pool_handle()
+    if (batch_size, 1) not in cache.callables:
+        cache.callables[batch_size, 1] = capture_graph(model, cache.inference_params, batch_size, cache.max_seqlen,
+                                                       mempool=cache.mempool, n_warmups=n_warmups)
+
+    def dispatch(input_ids, position_ids, seqlen):
+        return cache.callables[input_ids.shape[0], input_ids.shape[1]](input_ids, position_ids, seqlen)
+
+    cache.run = dispatch
+    cache.inference_params.seqlen_offset = 0
+    return cache
+
+
+def capture_graph(model, inference_params, batch_size, max_seqlen, mempool=None, n_warmups=2):
+    """Records model(one token) on static input tensors; the returned callable copies new inputs
+    in, sets the device-side positions and replays (reference capture_graph, :683-739).  Warm-up
+    runs on a side stream first so that lazily created buffers (workspaces, rotary tables) exist
+    before the recording starts."""
+    device = next(iter(model.parameters())).device
+    input_ids = torch.zeros(batch_size, 1, dtype=torch.long, device=device)
+    position_ids = torch.zeros(batch_size, 1, dtype=torch.long, device=device)
+    offset_og = inference_params.seqlen_offset
+    inference_params.seqlen_offset = max_seqlen - 1
+    inference_params.lengths_per_sample[:] = max_seqlen - 1
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(n_warmups):
+            logits = model(input_ids, position_ids=position_ids, inference_params=inference_params,
+                           num_last_tokens=1).logits
+        side.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, pool=mempool):
+        logits = model(input_ids, position_ids=position_ids, inference_params=inference_params,
+                       num_last_tokens=1).logits
+
+    def run(new_input_ids, new_position_ids, seqlen):
+        inference_params.lengths_per_sample[:] = seqlen
+        input_ids.copy_(new_input_ids)
+        position_ids.copy_(new_position_ids)
+        graph.replay()
+        return logits.clone()
+
+    inference_params.seqlen_offset = offset_og
+    return run
+
+
 @torch.inference_mode()
 def decode(input_ids, model, max_length, top_k=1, top_p=0.0, temperature=1.0, eos_token_id=None,
-           teacher_outputs=None, vocab_size=None, **kwargs) -> DecodeOutput:
+           teacher_outputs=None, vocab_size=None, cg=False, **kwargs) -> DecodeOutput:
     """Prefill on `input_ids` (batch, seq_len), then one token at a time up to max_length.
-    Same control flow as the reference's `decode` without the CUDA-graph branch."""
-    batch_size, _ = input_ids.shape
+    Same control flow as the reference's `decode`; cg=True replays a recorded graph for every
+    token after the prefill."""
+    batch_size, seqlen_og = input_ids.shape
     teacher_len = teacher_outputs.shape[1] if teacher_outputs is not None else 0
-    inference_params = InferenceParams(max_seqlen=max_length, max_batch_size=batch_size)
+    if cg:
+        if not hasattr(model, "_decoding_cache"):
+            model._decoding_cache = None
+        model._decoding_cache = update_graph_cache(model, model._decoding_cache, batch_size, seqlen_og, max_length)
+        inference_params = model._decoding_cache.inference_params
+        inference_params.reset(max_length, batch_size)
+    else:
+        inference_params = InferenceParams(max_seqlen=max_length, max_batch_size=batch_size)
 
     def get_logits(ids):
         decoding = inference_params.seqlen_offset > 0
@@ -82,8 +183,11 @@ def decode(input_ids, model, max_length, top_k=1, top_p=0.0, temperature=1.0, eo
         if decoding:
             position_ids = torch.full((batch_size, 1), inference_params.seqlen_offset, dtype=torch.long,
                                       device=ids.device)
-        logits = model(ids, position_ids=position_ids, inference_params=inference_params,
-                       num_last_tokens=1).logits.squeeze(dim=1)
+        if cg and decoding:
+            logits = model._decoding_cache.run(ids, position_ids, inference_params.seqlen_offset).squeeze(dim=1)
+        else:
+            logits = model(ids, position_ids=position_ids, inference_params=inference_params,
+                           num_last_tokens=1).logits.squeeze(dim=1)
         return logits[..., :vocab_size] if vocab_size is not None else logits
 
     def next_token(logits):

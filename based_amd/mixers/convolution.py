@@ -29,10 +29,11 @@ class ShortConvolution(nn.Module):
             self._init_state(inference_params)
             state = self._get_state(inference_params)
             kk = min(self.kernel_size, l)
-            state[..., -kk:] = x[:, -kk:].transpose(1, 2)
+            state[:b, :, -kk:] = x[:, -kk:].transpose(1, 2)
         return self.conv(x.transpose(1, 2))[..., :l].transpose(1, 2)
 
     def step(self, x: torch.Tensor, state: torch.Tensor):
+        state = state[: x.shape[0]]
         state.copy_(torch.roll(state, shifts=-1, dims=-1))
         state[:, :, -1] = x.squeeze(1)
         y = torch.einsum("bdk,dgk->bd", state, self.conv.weight).to(x.dtype)
@@ -45,20 +46,17 @@ class ShortConvolution(nn.Module):
                            dtype=self.conv.weight.dtype if dtype is None else dtype)
 
     def _init_state(self, inference_params):
+        """Creates the state if it does not exist, zeroes it otherwise (a pre-allocated state may
+        be larger than the running batch; it is cleared whole)."""
         outer, inner = self.layer_idx if isinstance(self.layer_idx, tuple) else (self.layer_idx, None)
         d = inference_params.key_value_memory_dict
-        empty = self.allocate_inference_cache(inference_params.max_batch_size, inference_params.max_seqlen)
-        if inner is None:
-            if outer in d:
-                d[outer].copy_(empty)
-            else:
-                d[outer] = empty
+        if inner is not None:
+            d = d.setdefault(outer, {})
+        key = outer if inner is None else inner
+        if key in d:
+            d[key].zero_()
         else:
-            d.setdefault(outer, {})
-            if inner in d[outer]:
-                d[outer][inner].copy_(empty)
-            else:
-                d[outer][inner] = empty
+            d[key] = self.allocate_inference_cache(inference_params.max_batch_size, inference_params.max_seqlen)
 
     def _get_state(self, inference_params):
         d = inference_params.key_value_memory_dict

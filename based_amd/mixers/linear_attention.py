@@ -105,12 +105,13 @@ class LinearAttention(nn.Module):
             return self.parallel_forward(hidden_states, q, k, v)
         if inference_params.seqlen_offset > 0:
             kv_state, k_state = self._get_inference_cache(inference_params)
-            return self._step(kv_state, k_state, q, k, v)
+            # caches allocated for a larger batch serve a smaller one through their leading rows
+            return self._step(kv_state[:b], k_state[:b], q, k, v)
         y, kv_state, k_state = self.parallel_forward(hidden_states, q, k, v)
         if self.layer_idx in inference_params.key_value_memory_dict:
             # pre-allocated caches (graph-style decoding) are filled in place
-            inference_params.key_value_memory_dict[self.layer_idx][0].copy_(kv_state)
-            inference_params.key_value_memory_dict[self.layer_idx][1].copy_(k_state)
+            inference_params.key_value_memory_dict[self.layer_idx][0][:b].copy_(kv_state)
+            inference_params.key_value_memory_dict[self.layer_idx][1][:b].copy_(k_state)
         else:
             inference_params.key_value_memory_dict[self.layer_idx] = (kv_state, k_state)
         return y

@@ -41,6 +41,10 @@ class RotaryEmbedding(nn.Module):
         demand and kept (a captured decode graph holds their addresses)."""
         cached = getattr(self, "_tables", None)
         if cached is None or cached[0].shape[0] < n_pos or cached[0].device != device:
+            if cached is not None:
+                # a recorded graph may still point at the smaller tables: they stay alive (and
+                # stay correct for the positions they cover)
+                self._retired_tables = getattr(self, "_retired_tables", []) + [cached]
             cos, sin = self._cos_sin(torch.arange(n_pos, device=device))
             self._tables = (cos.contiguous(), sin.contiguous())
         return self._tables

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Based sequence-mixer hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|stack|copy]
 
 Headline workload (`value`): the recurrent decode step of Taylor linear attention at
 B=128, H=16, dv=64 — fp32 kv_state (128,16,1,64,273) + k_state, initialised from a seeded
@@ -173,6 +173,37 @@ def bench_conv(torch, ops, steps, warmup, B=4, L=2048, D=2048, K=3, decode_B=128
     }
 
 
+def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128):
+    """configs[3]: the 27-layer 360M-shaped stack (random weights, bf16): prefill of 2048 tokens,
+    then greedy decoding, eagerly and through the recorded decode graph."""
+    from based_amd.stack import GPTLMHeadModel, based_360m_config
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    model = GPTLMHeadModel(based_360m_config(), device=dev, dtype=torch.bfloat16).eval()
+    ids = torch.randint(0, 50277, (B, prefill_len), dtype=torch.long, device=dev)
+    out = {"B": B, "prefill_len": prefill_len, "new_tokens": new_tokens}
+    with torch.inference_mode():
+        model(ids[:, :64])  # warm-up (library handles, workspaces)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model(ids, num_last_tokens=1)
+        torch.cuda.synchronize()
+        out["prefill_ms"] = (time.perf_counter() - t0) * 1e3
+        out["prefill_tok_s"] = B * prefill_len / (out["prefill_ms"] * 1e-3)
+    for name, cg in (("eager", False), ("graph", True)):
+        model.generate(input_ids=ids[:, :16], max_length=prefill_len + new_tokens, cg=cg)  # warm-up / graph capture
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model.generate(input_ids=ids, max_length=prefill_len + new_tokens, cg=cg)
+        torch.cuda.synchronize()
+        total = (time.perf_counter() - t0) * 1e3
+        ms_tok = (total - out["prefill_ms"]) / new_tokens
+        out[f"decode_{name}_ms_per_token"] = ms_tok
+        out[f"decode_{name}_tok_s"] = B / (ms_tok * 1e-3)
+    return out
+
+
 def cpu_baseline_decode(torch, B=128, H=16, dv=64, sample_steps=8):
     """The oracle's recurrent step on the host: `sample_steps` of the 256 steps at full batch."""
     from oracle import based_oracle as O
@@ -245,7 +276,7 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "copy"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "copy"], default=None,
                     help="one workload only; 'copy' is a plain 256 MiB device copy used to calibrate the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     ap.add_argument("--prefill-batches", default="1,8,48,96",
@@ -296,6 +327,13 @@ def main():
         out.update({"value": round(out["conv"]["prefill_tok_s"], 1), "ms_per_step": out["conv"]["prefill_ms"], "dtype": "bf16",
                     "config": {"workload": "gated short convolution prefill B=4 L=2048 D=2048 K=3"},
                     "roofline": out["conv"]["roofline"]})
+    if args.only in (None, "stack"):
+        st = bench_stack(torch)
+        out["stack"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in st.items()}
+    if args.only == "stack":
+        out.update({"value": round(out["stack"]["decode_graph_tok_s"], 1),
+                    "ms_per_step": out["stack"]["decode_graph_ms_per_token"], "dtype": "bf16",
+                    "config": {"workload": "configs[3]: 27-layer stack, B=4, prefill 2048 + 128 greedy tokens (decode graph)"}})
     if args.only == "prefill":
         p = out["prefill"][-1]
         out.update({"value": round(p["tok_s"], 1), "ms_per_step": p["ms"], "dtype": "bf16",
