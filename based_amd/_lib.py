@@ -52,6 +52,10 @@ SIGNATURES = {
         C.c_int,
         [_P, _P, _P, _P, _P] + [_I64] * 2 + [C.c_int] + [_I64] * 2 + [C.c_int, C.c_int, _P],
     ),
+    "based_add_rms_norm": (
+        C.c_int,
+        [_P, _P, _P, _P, _P] + [_I64] * 6 + [C.c_float, C.c_int, C.c_int, _P],
+    ),
     "based_swa_step": (
         C.c_int,
         [_P, _P, _P, _P, _P, _P, _P, _I64] + [_I64] * 3 + [_I64] * 8 + [_I64] * 3

@@ -273,3 +273,41 @@ def gated_conv_step(u, state, weight, bias=None) -> torch.Tensor:
             u2d.data_ptr(), state.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
             y.data_ptr(), B, D, K, u2d.stride(0), y.stride(0), _dtype_code(u), _dtype_code(state), _stream_ptr(u)))
     return y.unsqueeze(1) if squeeze else y
+
+
+def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool = True, want_residual: bool = True):
+    """Prenorm block glue in one launch: r = x + residual (r = x when residual is None),
+    y = rms_norm(r cast to x.dtype) * weight, and r itself (fp32 when residual_in_fp32, else
+    x.dtype).  x: (..., D) with contiguous rows; returns (y, r) with r None if not wanted."""
+    _require_cuda(x, weight)
+    D = x.shape[-1]
+    if weight.shape != (D,) or weight.dtype != x.dtype:
+        raise ValueError(f"weight must be ({D},) of {x.dtype}, got {tuple(weight.shape)} {weight.dtype}")
+    x2 = x.reshape(-1, D)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    res_dtype = torch.float32 if residual_in_fp32 else x.dtype
+    r2 = None
+    if residual is not None:
+        _require_cuda(x, residual)
+        if residual.shape != x.shape:
+            raise ValueError(f"residual {tuple(residual.shape)} does not match x {tuple(x.shape)}")
+        if residual.dtype != res_dtype:
+            # a residual stream of another dtype (first block with residual_in_fp32=False, ...)
+            res_dtype = residual.dtype
+        r2 = residual.reshape(-1, D)
+        if r2.stride(-1) != 1:
+            r2 = r2.contiguous()
+    if x.dtype == torch.float32 and res_dtype != torch.float32:
+        raise ValueError("fp32 activations need an fp32 residual stream")
+    y = torch.empty(rows, D, dtype=x.dtype, device=x.device)
+    out = torch.empty(rows, D, dtype=res_dtype, device=x.device) if want_residual else None
+    res_code = _lib.BASED_F32 if res_dtype == torch.float32 else _lib.BASED_BF16
+    with torch.cuda.device(x.device):
+        _lib.check(_lib.lib().based_add_rms_norm(
+            x2.data_ptr(), r2.data_ptr() if r2 is not None else None, weight.data_ptr(), y.data_ptr(),
+            out.data_ptr() if out is not None else None, rows, D, x2.stride(0),
+            r2.stride(0) if r2 is not None else 0, y.stride(0), out.stride(0) if out is not None else 0,
+            float(eps), _dtype_code(x), res_code, _stream_ptr(x)))
+    return y.view(x.shape), (out.view(x.shape) if out is not None else None)

@@ -19,6 +19,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import ops
+
 from .generation import GenerationMixin
 from .mixers.convolution import BaseConv
 from .mixers.linear_attention import LinearAttention, TaylorExp
@@ -164,20 +166,26 @@ class Block(nn.Module):
     def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None, **kwargs):
         return self.mixer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
 
-    def forward(self, hidden_states, residual=None, mixer_kwargs=None, position_ids=None, decay=None):
+    def _add_norm(self, norm, hidden_states, residual):
+        """residual + hidden, norm of the sum, and the sum kept for the next block.  Device tensors
+        take the one-pass kernel; host tensors the literal statement of block.py:134-139."""
+        if (hidden_states.is_cuda and isinstance(norm, RMSNorm) and hidden_states.dtype == norm.weight.dtype
+                and hidden_states.shape[-1] % 8 == 0 and hidden_states.shape[-1] <= 4096):
+            return ops.add_rms_norm(hidden_states, residual, norm.weight, norm.eps, self.residual_in_fp32)
         residual = (hidden_states + residual) if residual is not None else hidden_states
-        hidden_states = self.norm1(residual.to(dtype=self.norm1.weight.dtype))
+        hidden_states = norm(residual.to(dtype=norm.weight.dtype))
         if self.residual_in_fp32:
             residual = residual.to(torch.float32)
+        return hidden_states, residual
+
+    def forward(self, hidden_states, residual=None, mixer_kwargs=None, position_ids=None, decay=None):
+        hidden_states, residual = self._add_norm(self.norm1, hidden_states, residual)
         mixer_kwargs = mixer_kwargs or {}
         if position_ids is not None or decay is not None:
             hidden_states = self.mixer(hidden_states, position_ids=position_ids, decay=decay, **mixer_kwargs)
         else:
             hidden_states = self.mixer(hidden_states, **mixer_kwargs)
-        residual = hidden_states + residual
-        hidden_states = self.norm2(residual.to(dtype=self.norm2.weight.dtype))
-        if self.residual_in_fp32:
-            residual = residual.to(torch.float32)
+        hidden_states, residual = self._add_norm(self.norm2, hidden_states, residual)
         return self.mlp(hidden_states), residual
 
 
@@ -234,6 +242,10 @@ class GPTModel(nn.Module):
         for layer in self.layers:
             hidden_states, residual = layer(hidden_states, residual=residual, position_ids=position_ids,
                                             mixer_kwargs=mixer_kwargs)
+        if (hidden_states.is_cuda and isinstance(self.ln_f, RMSNorm) and hidden_states.dtype == self.ln_f.weight.dtype
+                and hidden_states.shape[-1] % 8 == 0 and hidden_states.shape[-1] <= 4096):
+            return ops.add_rms_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.eps,
+                                    residual_in_fp32=residual.dtype == torch.float32, want_residual=False)[0]
         residual = hidden_states + residual
         return self.ln_f(residual.to(dtype=self.ln_f.weight.dtype))
 

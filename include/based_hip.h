@@ -216,6 +216,25 @@ BASED_API int based_gated_conv_step(const void* u, void* state, const void* weig
                           void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
                           int io_dtype, int state_dtype, void* stream);
 
+/*
+ * Residual add + RMSNorm of the prenorm block, one pass.  Replaces, in based/models/block.py,
+ * `residual = dropped + residual; hidden = norm(residual.to(dtype=norm.weight.dtype));
+ * residual = residual.to(torch.float32)` (:134-139 and :151-155, dropout-free) with the RMSNorm
+ * of based/ops/triton/layer_norm.py:117-118,926-953 (no bias), and the closing
+ * add + ln_f of the model (gpt.py:667-674).
+ *
+ *   x            : (rows, D), row r at x[r*x_sr]; dtype x_dtype (also the dtype of weight and y)
+ *   residual_in  : NULL (first block: r = x) or (rows, D) of residual_dtype
+ *   weight       : (D) contiguous
+ *   y            : (rows, D) = rms_norm(cast(x + residual_in)) * weight, the cast being to x_dtype
+ *   residual_out : NULL or (rows, D) of residual_dtype, receives x + residual_in (fp32 sum)
+ * D multiple of 8, at most 4096; strides multiples of 8 elements; 16-byte aligned tensors.
+ */
+BASED_API int based_add_rms_norm(const void* x, const void* residual_in, const void* weight, void* y,
+                       void* residual_out, int64_t rows, int64_t D, int64_t x_sr, int64_t ri_sr,
+                       int64_t y_sr, int64_t ro_sr, float eps, int x_dtype, int residual_dtype,
+                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -251,3 +251,12 @@ def rotary_embedding(x, positions, base: float = 10000.0):
     cos, sin = ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]
     x1, x2 = x[..., : D // 2].float(), x[..., D // 2:].float()
     return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
+
+
+def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool = True):
+    """Prenorm block glue (based/models/block.py:134-139): r = x + residual (torch promotion: fp32
+    when the residual stream is fp32), y = rms_norm(r.to(x.dtype)), r kept in fp32 if asked.
+    Returns (y, r)."""
+    r = x if residual is None else x + residual
+    y = rms_norm(r.to(x.dtype), weight, eps)
+    return y, (r.float() if residual_in_fp32 else r)
