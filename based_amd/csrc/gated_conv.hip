@@ -122,36 +122,87 @@ __global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
   }
 }
 
-template <typename T, int K>
+// Loads / stores COUNT consecutive elements (a multiple of 16 bytes, 16-byte aligned) as floats.
+template <typename E, int COUNT> __device__ __forceinline__ void load_run(const void* p, long first, float (&out)[COUNT]) {
+  constexpr int kPer = 16 / (int)sizeof(E);
+  static_assert(COUNT % kPer == 0, "run must be whole 16-byte pieces");
+  typedef typename Vec16<E>::type vec_t;
+  const vec_t* src = reinterpret_cast<const vec_t*>(reinterpret_cast<const E*>(p) + first);
+#pragma unroll
+  for (int i = 0; i < COUNT / kPer; ++i) {
+    const vec_t x = src[i];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) out[i * kPer + j] = to_f32(x[j]);
+  }
+}
+template <typename E, int COUNT> __device__ __forceinline__ void store_run(void* p, long first, const float (&in)[COUNT]) {
+  constexpr int kPer = 16 / (int)sizeof(E);
+  typedef typename Vec16<E>::type vec_t;
+  vec_t* dst = reinterpret_cast<vec_t*>(reinterpret_cast<E*>(p) + first);
+#pragma unroll
+  for (int i = 0; i < COUNT / kPer; ++i) {
+    vec_t x;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) x[j] = from_f32<E>(in[i * kPer + j]);
+    dst[i] = x;
+  }
+}
+
+// A thread owns 8 consecutive channels: their K-entry state rows and weight rows are 8 K
+// consecutive elements each, moved as 16-byte pieces.
+template <typename T, typename TS, int K>
 __global__ __launch_bounds__(256) void gated_conv_step_kernel(
-    const T* __restrict__ u, void* __restrict__ state, const T* __restrict__ weight, const T* __restrict__ bias,
-    T* __restrict__ y, int B, int D, long u_sb, long y_sb, int state_dtype) {
-  constexpr int N = Vec16<T>::kN;
-  typedef typename Vec16<T>::type vec_t;
+    const T* __restrict__ u, TS* __restrict__ state, const T* __restrict__ weight, const T* __restrict__ bias,
+    T* __restrict__ y, int B, int D, long u_sb, long y_sb) {
+  constexpr int N = 8;
   const long item = (long)blockIdx.x * 256 + threadIdx.x;
   const int per_row = D / N;
   if (item >= (long)B * per_row) return;
   const int b = (int)(item / per_row);
   const int c0 = (int)(item % per_row) * N;
-  const vec_t x1 = *reinterpret_cast<const vec_t*>(u + b * u_sb + c0);
-  const vec_t x2 = *reinterpret_cast<const vec_t*>(u + b * u_sb + D + c0);
-  vec_t out;
+  float x1[N], x2[N], st[N * K], w[N * K], bs[N], out[N];
+  load_run<T, N>(u + b * u_sb, c0, x1);
+  load_run<T, N>(u + b * u_sb, D + c0, x2);
+  load_run<TS, N * K>(state, ((long)b * D + c0) * K, st);
+  load_run<T, N * K>(weight, (long)c0 * K, w);
+#pragma unroll
+  for (int c = 0; c < N; ++c) bs[c] = 0.0f;
+  if (bias != nullptr) load_run<T, N>(bias, c0, bs);
 #pragma unroll
   for (int c = 0; c < N; ++c) {
-    const long base = ((long)b * D + c0 + c) * K;
-    float st[K];
 #pragma unroll
-    for (int j = 0; j < K - 1; ++j) st[j] = load_dyn(state, base + j + 1, state_dtype);  // roll by one
-    st[K - 1] = to_f32(x1[c]);
-    float acc = bias != nullptr ? to_f32(bias[c0 + c]) : 0.0f;
+    for (int j = 0; j < K - 1; ++j) st[c * K + j] = st[c * K + j + 1];  // roll by one
+    st[c * K + K - 1] = x1[c];
+    float acc = bs[c];
 #pragma unroll
-    for (int j = 0; j < K; ++j) {
-      acc = __builtin_fmaf(to_f32(weight[(long)(c0 + c) * K + j]), st[j], acc);
-      store_dyn(state, base + j, state_dtype, st[j]);
-    }
-    out[c] = from_f32<T>(silu(acc) * to_f32(x2[c]));
+    for (int j = 0; j < K; ++j) acc = __builtin_fmaf(w[c * K + j], st[c * K + j], acc);
+    out[c] = silu(acc) * x2[c];
   }
-  *reinterpret_cast<vec_t*>(y + b * y_sb + c0) = out;
+  store_run<TS, N * K>(state, ((long)b * D + c0) * K, st);
+  store_run<T, N>(y + b * y_sb, c0, out);
+}
+
+// SwiGLU gate of the MLP: out = u[:, :F] * silu(u[:, F:]) (based/models/mlp.py:147-151).
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ u, T* __restrict__ out, long rows, int F,
+                                                     long u_sr, long o_sr) {
+  constexpr int N = Vec16<T>::kN;
+  typedef typename Vec16<T>::type vec_t;
+  const long item = (long)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = F / N;
+  if (item >= rows * per_row) return;
+  const long r = item / per_row;
+  const int c0 = (int)(item % per_row) * N;
+  const vec_t a = *reinterpret_cast<const vec_t*>(u + r * u_sr + c0);
+  const vec_t g = *reinterpret_cast<const vec_t*>(u + r * u_sr + F + c0);
+  vec_t o;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    // torch rounds silu(gate) to the tensor dtype before the product
+    const float sg = to_f32(from_f32<T>(silu(to_f32(g[i]))));
+    o[i] = from_f32<T>(to_f32(a[i]) * sg);
+  }
+  *reinterpret_cast<vec_t*>(out + r * o_sr + c0) = o;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -177,17 +228,15 @@ int launch_gated_conv_prefill(const void* u, const void* weight, const void* bia
   return check_launch("gated_conv_prefill");
 }
 
-template <typename T>
+template <typename T, typename TS>
 int launch_gated_conv_step(const void* u, void* state, const void* weight, const void* bias, void* y,
-                           int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb, int state_dtype,
-                           hipStream_t stream) {
-  constexpr int N = Vec16<T>::kN;
-  const int64_t items = B * (D / N);
+                           int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb, hipStream_t stream) {
+  const int64_t items = B * (D / 8);
   dim3 grid((unsigned)((items + 255) / 256)), block(256);
-#define BASED_CONV_CASE(KK)                                                                             \
-  case KK:                                                                                              \
-    hipLaunchKernelGGL((gated_conv_step_kernel<T, KK>), grid, block, 0, stream, (const T*)u, state,      \
-                       (const T*)weight, (const T*)bias, (T*)y, (int)B, (int)D, u_sb, y_sb, state_dtype); \
+#define BASED_CONV_CASE(KK)                                                                              \
+  case KK:                                                                                               \
+    hipLaunchKernelGGL((gated_conv_step_kernel<T, TS, KK>), grid, block, 0, stream, (const T*)u, (TS*)state, \
+                       (const T*)weight, (const T*)bias, (T*)y, (int)B, (int)D, u_sb, y_sb);              \
     break;
   switch (K) {
     BASED_CONV_CASE(2)
@@ -234,13 +283,38 @@ extern "C" BASED_API int based_gated_conv_step(const void* u, void* state, const
   BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_step: bad io dtype");
   BASED_REQUIRE(state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_step: bad state dtype");
   BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "gated_conv_step: kernel size %d unsupported (2..4)", K);
-  const int n = io_dtype == BASED_BF16 ? 8 : 4;
-  BASED_REQUIRE(D % n == 0, BASED_ERR_SHAPE, "gated_conv_step: channel count must be a multiple of %d", n);
-  BASED_REQUIRE(u_sb % n == 0 && y_sb % n == 0, BASED_ERR_ALIGN, "gated_conv_step: strides must be multiples of %d elements", n);
-  BASED_REQUIRE(aligned16(u) && aligned16(y), BASED_ERR_ALIGN, "gated_conv_step: tensors must be 16-byte aligned");
-  BASED_REQUIRE(B * (D / n) < (1ll << 39), BASED_ERR_SHAPE, "gated_conv_step: grid too large");
+  BASED_REQUIRE(D % 8 == 0, BASED_ERR_SHAPE, "gated_conv_step: channel count must be a multiple of 8");
+  BASED_REQUIRE(u_sb % 8 == 0 && y_sb % 8 == 0, BASED_ERR_ALIGN, "gated_conv_step: strides must be multiples of 8 elements");
+  BASED_REQUIRE(aligned16(u) && aligned16(y) && aligned16(state) && aligned16(weight) && aligned16(bias),
+                BASED_ERR_ALIGN, "gated_conv_step: tensors must be 16-byte aligned");
+  BASED_REQUIRE(B * (D / 8) < (1ll << 39), BASED_ERR_SHAPE, "gated_conv_step: grid too large");
   if (B == 0) return BASED_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  return io_dtype == BASED_BF16 ? launch_gated_conv_step<__bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, state_dtype, s)
-                                : launch_gated_conv_step<float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, state_dtype, s);
+  if (io_dtype == BASED_BF16)
+    return state_dtype == BASED_BF16 ? launch_gated_conv_step<__bf16, __bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s)
+                                     : launch_gated_conv_step<__bf16, float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s);
+  return state_dtype == BASED_BF16 ? launch_gated_conv_step<float, __bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s)
+                                   : launch_gated_conv_step<float, float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s);
+}
+
+extern "C" BASED_API int based_swiglu(const void* u, void* out, int64_t rows, int64_t F, int64_t u_sr, int64_t o_sr,
+                                      int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(u && out, BASED_ERR_ARG, "swiglu: null pointer argument");
+  BASED_REQUIRE(rows >= 0 && F > 0, BASED_ERR_ARG, "swiglu: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "swiglu: bad dtype");
+  const int n = io_dtype == BASED_BF16 ? 8 : 4;
+  BASED_REQUIRE(F % n == 0, BASED_ERR_SHAPE, "swiglu: width must be a multiple of %d", n);
+  BASED_REQUIRE(u_sr % n == 0 && o_sr % n == 0, BASED_ERR_ALIGN, "swiglu: strides must be multiples of %d elements", n);
+  BASED_REQUIRE(aligned16(u) && aligned16(out), BASED_ERR_ALIGN, "swiglu: tensors must be 16-byte aligned");
+  const int64_t items = rows * (F / n);
+  BASED_REQUIRE((items + 255) / 256 < (1ll << 31), BASED_ERR_SHAPE, "swiglu: grid too large");
+  if (rows == 0) return BASED_OK;
+  dim3 grid((unsigned)((items + 255) / 256)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (io_dtype == BASED_BF16)
+    hipLaunchKernelGGL(swiglu_kernel<__bf16>, grid, block, 0, s, (const __bf16*)u, (__bf16*)out, (long)rows, (int)F, u_sr, o_sr);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, s, (const float*)u, (float*)out, (long)rows, (int)F, u_sr, o_sr);
+  return check_launch("swiglu");
 }

@@ -311,3 +311,20 @@ def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool 
             r2.stride(0) if r2 is not None else 0, y.stride(0), out.stride(0) if out is not None else 0,
             float(eps), _dtype_code(x), res_code, _stream_ptr(x)))
     return y.view(x.shape), (out.view(x.shape) if out is not None else None)
+
+
+def swiglu(u) -> torch.Tensor:
+    """u (..., 2F) -> u[..., :F] * silu(u[..., F:]), one pass."""
+    _require_cuda(u)
+    F2 = u.shape[-1]
+    if F2 % 2 != 0:
+        raise ValueError(f"last dimension must be even, got {F2}")
+    F = F2 // 2
+    u2 = u.reshape(-1, F2)
+    if u2.stride(-1) != 1:
+        u2 = u2.contiguous()
+    out = torch.empty(u2.shape[0], F, dtype=u.dtype, device=u.device)
+    with torch.cuda.device(u.device):
+        _lib.check(_lib.lib().based_swiglu(u2.data_ptr(), out.data_ptr(), u2.shape[0], F, u2.stride(0), out.stride(0),
+                                           _dtype_code(u), _stream_ptr(u)))
+    return out.view(*u.shape[:-1], F)

@@ -146,7 +146,10 @@ class GatedMlp(nn.Module):
         self.fc2 = nn.Linear(hidden_features, in_features, bias=bias2, device=device, dtype=dtype)
 
     def forward(self, x):
-        y, gate = self.fc1(x).chunk(2, dim=-1)
+        u = self.fc1(x)
+        if u.is_cuda and u.dtype in (torch.bfloat16, torch.float32) and u.shape[-1] % 16 == 0:
+            return self.fc2(ops.swiglu(u))
+        y, gate = u.chunk(2, dim=-1)
         return self.fc2(y * F.silu(gate))
 
 

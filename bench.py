@@ -192,7 +192,7 @@ def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128):
         out["prefill_ms"] = (time.perf_counter() - t0) * 1e3
         out["prefill_tok_s"] = B * prefill_len / (out["prefill_ms"] * 1e-3)
     for name, cg in (("eager", False), ("graph", True)):
-        model.generate(input_ids=ids[:, :16], max_length=prefill_len + new_tokens, cg=cg)  # warm-up / graph capture
+        model.generate(input_ids=ids, max_length=prefill_len + new_tokens, cg=cg)  # warm-up / graph capture
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         model.generate(input_ids=ids, max_length=prefill_len + new_tokens, cg=cg)

@@ -211,6 +211,7 @@ BASED_API int based_gated_conv_prefill(const void* u, const void* weight, const 
  *   u     : (B, 2D) rows at u[b*u_sb + c]     y : (B, D) rows at y[b*y_sb + c]
  *   state : (B, D, K) contiguous, updated in place
  *   bias  : (D) or NULL
+ * D must be a multiple of 8; all tensors 16-byte aligned.
  */
 BASED_API int based_gated_conv_step(const void* u, void* state, const void* weight, const void* bias,
                           void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
@@ -234,6 +235,15 @@ BASED_API int based_add_rms_norm(const void* x, const void* residual_in, const v
                        void* residual_out, int64_t rows, int64_t D, int64_t x_sr, int64_t ri_sr,
                        int64_t y_sr, int64_t ro_sr, float eps, int x_dtype, int residual_dtype,
                        void* stream);
+
+/*
+ * SwiGLU gate of the MLP: out[r, c] = u[r, c] * silu(u[r, F + c]), the element-wise part of
+ * GatedMlp.forward between fc1 and fc2 (based/models/mlp.py:147-151: y, gate = fc1(x).chunk(2);
+ * y * silu(gate)).  u: (rows, 2F) rows at u[r*u_sr]; out: (rows, F) rows at out[r*o_sr].
+ * F multiple of 8 (bf16) / 4 (fp32); strides likewise; 16-byte aligned tensors.
+ */
+BASED_API int based_swiglu(const void* u, void* out, int64_t rows, int64_t F, int64_t u_sr, int64_t o_sr,
+                 int io_dtype, void* stream);
 
 #ifdef __cplusplus
 }
