@@ -100,7 +100,7 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512)
         "wall_ms": wall,
         "roofline": {"kernel": "lin_step_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"],
+                     "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else None,
                      "algorithmic_bytes_per_launch": bytes_per_launch},
         "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, bf16 q/k/v",
     }
@@ -121,7 +121,7 @@ def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
         "tok_s": B * L / (ms * 1e-3), "ms": ms, "B": B, "L": L, "dv": dv,
         "roofline": {"kernel": "lin_prefill_mfma_kernel", "bound": "mfma", "achieved": round(tf, 2),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["lin_prefill_mfma_kernel"].get(B),
+                     "traffic": MEASURED_TRAFFIC_BYTES["lin_prefill_mfma_kernel"].get(B) if (L, dv) == (4096, 64) else None,
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": byts,
                      "hbm_gbs": round(byts / (ms * 1e-3) / 1e9, 1)},
     }
@@ -317,6 +317,13 @@ def main():
     if args.only in (None, "prefill"):
         pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
+    if args.only in (None, "prefill"):
+        # configs[4]: one 32K-token sequence at head dim 128, and its decode batch of 64
+        c5 = bench_prefill(torch, ops, 10, 3, B=1, L=32768, dv=128)
+        d5 = bench_decode(torch, ops, 64, 8, B=64, dv=128, prefill_len=256)
+        out["long_context"] = {"prefill": {k: (round(v, 3) if isinstance(v, float) else v) for k, v in c5.items()},
+                               "decode": {"tok_s": round(d5["tok_s"], 1), "ms": round(d5["ms"], 5), "B": 64, "dv": 128,
+                                          "roofline": d5["roofline"]}}
     if args.only in (None, "swa"):
         s = bench_swa(torch, ops, 20, 3)
         out["swa"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in s.items()}
