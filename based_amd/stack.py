@@ -268,6 +268,33 @@ class GPTLMHeadModel(nn.Module, GenerationMixin):
     def allocate_inference_cache(self, batch_size, max_seqlen, dtype=None, **kwargs):
         return self.transformer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
 
+    @classmethod
+    def from_pretrained_local(cls, directory, device=None, dtype=None, strict=True):
+        """Builds the model from a LOCAL directory laid out like the released checkpoints:
+        `config.json` (the GPT2Config dictionary) and `pytorch_model.bin` or `model.safetensors`.
+        Counterpart of from_pretrained_hf (gpt.py:446-459) without the hub: same key clean-up
+        (leading "model." stripped, training-metric entries dropped).  The weights file is read
+        with a loader that executes nothing from it."""
+        import json
+        import os
+        import re
+
+        with open(os.path.join(directory, "config.json")) as f:
+            config = StackConfig(**json.load(f))
+        model = cls(config, device=device, dtype=dtype)
+        st_path = os.path.join(directory, "model.safetensors")
+        if os.path.exists(st_path):
+            from safetensors.torch import load_file
+
+            state = load_file(st_path, device="cpu")
+        else:
+            state = torch.load(os.path.join(directory, "pytorch_model.bin"), map_location="cpu", weights_only=True)
+        state = {re.sub(r"^model\.", "", k): v for k, v in state.items() if "metrics" not in k}
+        if config.tie_word_embeddings and "lm_head.weight" not in state:
+            state["lm_head.weight"] = state["transformer.embeddings.word_embeddings.weight"]
+        model.load_state_dict(state, strict=strict)
+        return model
+
     def forward(self, input_ids, position_ids=None, inference_params=None, num_last_tokens=0, stream=None, **kwargs):
         assert input_ids.ndim == 2, f"Expected `input_ids` to have shape [b, slen], but got shape {input_ids.shape}"
         hidden_states = self.transformer(input_ids, position_ids=position_ids, inference_params=inference_params,

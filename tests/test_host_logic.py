@@ -118,3 +118,28 @@ def test_inference_params_reset():
     ip.reset(16, 4)
     assert (ip.max_seqlen, ip.max_batch_size, ip.seqlen_offset) == (16, 4, 0)
     assert ip.lengths_per_sample.sum() == 0
+
+
+def test_local_checkpoint_round_trip(tmp_path):
+    """A checkpoint directory in the released layout (config.json + pytorch_model.bin with the
+    training wrapper's "model." prefix and metric entries) loads into an identical model."""
+    import json
+
+    from based_amd.stack import GPTLMHeadModel, based_360m_config
+
+    cfg = based_360m_config(n_embd=128, n_head=2, n_layer=3, n_inner=256, vocab_size=96,
+                            alt_mixer={"_target_": "based.models.mixers.linear_attention.LinearAttention", "l_max": 64,
+                                       "feature_map": {"_target_": "based.models.mixers.linear_attention.TaylorExp", "input_dim": 16},
+                                       "feature_dim": 16, "num_heads": 2},
+                            alt_mixer_layers=[1], alt_mixer_2_layers=[2])
+    torch.manual_seed(1)
+    src = GPTLMHeadModel(cfg)
+    state = {"model." + k: v for k, v in src.state_dict().items()}
+    state["train_metrics.num-tokens.count"] = torch.tensor(3)
+    torch.save(state, tmp_path / "pytorch_model.bin")
+    (tmp_path / "config.json").write_text(json.dumps(vars(cfg)))
+    dst = GPTLMHeadModel.from_pretrained_local(str(tmp_path))
+    a, b = src.state_dict(), dst.state_dict()
+    assert a.keys() == b.keys()
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    assert dst.lm_head.weight is dst.transformer.embeddings.word_embeddings.weight
