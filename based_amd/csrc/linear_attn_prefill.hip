@@ -181,6 +181,20 @@ __device__ __forceinline__ void lin_prefill_chain(
   bf16x8 pf_v[2];
   auto issue_loads = [&](int t0) {
     const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
+    if (ntok == kChunk) {  // whole chunk (all but possibly the last): no zero fill, no bounds
+      if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
+        const __bf16* base = wave == 0 ? q + (long)(t0 + lane) * q_sl : k + (long)(t0 + lane) * k_sl;
+        const u32x4* src = reinterpret_cast<const u32x4*>(base);
+        pf_qk[0] = src[0];
+        pf_qk[1] = src[1];
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int piece = 256 * i + tid;
+        pf_v[i] = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + (piece >> 3)) * v_sl + 8 * (piece & 7));
+      }
+      return;
+    }
     if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
       const u32x4 z4 = {0, 0, 0, 0};
       pf_qk[0] = pf_qk[1] = z4;
@@ -273,10 +287,9 @@ __device__ __forceinline__ void lin_prefill_chain(
       for (int et = 0; et < kETiles; ++et) O[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
       // within the chunk: A^T = tril(1 + s + s^2/2)^T from a K=16 product of raw q, k; O^T += V^T A^T.
-      // Lane groups 2, 3 hold the zero padding of the K=32 contraction slots.
       {
-        const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-        const bf16x8 bq = low_half ? *reinterpret_cast<const bf16x8*>(s_q + (16 * nt + col) * kFeat + 8 * grp) : zero8;
+        // the 16 features are exactly the contraction of a 16x16x16 MFMA: lane <-> (row, features 4 grp ..+3)
+        const s16x4 bq = *reinterpret_cast<const s16x4*>(s_q + (16 * nt + col) * kFeat + 4 * grp);
         float p[4][4];  // [key tile][r]; tiles above the diagonal stay zero
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt)
@@ -284,8 +297,8 @@ __device__ __forceinline__ void lin_prefill_chain(
           for (int r = 0; r < 4; ++r) p[mt][r] = 0.f;
         static_for<nt + 1>([&](auto MT) {
           constexpr int mt = decltype(MT)::value;
-          const bf16x8 ka = low_half ? *reinterpret_cast<const bf16x8*>(s_k + (16 * mt + col) * kFeat + 8 * grp) : zero8;
-          const f32x4 a = mfma(ka, bq, f32x4{0.f, 0.f, 0.f, 0.f});
+          const s16x4 ka = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * grp);
+          const f32x4 a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka, bq, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             float pv = __builtin_fmaf(a[r], __builtin_fmaf(a[r], 1.0f / 32.0f, 0.25f), 1.0f);
