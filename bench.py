@@ -44,11 +44,19 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def _events_ms(torch, fn, steps, warmup):
-    """Average milliseconds per call of fn(), HIP events on the current stream."""
+def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0):
+    """Average milliseconds per call of fn(), HIP events on the current stream.  warmup_ms > 0
+    keeps launching (untimed) until that much wall time has passed: the board's power management
+    needs ~20 ms of sustained MFMA load to settle (boost clock -> overshoot -> steady state), and
+    the timed region should see the steady state."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    t_w = time.perf_counter()
+    while (time.perf_counter() - t_w) * 1e3 < warmup_ms:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -113,7 +121,7 @@ def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
     q = torch.randn(B, L, H, 16, generator=g).bfloat16().to(dev).transpose(1, 2)
     k = torch.randn(B, L, H, 16, generator=g).bfloat16().to(dev).transpose(1, 2)
     v = torch.randn(B, L, H, dv, generator=g).bfloat16().to(dev).transpose(1, 2)
-    ms, _ = _events_ms(torch, lambda: ops.linear_attn_prefill(q, k, v, return_state=True), steps, warmup)
+    ms, _ = _events_ms(torch, lambda: ops.linear_attn_prefill(q, k, v, return_state=True), steps, warmup, warmup_ms=30.0)
     flops = B * L * H * (4 * D_EXP * dv + 4 * D_EXP)
     byts = B * L * H * (2 * 16 + 2 * dv) * 2
     tf = flops / (ms * 1e-3) / 1e12
@@ -315,11 +323,11 @@ def main():
                     "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
                     "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5)})
     if args.only in (None, "prefill"):
-        pre = [bench_prefill(torch, ops, 10, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
+        pre = [bench_prefill(torch, ops, 30, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
     if args.only in (None, "prefill"):
         # configs[4]: one 32K-token sequence at head dim 128, and its decode batch of 64
-        c5 = bench_prefill(torch, ops, 10, 3, B=1, L=32768, dv=128)
+        c5 = bench_prefill(torch, ops, 30, 3, B=1, L=32768, dv=128)
         d5 = bench_decode(torch, ops, 64, 8, B=64, dv=128, prefill_len=256)
         out["long_context"] = {"prefill": {k: (round(v, 3) if isinstance(v, float) else v) for k, v in c5.items()},
                                "decode": {"tok_s": round(d5["tok_s"], 1), "ms": round(d5["ms"], 5), "B": 64, "dv": 128,
