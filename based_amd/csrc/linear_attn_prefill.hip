@@ -1,10 +1,13 @@
 // Causal Taylor linear attention over a whole sequence (prefill) for gfx950.
 //
-// Two kernels behind one entry point:
+// Kernels behind the entry points:
 //
-//  * lin_prefill_mfma_kernel (bf16 in/out): chunked scan, 64 tokens per chunk, ONE wavefront
-//    per (batch, head, 64-channel block) that keeps the whole running state in MFMA
-//    accumulators for the length of the sequence (no state traffic to LDS or HBM).
+//  * lin_prefill_mfma_kernel (bf16 in/out): chunked scan, 64 tokens per chunk, one workgroup
+//    of FOUR wavefronts per (batch, head, 64-channel block).  The running state stays in MFMA
+//    accumulators for the length of the sequence, split by feature slots over the four
+//    wavefronts; a bf16 image of it goes through LDS once per chunk for the read-out, which is
+//    split by tokens.  Small batches scan every sequence as concurrent segments (two passes of
+//    this kernel around lin_prefill_prefix_kernel).
 //
 //      within a chunk   A = tril(1 + s + s^2/2), s = q.k/4, from a K=16 MFMA on the raw
 //                       16-dim q, k (never expanding the features), then O^T += V^T A^T
@@ -19,10 +22,11 @@
 //      - psi(q)^T (lane <-> token, registers <-> slots) is a product of two registers with
 //        compile-time indices, because each lane group keeps q rotated by 4*group.
 //    The normaliser is carried as a 65th value channel of ones, so numerator and
-//    denominator come out of the same MFMAs.  The state contracts with psi(q) straight from
-//    its accumulator registers (accumulator layout == B/A operand layout for a product
-//    contracted over the accumulator's row index); only V needs a transpose (through LDS).
-//    At the end the 160-slot state is expanded to the (dv, 273) decode layout.
+//    denominator come out of the same MFMAs.  The in-chunk weights feed their product with V
+//    straight from the accumulator registers (accumulator layout == B/A operand layout for a
+//    product contracted over the accumulator's row index); V needs a transpose, done by the
+//    transposing LDS read.  At the end the 160-slot state is expanded to the (dv, 273) decode
+//    layout.
 //
 //  * lin_prefill_f32_kernel (fp32 or bf16 in/out, fp32 arithmetic throughout): a plain
 //    recurrent evaluation, four tokens per round.  It serves fp32 callers (tolerance 1e-4
