@@ -59,6 +59,40 @@ def test_cpu_tensors_fail_loudly():
     x = torch.zeros(1, 4, 2, 64, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         ops.swa_prefill(x, x, x)
+    with pytest.raises(ValueError):
+        ops.swa_step(x[:, :1], x[:, :1], x[:, :1], torch.zeros(1, 8, 2, 2, 64, dtype=torch.bfloat16), 3)
+    u = torch.zeros(2, 5, 32, dtype=torch.bfloat16)
+    w = torch.zeros(16, 1, 3, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.gated_conv_prefill(u, w)
+    with pytest.raises(ValueError):
+        ops.gated_conv_step(u[:, :1], torch.zeros(2, 16, 3, dtype=torch.bfloat16), w)
+    with pytest.raises(ValueError):
+        ops.add_rms_norm(u, None, torch.ones(32, dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        ops.swiglu(u)
+
+
+def test_cpu_modules_take_the_torch_statement():
+    """Host tensors go through the literal torch statement of the glue (BaseConv, the prenorm
+    add + RMSNorm, the MLP gate), which must agree with the oracle's restatement."""
+    from based_amd.mixers.convolution import BaseConv
+    from based_amd.stack import GatedMlp, RMSNorm
+    from oracle import based_oracle as O
+
+    torch.manual_seed(0)
+    conv = BaseConv(32, expand_proj=4)
+    x = torch.randn(2, 9, 32)
+    u = conv.in_proj(x)
+    ref = conv.out_proj(O.gated_short_conv(u, conv.conv.conv.weight[:, 0]))
+    assert torch.allclose(conv(x), ref, atol=1e-5)
+    norm = RMSNorm(32)
+    with torch.no_grad():
+        norm.weight.mul_(1.5)
+    assert torch.allclose(norm(x), O.rms_norm(x, norm.weight), atol=1e-5)
+    mlp = GatedMlp(32, hidden_features=64)
+    ref = O.swiglu_mlp(x, mlp.fc1.weight, mlp.fc2.weight)
+    assert torch.allclose(mlp(x), ref, atol=1e-5)
 
 
 def test_stack_routing_and_state_dict_names():
