@@ -40,7 +40,7 @@ D_EXP = 273
 MEASURED_TRAFFIC_BYTES = {
     "lin_step_kernel": 293097062,   # B=128, H=16, dv=64: fetch 146,863,104 + write 146,233,958
     "lin_prefill_mfma_kernel": {96: 2126194673},  # B=96, L=4096, dv=64, states written; keyed by batch
-    "swa_prefill_kernel": 283239285,   # B=8, H=16, L=4096: fetch 216,130,421 + write 67,108,864
+    "swa_prefill_kernel": 283244310,   # B=8, H=16, L=4096: fetch 216,135,446 + write 67,108,864
 }
 
 
