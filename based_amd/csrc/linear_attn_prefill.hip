@@ -727,7 +727,10 @@ extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, in
   if (chains * 3 >= kPrefillSlots * 2 || chunks < 2) return BASED_OK;  // enough chains already
   int64_t want = (kPrefillSlots + chains - 1) / chains;
   if (want > chunks) want = chunks;
-  const int64_t seg_chunks = (chunks + want - 1) / want;
+  int64_t seg_chunks = (chunks + want - 1) / want;
+  // a segment costs about three chunks' worth of fixed work (loading its prefix, dumping or
+  // expanding its state): below four chunks per segment more segments stop paying
+  if (seg_chunks < 4) seg_chunks = chunks < 4 ? chunks : 4;
   const int64_t segs = (chunks + seg_chunks - 1) / seg_chunks;
   if (segs < 2) return BASED_OK;
   *n_seg = segs;
