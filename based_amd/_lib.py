@@ -10,8 +10,7 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# BASED_HIP_LIB points at an alternative build of the same library (kernel experiments)
-LIB_PATH = os.environ.get("BASED_HIP_LIB") or os.path.join(_HERE, "libbased_hip.so")
+LIB_PATH = os.path.join(_HERE, "libbased_hip.so")  # the in-tree build is the only library ever loaded
 
 BASED_BF16 = 0
 BASED_F32 = 1

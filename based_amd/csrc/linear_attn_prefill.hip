@@ -373,6 +373,9 @@ __device__ __forceinline__ void lin_prefill_chain(
         const uint32_t w1 = pack_bf16(O[et][2] * inv, O[et][3] * inv);
         *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
       }
+      // the tile is re-read below in another lane layout: order the wavefront's own LDS accesses
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
 #pragma unroll
       for (int hlf = 0; hlf < 2; ++hlf) {
         const int row = 8 * hlf + (lane >> 3);

@@ -285,6 +285,9 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
       const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
       *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
     }
+    // the tile is re-read below in another lane layout: order the wavefront's own LDS accesses
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
       const int row = 8 * hlf + (lane >> 3);
@@ -335,8 +338,13 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
   const int b = bh / H, h = bh % H;
   int pos = cache_seqlens ? cache_seqlens[b] : pos_host;
   pos = __builtin_amdgcn_readfirstlane(pos);
-  if (pos < 0 || pos >= max_seqlen) return;  // out-of-range position: nothing to attend or write
-  if (rope_cos != nullptr && pos >= rope_len) return;
+  if (pos < 0 || pos >= max_seqlen || (rope_cos != nullptr && pos >= rope_len)) {
+    // A device-side position outside the cache or the rotary table cannot be reported to the
+    // host from here (the call may be a graph replay): the cache is left untouched and the
+    // output row of this (batch, head) is NaN, so the failure is visible downstream.
+    if (wave == 0) o[b * o_sb + h * o_sh + lane] = (__bf16)__builtin_nanf("");
+    return;
+  }
 
   __bf16* kc = kcache + b * c_sb + h * c_sh;
   __bf16* vc = vcache + b * c_sb + h * c_sh;
@@ -382,6 +390,7 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
     ql = to_f32((__bf16)__builtin_fmaf(ql, cs, sgn * __shfl_xor(ql, 32, 64) * sn));
     kn = to_f32((__bf16)__builtin_fmaf(kn, cs, sgn * __shfl_xor(kn, 32, 64) * sn));
     s_qrot[wave][lane] = ql;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     const f32x4* src = reinterpret_cast<const f32x4*>(&s_qrot[wave][16 * kq4]);
 #pragma unroll

@@ -1,13 +1,11 @@
-"""Gated short convolution mixer; mirrors based/models/mixers/convolution.py:16-218 (non-CUDA
-branch): depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a rolling (B, D, K)
-state for decoding.  On a HIP device everything between the two projections is one kernel
-(`ops.gated_conv_prefill` / `ops.gated_conv_step`); host tensors take the literal torch
-statement of the same arithmetic, which is what the module-level CPU tests exercise."""
+"""Gated short convolution mixer; mirrors the interface of based/models/mixers/convolution.py:16-218:
+depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a rolling (B, D, K) state for
+decoding.  Everything between the two projections is one kernel (`ops.gated_conv_prefill` /
+`ops.gated_conv_step`); there is no host-tensor path."""
 from __future__ import annotations
 
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
 
 class ShortConvolution(nn.Module):
@@ -21,25 +19,10 @@ class ShortConvolution(nn.Module):
                               padding=kernel_size - 1, bias=conv_bias, device=device, dtype=dtype)
 
     def forward(self, x: torch.Tensor, inference_params=None, **kwargs):
-        """x (b, l, d) -> (b, l, d)."""
-        b, l, d = x.shape
-        if inference_params is not None:
-            if inference_params.seqlen_offset > 0:
-                return self.step(x, self._get_state(inference_params))
-            self._init_state(inference_params)
-            state = self._get_state(inference_params)
-            kk = min(self.kernel_size, l)
-            state[:b, :, -kk:] = x[:, -kk:].transpose(1, 2)
-        return self.conv(x.transpose(1, 2))[..., :l].transpose(1, 2)
-
-    def step(self, x: torch.Tensor, state: torch.Tensor):
-        state = state[: x.shape[0]]
-        state.copy_(torch.roll(state, shifts=-1, dims=-1))
-        state[:, :, -1] = x.squeeze(1)
-        y = torch.einsum("bdk,dgk->bd", state, self.conv.weight).to(x.dtype)
-        if self.conv.bias is not None:
-            y = y + self.conv.bias
-        return y.unsqueeze(1)
+        # Holds the nn.Conv1d parameters (state-dict names) and the rolling state of BaseConv, which
+        # runs conv + SiLU + gate as one kernel; the un-gated convolution as a mixer of its own is
+        # not part of the released Based stacks and has no kernel here.
+        raise NotImplementedError("ShortConvolution on its own is outside this build; use BaseConv")
 
     def allocate_inference_cache(self, batch_size: int, max_seqlen: int, dtype=None, **kwargs):
         return torch.zeros(batch_size, self.d_model, self.kernel_size, device=self.conv.weight.device,
@@ -79,12 +62,7 @@ class BaseConv(nn.Module):
                                      device=device, dtype=dtype)
 
     def forward(self, u, position_ids=None, inference_params=None, *args, **kwargs):
-        u = self.in_proj(u)
-        if u.is_cuda:
-            return self.out_proj(self._gated_conv_hip(u, inference_params))
-        u1, u2 = torch.split(u, self.d_inner, dim=-1)
-        u_conv = F.silu(self.conv(u1, inference_params=inference_params))
-        return self.out_proj(u_conv * u2)
+        return self.out_proj(self._gated_conv_hip(self.in_proj(u), inference_params))
 
     def _gated_conv_hip(self, u, inference_params):
         """silu(conv(u1)) * u2 and the state handling of ShortConvolution.forward/step in one launch."""

@@ -4,8 +4,9 @@ Just enough of based/models/gpt.py (create_mixer_cls :64-96, create_block :347-3
 :463-485, GPTModel :510-736, GPTLMHeadModel :739-827), block.py (:114-163), mlp.py (GatedMlp
 :99-157) and the RMSNorm closed form (based/ops/triton/layer_norm.py:117-118) to run the
 27-layer Based-360m shape end to end: embeddings -> [prenorm Block(mixer, SwiGLU MLP)] x N ->
-final norm -> tied LM head, with the generation cache threaded through.  Everything here is
-ordinary torch (GEMMs go to hipBLASLt); the sequence mixers are the HIP kernels.
+final norm -> tied LM head, with the generation cache threaded through.  The GEMMs and the
+embedding lookup are ordinary torch (hipBLASLt); mixers, add + RMSNorm and the SwiGLU gate are
+the HIP kernels, and there is no host-tensor path.
 """
 from __future__ import annotations
 
@@ -17,7 +18,6 @@ from typing import Optional
 
 import torch
 import torch.nn as nn
-import torch.nn.functional as F
 
 from . import ops
 
@@ -123,15 +123,15 @@ def create_mixer_cls(config, layer_idx=None, device=None, dtype=None):
 
 
 class RMSNorm(nn.Module):
+    """x * rsqrt(mean(x^2) + eps) * weight (based/ops/triton/layer_norm.py:117-118), no bias."""
+
     def __init__(self, hidden_size, eps=1e-5, device=None, dtype=None):
         super().__init__()
         self.eps = eps
         self.weight = nn.Parameter(torch.ones(hidden_size, device=device, dtype=dtype))
 
     def forward(self, x):
-        xf = x.float()
-        rstd = torch.rsqrt(xf.square().mean(dim=-1, keepdim=True) + self.eps)
-        return (xf * rstd * self.weight.float()).to(self.weight.dtype)
+        return ops.add_rms_norm(x, None, self.weight, self.eps, want_residual=False)[0]
 
 
 class GatedMlp(nn.Module):
@@ -146,11 +146,7 @@ class GatedMlp(nn.Module):
         self.fc2 = nn.Linear(hidden_features, in_features, bias=bias2, device=device, dtype=dtype)
 
     def forward(self, x):
-        u = self.fc1(x)
-        if u.is_cuda and u.dtype in (torch.bfloat16, torch.float32) and u.shape[-1] % 16 == 0:
-            return self.fc2(ops.swiglu(u))
-        y, gate = u.chunk(2, dim=-1)
-        return self.fc2(y * F.silu(gate))
+        return self.fc2(ops.swiglu(self.fc1(x)))
 
 
 class Block(nn.Module):
@@ -170,16 +166,9 @@ class Block(nn.Module):
         return self.mixer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
 
     def _add_norm(self, norm, hidden_states, residual):
-        """residual + hidden, norm of the sum, and the sum kept for the next block.  Device tensors
-        take the one-pass kernel; host tensors the literal statement of block.py:134-139."""
-        if (hidden_states.is_cuda and isinstance(norm, RMSNorm) and hidden_states.dtype == norm.weight.dtype
-                and hidden_states.shape[-1] % 8 == 0 and hidden_states.shape[-1] <= 4096):
-            return ops.add_rms_norm(hidden_states, residual, norm.weight, norm.eps, self.residual_in_fp32)
-        residual = (hidden_states + residual) if residual is not None else hidden_states
-        hidden_states = norm(residual.to(dtype=norm.weight.dtype))
-        if self.residual_in_fp32:
-            residual = residual.to(torch.float32)
-        return hidden_states, residual
+        """residual + hidden, the norm of the sum, and the sum kept for the next block
+        (block.py:134-139), one kernel."""
+        return ops.add_rms_norm(hidden_states, residual, norm.weight, norm.eps, self.residual_in_fp32)
 
     def forward(self, hidden_states, residual=None, mixer_kwargs=None, position_ids=None, decay=None):
         hidden_states, residual = self._add_norm(self.norm1, hidden_states, residual)
@@ -215,7 +204,9 @@ class GPTModel(nn.Module):
         self.embeddings.word_embeddings = nn.Embedding(vocab, config.hidden_size, **fk)
         if config.max_position_embeddings > 0:
             self.embeddings.position_embeddings = nn.Embedding(config.max_position_embeddings, config.hidden_size, **fk)
-        norm_cls = partial(RMSNorm if config.rms_norm else nn.LayerNorm, eps=config.layer_norm_epsilon, **fk)
+        if not config.rms_norm:
+            raise NotImplementedError("the block glue kernel implements RMSNorm (rms_norm: True in the released configs)")
+        norm_cls = partial(RMSNorm, eps=config.layer_norm_epsilon, **fk)
         mlp_cls = partial(GatedMlp, hidden_features=config.n_inner, bias1=config.mlp_fc1_bias,
                           bias2=config.mlp_fc2_bias, **fk)
         self.layers = nn.ModuleList([
@@ -245,12 +236,8 @@ class GPTModel(nn.Module):
         for layer in self.layers:
             hidden_states, residual = layer(hidden_states, residual=residual, position_ids=position_ids,
                                             mixer_kwargs=mixer_kwargs)
-        if (hidden_states.is_cuda and isinstance(self.ln_f, RMSNorm) and hidden_states.dtype == self.ln_f.weight.dtype
-                and hidden_states.shape[-1] % 8 == 0 and hidden_states.shape[-1] <= 4096):
-            return ops.add_rms_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.eps,
-                                    residual_in_fp32=residual.dtype == torch.float32, want_residual=False)[0]
-        residual = hidden_states + residual
-        return self.ln_f(residual.to(dtype=self.ln_f.weight.dtype))
+        return ops.add_rms_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.eps,
+                                residual_in_fp32=residual.dtype == torch.float32, want_residual=False)[0]
 
 
 class GPTLMHeadModel(nn.Module, GenerationMixin):

@@ -160,7 +160,10 @@ BASED_API int based_swa_prefill(const void* q, const void* k, const void* v, voi
  * Writes k_new/v_new (B,1,H,64) into row `pos` of the caches, then attends rows
  * [pos - w_left, pos].  pos is cache_seqlens[b] when cache_seqlens (device int32, B
  * entries) is non-NULL — nothing is read on the host, so the call is graph-capturable —
- * else pos_host for every b.
+ * else pos_host for every b.  A host position outside [0, max_seqlen) (or beyond the rotary
+ * table) is refused with BASED_ERR_ARG; a DEVICE-side position outside that range cannot be
+ * refused by the host, so the kernel leaves the cache row unwritten and fills o[b, :, :] of that
+ * batch entry with NaN.
  *
  * kcache, vcache : element (b,t,h,c) at p[b*c_sb + t*c_st + h*c_sh + c]; the reference's
  *   packed (B, max_seqlen, 2, H, 64) cache is passed as two pointers 1 plane apart.
