@@ -38,6 +38,10 @@ SIGNATURES = {
         C.c_int,
         [_P, _P, _P, _P, _P, _P] + [_I64] * 4 + [_I64] * 12 + [C.c_float, C.c_int, _I64, _P, _I64, _P],
     ),
+    "based_linear_attn_prefill_split_static": (
+        C.c_int,
+        [_P, _P, _P, _P, _P, _P] + [_I64] * 4 + [_I64] * 12 + [C.c_float, C.c_int, _I64, _P],
+    ),
     "based_swa_prefill": (
         C.c_int,
         [_P, _P, _P, _P] + [_I64] * 3 + [_I64] * 12 + [C.c_int, C.c_float]

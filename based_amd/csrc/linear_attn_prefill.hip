@@ -32,6 +32,8 @@
 //    recurrent evaluation, four tokens per round.  It serves fp32 callers (tolerance 1e-4
 //    is out of reach of bf16 operands) and is an independent second implementation that
 //    the tests compare the MFMA kernel against at sizes the CPU cannot reach.
+#include <atomic>
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -741,38 +743,41 @@ extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, in
   return BASED_OK;
 }
 
-extern "C" BASED_API int based_linear_attn_prefill_split(
-    const void* q, const void* k, const void* v, void* y, float* kv_state, float* k_state, int64_t B,
-    int64_t H, int64_t L, int64_t dv, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
-    int64_t k_sh, int64_t k_sl, int64_t v_sb, int64_t v_sh, int64_t v_sl, int64_t y_sb, int64_t y_sh,
-    int64_t y_sl, float eps, int io_dtype, int64_t n_seg, void* workspace, int64_t workspace_bytes,
-    void* stream) {
-  using namespace based;
-  if (n_seg <= 1)
-    return based_linear_attn_prefill(q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh,
-                                     k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype, stream);
-  BASED_REQUIRE(q && k && v && y && workspace, BASED_ERR_ARG, "linear_attn_prefill_split: null pointer argument");
+namespace based {
+
+// Validation and the three launches of the segmented scan, shared by the entry point that is
+// handed a workspace and the one that uses the library's own static scratch array.
+static int launch_prefill_split(const char* who, const void* q, const void* k, const void* v, void* y,
+                                float* kv_state, float* k_state, int64_t B, int64_t H, int64_t L, int64_t dv,
+                                int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb, int64_t k_sh, int64_t k_sl,
+                                int64_t v_sb, int64_t v_sh, int64_t v_sl, int64_t y_sb, int64_t y_sh, int64_t y_sl,
+                                float eps, int io_dtype, int64_t n_seg, void* workspace, int64_t workspace_bytes,
+                                int64_t workspace_limit, void* stream) {
+  BASED_REQUIRE(q && k && v && y, BASED_ERR_ARG, "%s: null pointer argument", who);
   BASED_REQUIRE((kv_state == nullptr) == (k_state == nullptr), BASED_ERR_ARG,
-                "linear_attn_prefill_split: kv_state and k_state must both be given or both be NULL");
+                "%s: kv_state and k_state must both be given or both be NULL", who);
   BASED_REQUIRE(io_dtype == BASED_BF16 && (dv == 64 || dv == 128), BASED_ERR_SHAPE,
-                "linear_attn_prefill_split: only the bf16 MFMA path (dv 64 or 128) can be split");
-  BASED_REQUIRE(B > 0 && H > 0 && L > 0 && B * H < (1ll << 31) && L < (1ll << 31), BASED_ERR_ARG,
-                "linear_attn_prefill_split: bad sizes");
+                "%s: only the bf16 MFMA path (dv 64 or 128) can be split", who);
+  BASED_REQUIRE(B > 0 && H > 0 && L > 0 && B * H < (1ll << 31) && L < (1ll << 31), BASED_ERR_ARG, "%s: bad sizes", who);
   const int64_t chunks = (L + kChunk - 1) / kChunk;
-  BASED_REQUIRE(n_seg <= chunks && n_seg < 65536, BASED_ERR_ARG,
-                "linear_attn_prefill_split: %ld segments for %ld chunks", (long)n_seg, (long)chunks);
+  BASED_REQUIRE(n_seg >= 2 && n_seg <= chunks && n_seg < 65536, BASED_ERR_ARG, "%s: %ld segments for %ld chunks", who,
+                (long)n_seg, (long)chunks);
   const int64_t seg_chunks = (chunks + n_seg - 1) / n_seg;
   BASED_REQUIRE((n_seg - 1) * seg_chunks < chunks, BASED_ERR_ARG,
-                "linear_attn_prefill_split: segment count %ld leaves empty segments (use the plan)", (long)n_seg);
+                "%s: segment count %ld leaves empty segments (use the plan)", who, (long)n_seg);
   const int64_t chains = B * H * (dv / 64);
-  BASED_REQUIRE(workspace_bytes >= chains * n_seg * (int64_t)kSegStateFloats * 4, BASED_ERR_ARG,
-                "linear_attn_prefill_split: workspace too small");
+  const int64_t need = chains * n_seg * (int64_t)kSegStateFloats * 4;
+  if (workspace_limit >= 0)
+    BASED_REQUIRE(need <= workspace_limit, BASED_ERR_SHAPE,
+                  "%s: %ld chains x %ld segments need %ld bytes of scratch, the static array holds %ld", who,
+                  (long)chains, (long)n_seg, (long)need, (long)workspace_limit);
+  BASED_REQUIRE(workspace != nullptr, BASED_ERR_ARG, "%s: null workspace", who);
+  BASED_REQUIRE(workspace_bytes >= need, BASED_ERR_ARG, "%s: workspace too small", who);
   const int64_t strides[] = {q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl};
   for (int64_t st : strides)
-    BASED_REQUIRE(st % 8 == 0, BASED_ERR_ALIGN,
-                  "linear_attn_prefill_split: bf16 strides must be multiples of 8 elements (16 bytes)");
+    BASED_REQUIRE(st % 8 == 0, BASED_ERR_ALIGN, "%s: bf16 strides must be multiples of 8 elements (16 bytes)", who);
   BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y) && aligned16(workspace),
-                BASED_ERR_ALIGN, "linear_attn_prefill_split: tensors must be 16-byte aligned");
+                BASED_ERR_ALIGN, "%s: tensors must be 16-byte aligned", who);
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   const int seg_tokens = (int)(seg_chunks * kChunk);
@@ -782,15 +787,87 @@ extern "C" BASED_API int based_linear_attn_prefill_split(
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
-  int rc = check_launch("linear_attn_prefill_split (delta)");
+  int rc = check_launch(who);
   if (rc) return rc;
   hipLaunchKernelGGL(lin_prefill_prefix_kernel, dim3((unsigned)chains, (kSegStateFloats / 4 + 255) / 256), dim3(256), 0, s,
                      ws, (int)n_seg);
-  rc = check_launch("linear_attn_prefill_split (prefix)");
+  rc = check_launch(who);
   if (rc) return rc;
   hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)n_seg),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
-  return check_launch("linear_attn_prefill_split (read-out)");
+  return check_launch(who);
+}
+
+// Scratch of based_linear_attn_prefill_split_static: one array per GPU, part of the code object,
+// alive until the process ends.  64 MiB hold 1310 (chain, segment) state images, more than any
+// segment count the plan entry point returns (it aims at 768 workgroup slots and never exceeds
+// 1150 images).  In host code the array's name is only a handle for hipGetSymbolAddress; the
+// device address is looked up once per device and kept in g_scratch_ptr.
+constexpr int64_t kStaticScratchBytes = BASED_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char g_split_scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Device address of the current device's copy of the scratch array (nullptr + error set on failure).
+static void* static_scratch_for_current_device(const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    set_error("%s: cannot identify the current device (%s)", who, e != hipSuccess ? hipGetErrorString(e) : "index out of range");
+    return nullptr;
+  }
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p != nullptr) return p;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p != nullptr) return p;
+  e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_split_scratch));
+  if (e != hipSuccess || p == nullptr) {
+    set_error("%s: hipGetSymbolAddress of the scratch array failed on device %d: %s", who, dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  g_scratch_ptr[dev].store(p, std::memory_order_release);
+  return p;
+}
+
+}  // namespace based
+
+extern "C" BASED_API int based_linear_attn_prefill_split(
+    const void* q, const void* k, const void* v, void* y, float* kv_state, float* k_state, int64_t B,
+    int64_t H, int64_t L, int64_t dv, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+    int64_t k_sh, int64_t k_sl, int64_t v_sb, int64_t v_sh, int64_t v_sl, int64_t y_sb, int64_t y_sh,
+    int64_t y_sl, float eps, int io_dtype, int64_t n_seg, void* workspace, int64_t workspace_bytes,
+    void* stream) {
+  if (n_seg <= 1)
+    return based_linear_attn_prefill(q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh,
+                                     k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype, stream);
+  return based::launch_prefill_split("linear_attn_prefill_split", q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb,
+                                     q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype,
+                                     n_seg, workspace, workspace_bytes, -1, stream);
+}
+
+extern "C" BASED_API int based_linear_attn_prefill_split_static(
+    const void* q, const void* k, const void* v, void* y, float* kv_state, float* k_state, int64_t B,
+    int64_t H, int64_t L, int64_t dv, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+    int64_t k_sh, int64_t k_sl, int64_t v_sb, int64_t v_sh, int64_t v_sl, int64_t y_sb, int64_t y_sh,
+    int64_t y_sl, float eps, int io_dtype, int64_t n_seg, void* stream) {
+  using namespace based;
+  if (n_seg <= 1)  // the unsplit kernel has no scratch at all
+    return based_linear_attn_prefill(q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh,
+                                     k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype, stream);
+  // size check first: an oversized request is refused without touching the device
+  if (io_dtype == BASED_BF16 && (dv == 64 || dv == 128) && B > 0 && H > 0)
+    BASED_REQUIRE(B * H * (dv / 64) * n_seg * (int64_t)kSegStateFloats * 4 <= kStaticScratchBytes, BASED_ERR_SHAPE,
+                  "linear_attn_prefill_split_static: %ld chains x %ld segments need %ld bytes of scratch, the "
+                  "static array holds %ld",
+                  (long)(B * H * (dv / 64)), (long)n_seg, (long)(B * H * (dv / 64) * n_seg * (int64_t)kSegStateFloats * 4),
+                  (long)kStaticScratchBytes);
+  void* scratch = static_scratch_for_current_device("linear_attn_prefill_split_static");
+  if (scratch == nullptr) return BASED_ERR_LAUNCH;
+  return launch_prefill_split("linear_attn_prefill_split_static", q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb,
+                              q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype, n_seg,
+                              scratch, kStaticScratchBytes, kStaticScratchBytes, stream);
 }

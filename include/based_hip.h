@@ -122,6 +122,31 @@ BASED_API int based_linear_attn_prefill_split(const void* q, const void* k, cons
                               int64_t n_seg, void* workspace, int64_t workspace_bytes, void* stream);
 
 /*
+ * based_linear_attn_prefill_split without a workspace argument and without any allocation.
+ * No counterpart in the reference: it exists for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The
+ * per-segment states go to a static device array that is part of the library's code object:
+ * BASED_STATIC_SCRATCH_BYTES (64 MiB) per GPU the library runs on, held until the process
+ * ends.  B*H*(dv/64) * n_seg * 51,200 bytes must fit (every segment count that
+ * based_linear_attn_prefill_plan returns does); larger requests return BASED_ERR_SHAPE and
+ * launch nothing.  The first call on a device looks the array's address up (make it outside
+ * a capture).  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (different streams, different threads) race; calls ordered on one stream do not.  The array
+ * keeps the previous call's contents; the kernels overwrite every entry they read.
+ * Arguments and results are those of based_linear_attn_prefill_split; n_seg <= 1 forwards to
+ * based_linear_attn_prefill, which uses no scratch.
+ */
+#define BASED_STATIC_SCRATCH_BYTES (64ll << 20)
+BASED_API int based_linear_attn_prefill_split_static(const void* q, const void* k, const void* v, void* y,
+                              float* kv_state, float* k_state,
+                              int64_t B, int64_t H, int64_t L, int64_t dv,
+                              int64_t q_sb, int64_t q_sh, int64_t q_sl,
+                              int64_t k_sb, int64_t k_sh, int64_t k_sl,
+                              int64_t v_sb, int64_t v_sh, int64_t v_sl,
+                              int64_t y_sb, int64_t y_sh, int64_t y_sl,
+                              float eps, int io_dtype, int64_t n_seg, void* stream);
+
+/*
  * Sliding-window causal softmax attention over a whole sequence.
  * Replaces the flash-attn call behind FlashSelfAttention / FlashCrossAttention with
  * causal=True, window_size=(w_left, 0): based/models/mixers/slide_attention.py:100-106,

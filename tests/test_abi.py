@@ -67,3 +67,8 @@ def test_argument_validation_without_gpu():
     # gated convolution: kernel size outside 2..4 -> BASED_ERR_SHAPE
     rc = lib.based_gated_conv_prefill(p, p, None, p, None, 1, 4, 8, 5, 64, 16, 32, 8, 0, 0, None)
     assert rc == 1
+    # allocation-free segmented prefill: more scratch than the static array holds -> BASED_ERR_SHAPE,
+    # refused before any HIP call
+    rc = lib.based_linear_attn_prefill_split_static(p, p, p, p, None, None, 256, 16, 4096, 64, 0, 0, 16, 0, 0, 16,
+                                                    0, 0, 64, 0, 0, 64, 1e-12, 0, 4, None)
+    assert rc == 1 and b"scratch" in lib.based_hip_last_error()
