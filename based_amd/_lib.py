@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libbased_hip.so")  # the in-tree build is the on
 
 BASED_BF16 = 0
 BASED_F32 = 1
+PREFILL_SEGMENT_STATE_BYTES = 43008  # BASED_PREFILL_SEGMENT_STATE_BYTES of include/based_hip.h
 
 _I64 = C.c_int64
 _P = C.c_void_p

@@ -74,10 +74,7 @@ __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
 
 constexpr int kChunk = 64;       // tokens per chunk
 constexpr int kFTiles = 10;      // 160 symmetric feature slots = 10 tiles of 16 (see own_tile)
-constexpr int kETiles = 5;       // 64 value channels + 1 normaliser channel (tile 4, column 0)
-constexpr int kVStride = 80;     // bf16 per V row in LDS (64 channels + pad): 160 B rows make the
-                                 // transposing reads below conflict-free
-constexpr int kOStride = 72;     // bf16 per row of the output staging tile (64 channels + pad, 144 B)
+constexpr int kCTiles = 4;       // 64 value channels = 4 tiles of 16
 constexpr float kSqrt2 = 1.4142135623730951f;
 
 // Position of chunk-relative token tau inside a V^T row / inside the contraction slots:
@@ -89,19 +86,54 @@ __device__ __forceinline__ int slot_token(int s, int g, int jj) {
 
 constexpr int kWavesPerChain = 4;   // wavefronts cooperating on one (batch, head, channel block)
 // Slot tiles of the state owned by wavefront w: {0,1,2}, {3,4,5}, {6,7}, {8,9}.  The wavefronts
-// with fewer slot tiles own the token tiles with more causal work (see the kernel), which
-// balances the MFMA count per wavefront to 58..62 per chunk.
+// with fewer slot tiles own the token tiles with more causal work (see the kernel), and
+// wavefront kNormWave also carries the normaliser state, which balances the MFMA count per
+// wavefront to 46..49 per chunk.
 __host__ __device__ constexpr int own_count(int wave) { return wave < 2 ? 3 : 2; }
 __host__ __device__ constexpr int own_tile(int wave, int i) { return (wave < 2 ? 3 * wave : 2 * wave + 2) + i; }
 static_assert(own_tile(3, own_count(3) - 1) == kFTiles - 1, "slot tiles must be covered exactly");
+constexpr int kNormWave = 2;
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
-constexpr int kSbBytes = 5 * kETiles * 64 * 16;   // bf16 image of the state: [slab][channel tile][lane] x 16 B
 
-// The whole per-chain loop as seen by wavefront `wave` (a compile-time role: the four roles run
-// different instruction streams, chosen by a scalar branch at kernel entry, and meet only at
-// the workgroup barriers).
+// LDS of one workgroup (80,000 B: two workgroups per compute unit).
+//   data ring, 3 slots : the q, k, v rows of a chunk, written by direct global->LDS loads two
+//                        chunks ahead of their use (no registers, HBM latency fully covered).
+//                        q, k: 64 rows x 32 B.  v: 64 rows x 128 B whose eight 16-byte pieces
+//                        are stored at piece index p ^ 2 (row & 3), which makes the transposing
+//                        reads below bank-conflict free without row padding (a direct load
+//                        writes the 64 lanes' pieces back to back, so rows cannot be padded).
+//   state image, 2     : bf16 image of the state, [slab][channel tile][lane] x 16 B; chunk c is
+//                        read out from image[c & 1] while image[(c+1) & 1] is being written.
+//   K2, K1, 2 each     : normaliser state (see below).
+constexpr int kRing = 3;
+constexpr int kQkBytes = kChunk * kFeat * 2;       // 2 KB
+constexpr int kVBytes = kChunk * 64 * 2;           // 8 KB
+constexpr int kDataBytes = 2 * kQkBytes + kVBytes; // one ring slot: q | k | v
+constexpr int kDataK = kQkBytes, kDataV = 2 * kQkBytes;
+constexpr int kImgBytes = 5 * kCTiles * 64 * 16;   // state image: [slab][channel tile][lane] x 16 B
+constexpr int kK2Bytes = 2 * 64 * 8;               // hi and lo halves of the 16x16 second-moment operand
+constexpr int kOffData = 0;
+constexpr int kOffImg = kOffData + kRing * kDataBytes;
+constexpr int kOffK2 = kOffImg + 2 * kImgBytes;
+constexpr int kOffK1 = kOffK2 + 2 * kK2Bytes;      // [2][16] floats: first moment of k
+constexpr int kLdsBytes = kOffK1 + 2 * 16 * 4;
+static_assert(kLdsBytes <= 80 * 1024, "two workgroups must fit the 160 KB of a compute unit");
+static_assert(kOffImg % 16 == 0 && kOffK2 % 16 == 0 && kOffK1 % 16 == 0, "16-byte aligned sections");
+constexpr int kLoadsPerUpdater = 3;   // of the 12 wave-wide direct loads of a chunk: q 2, k 2, v 8
+
+// One chain = one (batch, head, 64-channel block), scanned in chunks of 64 tokens by a workgroup
+// of EIGHT wavefronts in two kinds of roles that run concurrently and meet at one barrier per
+// chunk:
+//   readers  (wavefronts 0..3, one per token tile of the chunk): O^T = V^T A^T + S^T psi(q)^T, the
+//            normaliser, the division and the store.  They read the chunk's rows and the bf16
+//            image of the state as it was before the chunk.
+//   updaters (wavefronts 4..7, each owning slot tiles own_tile(w, .)): stage the next chunk's rows
+//            into LDS, request the rows after that, S += psi(k)^T V in fp32 accumulators, and
+//            publish the bf16 image of the new state for the next chunk's readers.
+// A SIMD hosts one reader and one updater of each resident workgroup, so the vector work of one
+// role runs under the MFMAs of the other.  Every psi element is generated exactly once.
 //
 // MODE selects how much of a sequence one workgroup scans (small batches split each sequence
 // into segments so that the whole GPU has work; see based_linear_attn_prefill_split):
@@ -110,52 +142,346 @@ constexpr int kSbBytes = 5 * kETiles * 64 * 16;   // bf16 image of the state: [s
 //               zero and dumped to the workspace at the end (the segment's contribution);
 //   kModeFrom   tokens [t_begin, t_end) in full, state starting from the workspace entry (the
 //               exclusive prefix over the earlier segments).
+//
+// The normaliser z_i = sum_{j<=i} (1 + s_ij + s_ij^2/2), s_ij = q_i.k_j/4, is NOT carried as a
+// 65th value channel.  Over the earlier chunks it is the quadratic form
+//   N + q_i.K1/4 + q_i^T K2 q_i/32,  N = number of earlier tokens, K1 = sum_j k_j, K2 = sum_j k_j k_j^T,
+// which costs one MFMA on the raw q (K2 as a hi + lo pair of bf16 operands) and four
+// multiply-adds per lane; inside the chunk it is the row sum of the in-chunk weights.  K2 is one
+// 16x16 accumulator tile (two MFMAs per chunk on the k^T operand that psi(k) is generated from).
 constexpr int kModeFull = 0, kModeDelta = 1, kModeFrom = 2;
-constexpr int kSegStateFloats = kFTiles * kETiles * 64 * 4;  // accumulator image of one chain's state
+// One chain's state as it goes through the workspace of the segmented scan: the accumulator image
+// of S (slot tile, channel tile, lane, 4), then the accumulators of K2 and of K1 (lane, 4 each).
+constexpr int kSegStateFloats = BASED_PREFILL_SEGMENT_STATE_BYTES / 4;
+constexpr int kWsK2 = kFTiles * kCTiles * 256;
+constexpr int kWsK1 = kWsK2 + 256;
+static_assert(kWsK1 + 256 == kSegStateFloats, "workspace layout");
+constexpr int kThreads = 64 * 2 * kWavesPerChain;  // 4 readers + 4 updaters
 
-template <int wave, int MODE>
-__device__ __forceinline__ void lin_prefill_chain(
-    __bf16* s_q, __bf16* s_k, __bf16* s_v, unsigned char* s_sb, __bf16* s_o,
-    const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
-    __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
-    int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
-    long v_sl, long y_sb, long y_sh, long y_sl, float eps, float* __restrict__ ws, int seg_tokens, int n_seg) {
-  const int tid = threadIdx.x;
+// sum over the four lane groups (lanes col, col+16, col+32, col+48); every lane gets the total
+__device__ __forceinline__ float group_allreduce(float x) {
+  x += __shfl_xor(x, 16, 64);
+  x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+// The loop bodies below are written as sequences of STAGES.  A stage first issues the LDS reads
+// for the operands of the next stage, then runs its own group of MFMAs interleaved with the
+// vector instructions that build the next stage's register operand (psi(q) or psi(k) tiles, the
+// in-chunk weights), so that neither LDS latency nor the vector work sits between two MFMAs of
+// one wavefront.  sched_barrier pins the stage boundaries, sched_group_barrier the interleave.
+#define BASED_STAGE_END() __builtin_amdgcn_sched_barrier(0)
+// NM groups of (1 MFMA, NV vector instructions); the rest of the region floats behind
+template <int NM, int NV>
+__device__ __forceinline__ void interleave() {
+  static_for<NM>([](auto) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);
+  });
+}
+
+#define BASED_CHAIN_PARAMS                                                                                          \
+  unsigned char *lds, const __bf16 *__restrict__ q, const __bf16 *__restrict__ k, const __bf16 *__restrict__ v,      \
+      __bf16 *__restrict__ y, float *__restrict__ kv_state, float *__restrict__ k_state, int H, int L, int dv,       \
+      long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh, long v_sl, long y_sb,  \
+      long y_sh, long y_sl, float eps, float *__restrict__ ws, int seg_tokens, int n_seg
+
+// chain number of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin by workgroup
+// id.  Chains whose q/k rows share cache lines (neighbouring heads of one batch entry: 32-byte
+// rows, 512 bytes apart) should sit behind the same L2, so consecutive chain numbers are laid
+// along one XCD: chain = (id mod 8) * ceil(n / 8) + id / 8 when that stays in range.
+__device__ __forceinline__ long chain_of_block() {
+  const long n_chain = gridDim.x;
+  const long per_xcd = (n_chain + 7) / 8;
+  if (n_chain % 8 != 0) return blockIdx.x;  // irregular grids keep the identity mapping
+  return (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+}
+
+// Transposing 64-bit LDS read pair: inside each group of 16 lanes, lane 4a + b receives element
+// b of what lanes a, a+4, a+8, a+12 loaded.  `p` is the lane's source address for the first four
+// tokens; the second four are `hi_bytes` further on.
+__device__ __forceinline__ bf16x8 load_tr_pair(const unsigned char* p, int hi_bytes) {
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(p + hi_bytes));
+  const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(bf16x8, both);
+}
+// V^T operand tile of channel tile et, token slab s (lane <-> channel 16 et + col, slots jj <->
+// tokens 32 s + 16 (jj/4) + 4 grp + jj%4) from the swizzled V rows of a ring slot: source lane
+// 4j + a of a group fetches channels 16 et + 4a..+3 of token 32 s + 4 grp + j (+16), which sit in
+// 16-byte piece (2 et + a/2) ^ 2j of the row, i.e. at byte ((et ^ j) << 5) + 8a.
+// vt_lane = 128 (4 grp + j) + 8a is the lane's part of the address.
+__device__ __forceinline__ bf16x8 load_vt(const unsigned char* slot, int vt_lane, int j, int et, int s) {
+  return load_tr_pair(slot + kDataV + vt_lane + (((et ^ j) & 3) << 5) + 4096 * s, 2048);
+}
+// k^T operand tile of token slab s (lane <-> feature col) from the row-major 32-byte k rows
+__device__ __forceinline__ bf16x8 load_kt(const unsigned char* slot, int kt_lane, int s) {
+  return load_tr_pair(slot + kDataK + kt_lane + 1024 * s, 512);
+}
+
+// Workgroup barriers of the chunk loop.  __syncthreads() would make an updater wait for ALL of
+// its outstanding direct global->LDS loads, including the ones requested two chunks ahead, so
+// the two roles use narrower forms:
+//  * readers only touch LDS: a workgroup fence restricted to the LDS address space;
+//  * updaters spell the waits out: own LDS traffic done (lgkmcnt 0), and all but the newest
+//    `newest` direct loads landed (vmcnt); s_waitcnt immediates are gfx9-encoded
+//    (vmcnt[3:0] | expcnt 7 << 4 | lgkmcnt << 8).
+__device__ __forceinline__ void barrier_reader() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+template <int newest>
+__device__ __forceinline__ void barrier_updater() {
+  static_assert(newest >= 0 && newest < 16, "vmcnt immediate");
+  __builtin_amdgcn_s_waitcnt(0x0070 | newest);
+  __builtin_amdgcn_s_barrier();
+}
+
+// ------------------------------------------------------------------------------------------
+// reader of token tile nt
+// ------------------------------------------------------------------------------------------
+template <int nt, int MODE>
+__device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
+  const int lane = threadIdx.x & 63;
+  const int col = lane & 15;
+  const int grp = lane >> 4;
+  const long bh = chain_of_block();
+  const int eb = blockIdx.y;  // 64-channel block of the value dimension
+  const int b = (int)(bh / H), h = (int)(bh % H);
+  y += b * y_sb + h * y_sh + 64 * eb;
+  const int seg = blockIdx.z;
+  const int t_begin = MODE == kModeFull ? 0 : seg * seg_tokens;
+  const int t_end = MODE == kModeFull ? L : (t_begin + seg_tokens < L ? t_begin + seg_tokens : L);
+  const bool last_seg = MODE == kModeFull || seg == n_seg - 1;
+  const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
+  const int vt_j = col >> 2;
+  const int vt_lane = 128 * (4 * grp + vt_j) + 8 * (col & 3);
+  // output: after the lane-group exchange below a lane owns 2 x 8 consecutive channels of its token
+  const int out_ch = (grp & 1) * 32 + 4 * (grp & 2);
+  using std::integral_constant;
+
+  barrier_reader();  // chunk 0 and the initial state are staged
+  int slot_i = 0, buf = 0;
+  for (int t0 = t_begin; t0 < t_end; t0 += kChunk, buf ^= 1, slot_i = slot_i == kRing - 1 ? 0 : slot_i + 1) {
+    if constexpr (MODE != kModeDelta) {
+      const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
+      const unsigned char* slot = lds + kOffData + slot_i * kDataBytes;
+      const __bf16* s_q = reinterpret_cast<const __bf16*>(slot);
+      const __bf16* s_k = reinterpret_cast<const __bf16*>(slot + kDataK);
+      const unsigned char* s_img = lds + kOffImg + buf * kImgBytes;
+
+      // O^T[channel tile]: lane <-> token 16 nt + col, regs <-> channel 4 grp + r
+      f32x4 O[kCTiles];
+#pragma unroll
+      for (int et = 0; et < kCTiles; ++et) O[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+      // ---- reads of the first stages ----
+      // the 16 raw features are exactly the contraction of a 16x16x16 MFMA: lane <-> (row, features 4 grp ..+3)
+      const s16x4 bq = *reinterpret_cast<const s16x4*>(s_q + (16 * nt + col) * kFeat + 4 * grp);
+      bf16x4 qx[4];  // q of token 16 nt + col, rotated by 4 grp
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        qx[i] = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + ((4 * grp + 4 * i) & 15));
+      const unsigned char* k2 = lds + kOffK2 + buf * kK2Bytes;
+      const s16x4 k2hi = *reinterpret_cast<const s16x4*>(k2 + lane * 8);
+      const s16x4 k2lo = *reinterpret_cast<const s16x4*>(k2 + 512 + lane * 8);
+      const f32x4 k1 = *reinterpret_cast<const f32x4*>(lds + kOffK1 + buf * 64 + 16 * grp);
+      s16x4 ka[nt + 1];
+#pragma unroll
+      for (int mt = 0; mt <= nt; ++mt)
+        ka[mt] = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * grp);
+      auto img_load = [&](int sg, bf16x8 (&A)[kCTiles]) {
+#pragma unroll
+        for (int et = 0; et < kCTiles; ++et)
+          A[et] = *reinterpret_cast<const bf16x8*>(s_img + ((sg * kCTiles + et) * 64 + lane) * 16);
+      };
+      bf16x8 A[5][kCTiles];
+      img_load(0, A[0]);
+      BASED_STAGE_END();
+
+      // ---- qr[r] = q[(4 grp + r) mod 16] as floats ----
+      float qr[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) qr[4 * i + c] = to_f32(qx[i][c]);
+      const float fix8_0 = (grp == 2) ? 1.0f : 0.0f;  // slot (tile 8, position 8) = constant feature
+      auto psi_q = [&](auto SG) -> bf16x8 {
+        constexpr int sg = decltype(SG)::value;  // slab of 32 slots = slot tiles 2 sg, 2 sg + 1
+        float f[8];
+        static_for<8>([&](auto JJ) {
+          constexpr int jj = decltype(JJ)::value;
+          constexpr int t = 2 * sg + jj / 4;  // slot tile
+          constexpr int c = jj % 4;           // position 4 grp + c
+          const float own = qr[c];
+          if constexpr (t == 0) {
+            f[jj] = own * own;
+          } else if constexpr (t <= 7) {
+            f[jj] = own * qr[(c - t) & 15];
+          } else if constexpr (t == 8) {
+            const float prod = own * qr[(c - 8) & 15];
+            f[jj] = low_half ? prod : (c == 0 ? fix8_0 : 0.0f);
+          } else {
+            f[jj] = own;
+          }
+        });
+        return pack8(f);
+      };
+      BASED_STAGE_END();
+
+      // ---- stage Z: normaliser product and in-chunk scores (raw q, k operands) | psi(q) slab 0 ----
+      // normaliser over the earlier chunks: U = K2 q with K2 = hi + lo (one K=32 MFMA over [hi | lo] x [q; q])
+      const s16x8 k2both = {k2hi[0], k2hi[1], k2hi[2], k2hi[3], k2lo[0], k2lo[1], k2lo[2], k2lo[3]};
+      const s16x8 bqbq = {bq[0], bq[1], bq[2], bq[3], bq[0], bq[1], bq[2], bq[3]};
+      const f32x4 u = mfma(__builtin_bit_cast(bf16x8, k2both), __builtin_bit_cast(bf16x8, bqbq), f32x4{0.f, 0.f, 0.f, 0.f});
+      f32x4 a[nt + 1];
+#pragma unroll
+      for (int mt = 0; mt <= nt; ++mt)
+        a[mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka[mt], bq, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      bf16x8 Bq[5];
+      Bq[0] = psi_q(integral_constant<int, 0>{});
+      interleave<nt + 2, 3>();
+      BASED_STAGE_END();
+
+      // ---- stages R0..R4: O^T += S^T psi(q)^T, slab by slab | next psi(q) slab, in-chunk weights ----
+      // this lane's share of the normaliser of token 16 nt + col: first the quadratic form over
+      // the earlier chunks, then the row sums of the in-chunk weights
+      float zpart = 0.f;
+      bf16x8 vt_p[2][kCTiles];
+      bf16x8 bp[2];
+      // in-chunk weights 1 + s + s^2/2 (s = a/4) of key tiles 2 s, 2 s + 1, masked on the diagonal
+      // tile, packed as the B operand of the V^T A^T product; tiles above the diagonal are zero
+      auto weights = [&](auto SS) {
+        constexpr int s = decltype(SS)::value;
+        float pb[8];
+        static_for<2>([&](auto HH) {
+          constexpr int mt = 2 * s + decltype(HH)::value;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float pv = 0.f;
+            if constexpr (mt <= nt) {
+              pv = __builtin_fmaf(a[mt][r], __builtin_fmaf(a[mt][r], 1.0f / 32.0f, 0.25f), 1.0f);
+              if (mt == nt) pv = (4 * grp + r <= col) ? pv : 0.f;  // key <= query on the diagonal tile
+              zpart += pv;
+            }
+            pb[4 * decltype(HH)::value + r] = pv;
+          }
+        });
+        bp[s] = pack8(pb);
+      };
+      static_for<5>([&](auto SG) {
+        constexpr int sg = decltype(SG)::value;
+        if constexpr (sg + 1 < 5) img_load(sg + 1, A[sg + 1]);
+        if constexpr (sg == 3) {
+#pragma unroll
+          for (int et = 0; et < kCTiles; ++et) vt_p[0][et] = load_vt(slot, vt_lane, vt_j, et, 0);
+        }
+        if constexpr (sg == 4 && nt >= 2) {
+#pragma unroll
+          for (int et = 0; et < kCTiles; ++et) vt_p[1][et] = load_vt(slot, vt_lane, vt_j, et, 1);
+        }
+#pragma unroll
+        for (int et = 0; et < kCTiles; ++et) O[et] = mfma(A[sg][et], Bq[sg], O[et]);
+        if constexpr (sg + 1 < 5) Bq[sg + 1] = psi_q(integral_constant<int, sg + 1>{});
+        if constexpr (sg == 0) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            zpart = __builtin_fmaf(qr[r], __builtin_fmaf(u[r], 1.0f / 32.0f, k1[r] * 0.25f), zpart);
+          weights(integral_constant<int, 0>{});
+        }
+        if constexpr (sg == 1 && nt >= 2) weights(integral_constant<int, 1>{});
+        interleave<4, (sg == 0 ? 9 : (sg == 1 && nt >= 2) ? 8 : 3)>();
+        BASED_STAGE_END();
+      });
+
+      // ---- stages P0, P1: O^T += V^T A^T | the normaliser ----
+      float inv = 0.f;
+      static_for<nt / 2 + 1>([&](auto SS) {
+        constexpr int s = decltype(SS)::value;
+#pragma unroll
+        for (int et = 0; et < kCTiles; ++et) O[et] = mfma(vt_p[s][et], bp[s], O[et]);
+        if constexpr (s == 0) {
+          // the earlier tokens count 1 each, the lane groups hold partial sums of the rest
+          const float z = group_allreduce(zpart) + (float)t0;
+          inv = __builtin_amdgcn_rcpf(z + eps);
+        }
+        BASED_STAGE_END();
+      });
+
+      // ---- normalise and store ----
+      // A lane holds 4 channels (8 bytes) of each channel tile.  Lane groups g and g ^ 1 trade two
+      // tiles (one row swap per dword), after which every lane holds 2 x 8 consecutive channels
+      // and stores 16 contiguous bytes twice, straight from registers.
+      uint32_t P[kCTiles][2];
+#pragma unroll
+      for (int et = 0; et < kCTiles; ++et) {
+        P[et][0] = pack_bf16(O[et][0] * inv, O[et][1] * inv);
+        P[et][1] = pack_bf16(O[et][2] * inv, O[et][3] * inv);
+      }
+#pragma unroll
+      for (int e = 0; e < 2; ++e)
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+          asm volatile("v_permlane16_swap_b32 %0, %1" : "+v"(P[e][d]), "+v"(P[e + 2][d]));
+      {
+        const int tau = 16 * nt + col;
+        if (tau < ntok) {
+          __bf16* dst = y + (long)(t0 + tau) * y_sl + out_ch;
+          *reinterpret_cast<u32x4*>(dst) = u32x4{P[0][0], P[0][1], P[2][0], P[2][1]};
+          *reinterpret_cast<u32x4*>(dst + 16) = u32x4{P[1][0], P[1][1], P[3][0], P[3][1]};
+        }
+      }
+    }
+    barrier_reader();  // the next chunk's rows and state image are complete
+  }
+
+  // the updaters expand the state into the decode layout; readers help to copy it out
+  if constexpr (MODE != kModeDelta) {
+    if (kv_state != nullptr && last_seg) {
+      const float* blk = reinterpret_cast<const float*>(lds + kOffImg);
+#pragma unroll 1
+      for (int et = 0; et < kCTiles; ++et) {
+        __syncthreads();
+        __syncthreads();
+        f32x4* dst = reinterpret_cast<f32x4*>(kv_state + (bh * dv + 64 * eb + 16 * et) * kExp);
+        const f32x4* src = reinterpret_cast<const f32x4*>(blk);
+        for (int idx = threadIdx.x; idx < 16 * kExp / 4; idx += kThreads) dst[idx] = src[idx];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// updater owning slot tiles own_tile(w, .)
+// ------------------------------------------------------------------------------------------
+template <int w, int MODE>
+__device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
+  const int tid = threadIdx.x - 64 * kWavesPerChain;  // 0..255 among the updaters
   const int lane = tid & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
-  // Workgroups are dealt to the 8 XCDs round-robin by workgroup id.  Chains whose q/k rows share
-  // cache lines (neighbouring heads of one batch entry: 32-byte rows, 512 bytes apart) should
-  // sit behind the same L2, so consecutive chain numbers are laid along one XCD:
-  // chain = (id mod 8) * ceil(n / 8) + id / 8 when that stays in range.
-  const long n_chain = gridDim.x;
-  const long per_xcd = (n_chain + 7) / 8;
-  long bh = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (n_chain % 8 != 0) bh = blockIdx.x;  // irregular grids keep the identity mapping
+  const long bh = chain_of_block();
   const int eb = blockIdx.y;  // 64-channel block of the value dimension
   const int b = (int)(bh / H), h = (int)(bh % H);
-
   q += b * q_sb + h * q_sh;
   k += b * k_sb + h * k_sh;
   v += b * v_sb + h * v_sh + 64 * eb;
-  y += b * y_sb + h * y_sh + 64 * eb;
+  constexpr int kOwn = own_count(w);
+  constexpr bool kNorm = w == kNormWave;
+  using std::integral_constant;
 
-  // Division of labour between the four wavefronts of a chain:
-  //   read-out  (O^T = V^T A^T + S^T psi(q)^T)  split by TOKENS : wave w owns token tile w of the
-  //             chunk and contracts it against the whole state;
-  //   update    (S += psi(k)^T V)               split by SLOTS  : wave w owns slot tiles own_tile(w, .).
-  // Each wavefront therefore generates every psi element exactly once, holds only its share of
-  // the fp32 state in accumulators, and publishes a bf16 image of that share in LDS once per
-  // chunk for the others' read-out.
-  constexpr int kOwn = own_count(wave);
-
-  // own share of the running state S[i <-> slot tile own_tile(wave, i)][channel tile]:
+  // own share of the running state S[i <-> slot tile own_tile(w, i)][channel tile]:
   // lane <-> channel 16 et + col, regs <-> slot positions 4 grp + r
-  f32x4 S[kOwn][kETiles];
+  f32x4 S[kOwn][kCTiles];
 #pragma unroll
   for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-    for (int et = 0; et < kETiles; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int et = 0; et < kCTiles; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // normaliser state (updater kNormWave only), both as MFMA accumulators:
+  // K2[4 grp + r][col] (= K2[col][4 grp + r]) and K1[4 grp + r] (the same in every column)
+  f32x4 K2 = {0.f, 0.f, 0.f, 0.f};
+  f32x4 K1 = {0.f, 0.f, 0.f, 0.f};
 
   // token range of this workgroup and its slot in the workspace
   const int seg = blockIdx.z;
@@ -169,284 +495,204 @@ __device__ __forceinline__ void lin_prefill_chain(
 #pragma unroll
     for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-      for (int et = 0; et < kETiles; ++et)
-        S[i][et] = *reinterpret_cast<const f32x4*>(ws_mine + ((own_tile(wave, i) * kETiles + et) * 64 + lane) * 4);
+      for (int et = 0; et < kCTiles; ++et)
+        S[i][et] = *reinterpret_cast<const f32x4*>(ws_mine + ((own_tile(w, i) * kCTiles + et) * 64 + lane) * 4);
+    if constexpr (kNorm) {
+      K2 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK2 + lane * 4);
+      K1 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK1 + lane * 4);
+    }
   }
 
-  // operand of the normaliser channel: row/column 64 (col == 0) is all ones
-  const uint32_t one2 = col == 0 ? 0x3F803F80u : 0u;
-  const bf16x8 ones_op = __builtin_bit_cast(bf16x8, u32x4{one2, one2, one2, one2});
-  const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
   const uint32_t t8_keep = col < 8 ? 0xFFFFFFFFu : 0u;      // slot tile 8: pair products live in positions 0..7,
   const uint32_t t8_const = col == 8 ? 0x3F803F80u : 0u;    // the constant feature (bf16 1.0) in position 8
+  const bf16x8 ones8 = __builtin_bit_cast(bf16x8, u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
+  const int vt_j = col >> 2;
+  const int vt_lane = 128 * (4 * grp + vt_j) + 8 * (col & 3);
+  const int kt_lane = 32 * (4 * grp + vt_j) + 8 * (col & 3);
 
-  // Global loads of a chunk, issued one phase ahead of their use.  q (wave 0) / k (wave 1):
-  // 64 rows x 32 B, lane <-> row.  v: 64 rows x 128 B = 512 pieces of 16 B, two per thread:
-  // piece 256 i + tid <-> (token piece / 8, channels 8 (piece % 8) ..+8).
-  u32x4 pf_qk[2];
-  bf16x8 pf_v[2];
-  auto issue_loads = [&](int t0) {
-    const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
-    if (ntok == kChunk) {  // whole chunk (all but possibly the last): no zero fill, no bounds
-      if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
-        const __bf16* base = wave == 0 ? q + (long)(t0 + lane) * q_sl : k + (long)(t0 + lane) * k_sl;
-        const u32x4* src = reinterpret_cast<const u32x4*>(base);
-        pf_qk[0] = src[0];
-        pf_qk[1] = src[1];
+  // Direct global->LDS loads of a chunk.  The twelve wave-wide loads of a chunk (64 lanes x 16 B
+  // each, landing back to back in LDS) are dealt three to an updater: load id 0,1 = q rows 0..31,
+  // 32..63 (lane <-> row id*32 + lane/2, half lane%2); 2,3 = k likewise; 4 + j = v rows 8j..8j+7
+  // (lane <-> row 8j + lane/8, LDS piece lane%8 = global piece (lane%8) ^ 2((lane/8) & 3)).
+  // Rows past the end of the sequence are zero-filled instead.
+  auto issue_loads = [&](int tc, int slot_index) {
+    unsigned char* slot = lds + kOffData + slot_index * kDataBytes;
+    const int ntok = t_end - tc < kChunk ? t_end - tc : kChunk;
+    static_for<kLoadsPerUpdater>([&](auto II) {
+      constexpr int id = kLoadsPerUpdater * w + decltype(II)::value;
+      if constexpr (MODE == kModeDelta && id < 2) return;  // no read-out, no q
+      int row;
+      const __bf16* src;
+      unsigned char* dst;
+      if constexpr (id < 4) {
+        row = 32 * (id & 1) + (lane >> 1);
+        src = (id < 2 ? q + (long)(tc + row) * q_sl : k + (long)(tc + row) * k_sl) + 8 * (lane & 1);
+        dst = slot + (id < 2 ? 0 : kDataK) + 1024 * (id & 1);
+      } else {
+        row = 8 * (id - 4) + (lane >> 3);
+        src = v + (long)(tc + row) * v_sl + 8 * ((lane & 7) ^ (2 * ((lane >> 3) & 3)));
+        dst = slot + kDataV + 1024 * (id - 4);
       }
+      if (ntok == kChunk || row < ntok) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                         (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      } else {
+        *reinterpret_cast<u32x4*>(dst + 16 * lane) = u32x4{0, 0, 0, 0};
+      }
+    });
+  };
+  // bf16 image of own slot tile i (and, after the last one, of the normaliser state) into image
+  // buffer `buf`.  img[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes
+  // 0..7 come from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
+  auto publish_tile = [&](auto II, int buf) {
+    constexpr int i = decltype(II)::value;
+    constexpr int t = own_tile(w, i);
+    unsigned char* img = lds + kOffImg + buf * kImgBytes;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int piece = 256 * i + tid;
-        pf_v[i] = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + (piece >> 3)) * v_sl + 8 * (piece & 7));
-      }
-      return;
-    }
-    if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
-      const u32x4 z4 = {0, 0, 0, 0};
-      pf_qk[0] = pf_qk[1] = z4;
-      if (lane < ntok) {
-        const __bf16* base = wave == 0 ? q + (long)(t0 + lane) * q_sl : k + (long)(t0 + lane) * k_sl;
-        const u32x4* src = reinterpret_cast<const u32x4*>(base);
-        pf_qk[0] = src[0];
-        pf_qk[1] = src[1];
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int piece = 256 * i + tid;
-      const int tau = piece >> 3;
-      bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (tau < ntok) x = *reinterpret_cast<const bf16x8*>(v + (long)(t0 + tau) * v_sl + 8 * (piece & 7));
-      pf_v[i] = x;
+    for (int et = 0; et < kCTiles; ++et) {
+      const uint2 w2 = make_uint2(pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]));
+      *reinterpret_cast<uint2*>(img + (((t >> 1) * kCTiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
     }
   };
-  if (t_begin < t_end) issue_loads(t_begin);
-
-  // V^T operand tile (lane <-> channel 16 et + col, slots jj <-> tokens 32 s + 16 (jj/4) + 4 grp + jj%4)
-  // straight from the row-major V chunk in LDS with the transposing 64-bit LDS read: inside
-  // each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
-  // loaded, so source lane 4j + a fetches channels 4a..4a+3 of token j of the group's four.
-  const __bf16* vt_base = s_v + (4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
-  const __bf16* kt_base = s_k + (4 * grp + (col >> 2)) * kFeat + 4 * (col & 3);
-  auto load_vt = [&](int et, int s) -> bf16x8 {
-    const __bf16* p0 = vt_base + (32 * s) * kVStride + 16 * et;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kVStride));
-    const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    return __builtin_bit_cast(bf16x8, both);
+  auto publish_norm = [&](int buf) {
+    if constexpr (kNorm) {
+      // K2 as hi + lo bf16 operands: the accumulator registers K2[4 grp + r][col] are, by the
+      // symmetry of K2, the A operand K2[m = col][k = 4 grp + r] of the readers' MFMA
+      const uint32_t h0 = pack_bf16(K2[0], K2[1]), h1 = pack_bf16(K2[2], K2[3]);
+      const float l0 = K2[0] - bf16_bits_to_f32(h0 & 0xFFFFu), l1 = K2[1] - __builtin_bit_cast(float, h0 & 0xFFFF0000u);
+      const float l2 = K2[2] - bf16_bits_to_f32(h1 & 0xFFFFu), l3 = K2[3] - __builtin_bit_cast(float, h1 & 0xFFFF0000u);
+      unsigned char* k2 = lds + kOffK2 + buf * kK2Bytes;
+      *reinterpret_cast<uint2*>(k2 + lane * 8) = make_uint2(h0, h1);
+      *reinterpret_cast<uint2*>(k2 + 512 + lane * 8) = make_uint2(pack_bf16(l0, l1), pack_bf16(l2, l3));
+      if (col == 0) *reinterpret_cast<f32x4*>(lds + kOffK1 + buf * 64 + 16 * grp) = K1;
+    }
   };
 
-  for (int t0 = t_begin; t0 < t_end; t0 += kChunk) {
-    const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
-
-    // ---------------- stage the chunk (q, k, v rows as they come) into LDS ----------------
-    {
-      if constexpr (wave == 1 || (wave == 0 && MODE != kModeDelta)) {
-        u32x4* dst = reinterpret_cast<u32x4*>((wave == 0 ? s_q : s_k) + lane * kFeat);
-        dst[0] = pf_qk[0];
-        dst[1] = pf_qk[1];
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        const int piece = 256 * i + tid;
-        *reinterpret_cast<bf16x8*>(s_v + (piece >> 3) * kVStride + 8 * (piece & 7)) = pf_v[i];
-      }
+  // ---------------- prologue: chunks 0 and 1 requested, initial state published ----------------
+  if (t_begin < t_end) issue_loads(t_begin, 0);
+  if (t_begin + kChunk < t_end) issue_loads(t_begin + kChunk, 1);
+  if constexpr (MODE != kModeDelta) {
+    static_for<kOwn>([&](auto II) { publish_tile(II, 0); });
+    publish_norm(0);
+  }
+  // Chunk 0 has landed; chunk 1 may stay in flight when it is a whole chunk (a partial chunk may
+  // issue fewer loads than counted on, so then everything is awaited).
+  if (t_begin + 2 * kChunk <= t_end) {
+    if constexpr (MODE == kModeDelta && w == 0) {
+      barrier_updater<1>();
+    } else {
+      barrier_updater<3>();
     }
-    // ---------------- publish the bf16 image of the own share of the state ----------------
-    // s_sb[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes 0..7 come
-    // from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
-    // A wavefront that owns both slot tiles of a slab writes the operand in one 16-byte piece.
-    if constexpr (MODE != kModeDelta) {
-      static_for<kOwn>([&](auto II) {
-        constexpr int i = decltype(II)::value;
-        constexpr int t = own_tile(wave, i);
-        constexpr bool pair_lo = (t % 2 == 0) && (i + 1 < kOwn);
-        constexpr bool pair_hi = (t % 2 == 1) && (i > 0);
-        if constexpr (pair_lo) {
+  } else {
+    barrier_updater<0>();
+  }
+
+  int slot_i = 0, buf = 0;
+  for (int t0 = t_begin; t0 < t_end; t0 += kChunk, buf ^= 1, slot_i = slot_i == kRing - 1 ? 0 : slot_i + 1) {
+    const unsigned char* slot = lds + kOffData + slot_i * kDataBytes;
+    // operands of the first stage
+    bf16x8 kt0 = load_kt(slot, kt_lane, 0);
+    bf16x8 vt_s0[kCTiles], vt_s1[kCTiles];
 #pragma unroll
-          for (int et = 0; et < kETiles; ++et) {
-            const u32x4 w4 = {pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]),
-                              pack_bf16(S[i + 1][et][0], S[i + 1][et][1]), pack_bf16(S[i + 1][et][2], S[i + 1][et][3])};
-            *reinterpret_cast<u32x4*>(s_sb + (((t >> 1) * kETiles + et) * 64 + lane) * 16) = w4;
-          }
-        } else if constexpr (!pair_hi) {
+    for (int et = 0; et < kCTiles; ++et) vt_s0[et] = load_vt(slot, vt_lane, vt_j, et, 0);
+    // the rows of the chunk after the next are requested (their slot was last read one chunk ago)
+    const bool more2 = t0 + 2 * kChunk < t_end;
+    if (more2) issue_loads(t0 + 2 * kChunk, slot_i == 0 ? 2 : slot_i - 1);
+    BASED_STAGE_END();
+
+    // psi(k)^T tile (slot tile own_tile(w, i), current slab) from the raw k^T values of the slab;
+    // lane <-> slot position col, registers <-> the slab's 8 token slots
+    float k4[8];  // k / 4 of the slab's tokens (weights 1/16 on cross terms, 1/32 on squares, 1/4 on linear terms)
+    auto psi_k = [&](auto II) -> bf16x8 {
+      constexpr int t = own_tile(w, decltype(II)::value);
+      bf16x8 ak;
+      if constexpr (t == 9) {
+        ak = pack8(k4);
+      } else {
+        float f[8];
 #pragma unroll
-          for (int et = 0; et < kETiles; ++et) {
-            const uint2 w2 = make_uint2(pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]));
-            *reinterpret_cast<uint2*>(s_sb + (((t >> 1) * kETiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
+        for (int jj = 0; jj < 8; ++jj) {
+          if constexpr (t == 0) {
+            f[jj] = k4[jj] * k4[jj] * 0.5f;
+          } else {
+            f[jj] = row_ror<t>(k4[jj]) * k4[jj];  // tile 8: positions 8..15 are replaced below
           }
         }
-      });
-    }
-    __syncthreads();
-
-    // next chunk's global loads are in flight for the whole of this chunk's compute
-    if (t0 + kChunk < t_end) issue_loads(t0 + kChunk);
-
-    // ---------------- read-out of one own token tile: intra-chunk part, state part, store ----------------
-    auto readout = [&](auto NT) {
-      constexpr int nt = decltype(NT)::value;  // token tile within the chunk
-      // O^T[channel tile]: lane <-> token 16 nt + col, regs <-> channel 4 grp + r
-      f32x4 O[kETiles];
-#pragma unroll
-      for (int et = 0; et < kETiles; ++et) O[et] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-      // within the chunk: A^T = tril(1 + s + s^2/2)^T from a K=16 product of raw q, k; O^T += V^T A^T.
-      {
-        // the 16 features are exactly the contraction of a 16x16x16 MFMA: lane <-> (row, features 4 grp ..+3)
-        const s16x4 bq = *reinterpret_cast<const s16x4*>(s_q + (16 * nt + col) * kFeat + 4 * grp);
-        float p[4][4];  // [key tile][r]; tiles above the diagonal stay zero
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) p[mt][r] = 0.f;
-        static_for<nt + 1>([&](auto MT) {
-          constexpr int mt = decltype(MT)::value;
-          const s16x4 ka = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * grp);
-          const f32x4 a = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ka, bq, f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float pv = __builtin_fmaf(a[r], __builtin_fmaf(a[r], 1.0f / 32.0f, 0.25f), 1.0f);
-            if (mt == nt) pv = (4 * grp + r <= col) ? pv : 0.f;  // key <= query on the diagonal tile
-            p[mt][r] = pv;
-          }
-        });
-        static_for<nt / 2 + 1>([&](auto SS) {
-          constexpr int s = decltype(SS)::value;
-          const float pb[8] = {p[2 * s][0], p[2 * s][1], p[2 * s][2], p[2 * s][3],
-                               p[2 * s + 1][0], p[2 * s + 1][1], p[2 * s + 1][2], p[2 * s + 1][3]};
-          const bf16x8 bp = pack8(pb);
-#pragma unroll
-          for (int et = 0; et < 4; ++et) O[et] = mfma(load_vt(et, s), bp, O[et]);
-          O[4] = mfma(ones_op, bp, O[4]);
-        });
+        ak = pack8(f);
       }
-
-      // across chunks: O^T += S^T psi(q)^T with the state as it was before this chunk
-      {
-        // q of token 16 nt + col, rotated by 4 grp: qr[r] = q[(4 grp + r) mod 16]
-        float qr[16];
+      if constexpr (t == 8) {
+        // position 8 is the constant feature, 9..15 are unused.  The constant is also set
+        // for the zero rows that pad the last chunk: their v is zero, so they add nothing.
+        u32x4 x = __builtin_bit_cast(u32x4, ak);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const bf16x4 x = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + ((4 * grp + 4 * i) & 15));
-#pragma unroll
-          for (int c = 0; c < 4; ++c) qr[4 * i + c] = to_f32(x[c]);
-        }
-        const float fix8_0 = (grp == 2) ? 1.0f : 0.0f;  // slot (tile 8, position 8) = constant feature
-        static_for<5>([&](auto SG) {
-          constexpr int sg = decltype(SG)::value;  // slab of 32 slots = slot tiles 2 sg, 2 sg + 1
-          float f[8];
-          static_for<8>([&](auto JJ) {
-            constexpr int jj = decltype(JJ)::value;
-            constexpr int t = 2 * sg + jj / 4;  // slot tile
-            constexpr int c = jj % 4;           // position 4 grp + c
-            const float own = qr[c];
-            if constexpr (t == 0) {
-              f[jj] = own * own;
-            } else if constexpr (t <= 7) {
-              f[jj] = own * qr[(c - t) & 15];
-            } else if constexpr (t == 8) {
-              const float prod = own * qr[(c - 8) & 15];
-              f[jj] = low_half ? prod : (c == 0 ? fix8_0 : 0.0f);
-            } else {
-              f[jj] = own;
-            }
-          });
-          const bf16x8 bq = pack8(f);
-#pragma unroll
-          for (int et = 0; et < kETiles; ++et) {
-            const bf16x8 sa = *reinterpret_cast<const bf16x8*>(s_sb + ((sg * kETiles + et) * 64 + lane) * 16);
-            O[et] = mfma(sa, bq, O[et]);
-          }
-        });
+        for (int d = 0; d < 4; ++d) x[d] = (x[d] & t8_keep) | t8_const;
+        ak = __builtin_bit_cast(bf16x8, x);
       }
-
-      // normalise: the denominator sits in lane group 0, register 0 of channel tile 4
-      const float z = __shfl(O[4][0], col, 64);
-      const float inv = 1.0f / (z + eps);
-      // store: the 16 x 64 output tile goes through a wave-private LDS tile so that each lane
-      // writes 16 contiguous bytes and 8 lanes cover one 128-byte row (8-byte scattered stores
-      // cost four times the L2 write requests)
-      __bf16* so = s_o + wave * (16 * kOStride);
+      return ak;
+    };
+    auto unpack_k = [&](const bf16x8& kt) {
+      const u32x4 x = __builtin_bit_cast(u32x4, kt);
 #pragma unroll
-      for (int et = 0; et < 4; ++et) {
-        const uint32_t w0 = pack_bf16(O[et][0] * inv, O[et][1] * inv);
-        const uint32_t w1 = pack_bf16(O[et][2] * inv, O[et][3] * inv);
-        *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
-      }
-      // the tile is re-read below in another lane layout: order the wavefront's own LDS accesses
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-#pragma unroll
-      for (int hlf = 0; hlf < 2; ++hlf) {
-        const int row = 8 * hlf + (lane >> 3);
-        const u32x4 w4 = *reinterpret_cast<const u32x4*>(so + row * kOStride + 8 * (lane & 7));
-        const int tau = 16 * nt + row;
-        if (tau < ntok) *reinterpret_cast<u32x4*>(y + (long)(t0 + tau) * y_sl + 8 * (lane & 7)) = w4;
+      for (int d = 0; d < 4; ++d) {
+        k4[2 * d] = __builtin_bit_cast(float, x[d] << 16) * 0.25f;
+        k4[2 * d + 1] = __builtin_bit_cast(float, x[d] & 0xFFFF0000u) * 0.25f;
       }
     };
-    if constexpr (MODE != kModeDelta) readout(std::integral_constant<int, wave>{});
-    __builtin_amdgcn_sched_barrier(0);
+    unpack_k(kt0);
+    bf16x8 ak = psi_k(integral_constant<int, 0>{});
+    if constexpr (kNorm) {
+      K2 = mfma(kt0, kt0, K2);    // K2 += k^T k: the raw k^T tile is both operands (K2 is symmetric)
+      K1 = mfma(kt0, ones8, K1);  // K1 += k^T 1
+    }
+    BASED_STAGE_END();
 
-    // ---------------- state update: S += psi(k)^T V for the own slot tiles ----------------
-    {
-      // lane <-> slot position j = col; registers <-> the 8 token slots of a slab.  One slab of
-      // 32 tokens at a time, so that only its k values and V^T tiles are live.
+    // One slab of 32 tokens at a time; stage (s, i) runs the four MFMAs of slot tile i while the
+    // operand of the next tile is generated and the finished tile before it is published.
+    bf16x8 kt1 = load_kt(slot, kt_lane, 1);
+    const bool more1 = t0 + kChunk < t_end;
+    static_for<2 * kOwn>([&](auto ST) {
+      constexpr int st = decltype(ST)::value;
+      constexpr int s = st / kOwn, i = st % kOwn;
+      if constexpr (s == 0 && i == kOwn - 1) {
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        float kraw[8], k16[8];
-        bf16x8 vt[4];
-        {
-          // k^T (lane <-> feature col, slots <-> tokens) with the same transposing read as V^T
-          const __bf16* p0 = kt_base + (32 * s) * kFeat;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)p0);
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (s16x4 __attribute__((address_space(3)))*)(p0 + 16 * kFeat));
+        for (int et = 0; et < kCTiles; ++et) vt_s1[et] = load_vt(slot, vt_lane, vt_j, et, 1);
+      }
 #pragma unroll
-          for (int jj = 0; jj < 8; ++jj) {
-            const uint32_t bits = (uint32_t)(uint16_t)(jj < 4 ? lo[jj & 3] : hi[jj & 3]) << 16;
-            const float x = __builtin_bit_cast(float, bits);
-            kraw[jj] = x;
-            k16[jj] = x * (1.0f / 16.0f);
+      for (int et = 0; et < kCTiles; ++et) S[i][et] = mfma(ak, s == 0 ? vt_s0[et] : vt_s1[et], S[i][et]);
+      if constexpr (st + 1 < 2 * kOwn) {
+        if constexpr (i + 1 == kOwn) {  // the next stage starts slab 1
+          unpack_k(kt1);
+          if constexpr (kNorm) {
+            K2 = mfma(kt1, kt1, K2);
+            K1 = mfma(kt1, ones8, K1);
           }
         }
-#pragma unroll
-        for (int et = 0; et < 4; ++et) vt[et] = load_vt(et, s);
-        static_for<kOwn>([&](auto II) {
-          constexpr int i = decltype(II)::value;
-          constexpr int t = own_tile(wave, i);  // slot tile
-          float f[8];
-#pragma unroll
-          for (int jj = 0; jj < 8; ++jj) {
-            if constexpr (t == 0) {
-              f[jj] = kraw[jj] * k16[jj] * 0.5f;
-            } else if constexpr (t <= 7) {
-              f[jj] = row_ror<t>(kraw[jj]) * k16[jj];
-            } else if constexpr (t == 8) {
-              f[jj] = row_ror<8>(kraw[jj]) * k16[jj];  // positions 8..15 are replaced below
-            } else {
-              f[jj] = kraw[jj] * 0.25f;
-            }
-          }
-          bf16x8 ak = pack8(f);
-          if constexpr (t == 8) {
-            // position 8 is the constant feature, 9..15 are unused.  The constant is also set
-            // for the zero rows that pad the last chunk: their v is zero, and the count they
-            // add to the normaliser state is taken off when the state is written out.
-            u32x4 w = __builtin_bit_cast(u32x4, ak);
-#pragma unroll
-            for (int d = 0; d < 4; ++d) w[d] = (w[d] & t8_keep) | t8_const;
-            ak = __builtin_bit_cast(bf16x8, w);
-          }
-#pragma unroll
-          for (int et = 0; et < 4; ++et) S[i][et] = mfma(ak, vt[et], S[i][et]);
-          S[i][4] = mfma(ak, ones_op, S[i][4]);
-        });
-        __builtin_amdgcn_sched_barrier(0);
+        ak = psi_k(integral_constant<int, (i + 1) % kOwn>{});
+      }
+      if constexpr (MODE != kModeDelta && s == 1 && i > 0) {
+        if (more1) publish_tile(integral_constant<int, i - 1>{}, buf ^ 1);
+      }
+      interleave<4, ((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i > 0) ? 5 : 3)>();
+      BASED_STAGE_END();
+    });
+    // the rest of the state after this chunk, for the next chunk's readers
+    if constexpr (MODE != kModeDelta) {
+      if (more1) {
+        publish_tile(integral_constant<int, kOwn - 1>{}, buf ^ 1);
+        publish_norm(buf ^ 1);
       }
     }
-    __syncthreads();  // LDS is overwritten by the next chunk
+    // The next chunk's rows (requested one chunk ago) must have landed before anyone reads them;
+    // the loads requested in this iteration may stay in flight if they were a whole chunk's.
+    if (t0 + 3 * kChunk <= t_end) {
+      if constexpr (MODE == kModeDelta && w == 0) {
+        barrier_updater<1>();
+      } else {
+        barrier_updater<3>();
+      }
+    } else {
+      barrier_updater<0>();
+    }
   }
 
   // ---------------- a segment's contribution goes to the workspace as it sits in registers ----------------
@@ -454,27 +700,30 @@ __device__ __forceinline__ void lin_prefill_chain(
 #pragma unroll
     for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-      for (int et = 0; et < kETiles; ++et)
-        *reinterpret_cast<f32x4*>(ws_mine + ((own_tile(wave, i) * kETiles + et) * 64 + lane) * 4) = S[i][et];
+      for (int et = 0; et < kCTiles; ++et)
+        *reinterpret_cast<f32x4*>(ws_mine + ((own_tile(w, i) * kCTiles + et) * 64 + lane) * 4) = S[i][et];
+    if constexpr (kNorm) {
+      *reinterpret_cast<f32x4*>(ws_mine + kWsK2 + lane * 4) = K2;
+      *reinterpret_cast<f32x4*>(ws_mine + kWsK1 + lane * 4) = K1;
+    }
     return;
   }
 
   // ---------------- expand the 160-slot state into the (dv, 273) decode layout ----------------
-  // Sixteen channels at a time: the four wavefronts scatter their slot tiles of one channel
+  // Sixteen channels at a time: the four updaters scatter their slot tiles of one channel
   // tile into a 16 x 273 fp32 block in LDS (each cross slot lands on both (i, j) and (j, i),
   // with the factor that undoes the packing weights), and the block, which is contiguous in
-  // the decode state, leaves with coalesced 16-byte stores.
+  // the decode state, leaves with coalesced 16-byte stores by the whole workgroup.
   if (kv_state != nullptr && last_seg) {
-    const int pad_tokens = (kChunk - (t_end - t_begin) % kChunk) % kChunk;
-    float* blk = reinterpret_cast<float*>(s_sb);
-    static_assert(16 * kExp * 4 <= kSbBytes, "expansion block must fit in the state image buffer");
-    static_for<kETiles>([&](auto ET) {
+    float* blk = reinterpret_cast<float*>(lds + kOffImg);
+    static_assert(16 * kExp * 4 <= kImgBytes, "expansion block must fit in a state image buffer");
+    static_for<kCTiles>([&](auto ET) {
       constexpr int et = decltype(ET)::value;
       __syncthreads();  // the buffer is free (main loop done / previous block copied out)
       float* row = blk + col * kExp;
       static_for<kOwn>([&](auto II) {
         constexpr int i = decltype(II)::value;
-        constexpr int t = own_tile(wave, i);
+        constexpr int t = own_tile(w, i);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int j = 4 * grp + r;
@@ -490,8 +739,7 @@ __device__ __forceinline__ void lin_prefill_chain(
               row[1 + kFeat + 16 * j + j + 8] = x * (2.0f * kSqrt2);
               row[1 + kFeat + 16 * (j + 8) + j] = x * (2.0f * kSqrt2);
             } else if (j == 8) {
-              // constant feature; in the normaliser column it counted the padding rows too
-              row[0] = et == 4 ? x - (float)pad_tokens : x;
+              row[0] = x;  // constant feature
             }
           } else {
             row[1 + j] = x * 2.0f;
@@ -499,36 +747,44 @@ __device__ __forceinline__ void lin_prefill_chain(
         }
       });
       __syncthreads();
-      if constexpr (et < 4) {
-        f32x4* dst = reinterpret_cast<f32x4*>(kv_state + (bh * dv + 64 * eb + 16 * et) * kExp);
-        const f32x4* src = reinterpret_cast<const f32x4*>(blk);
-        for (int idx = tid; idx < 16 * kExp / 4; idx += 64 * kWavesPerChain) dst[idx] = src[idx];
-      } else if (eb == 0) {
-        // channel tile 4 carries the normaliser state in its column 0 (= row 0 of the block)
-        for (int idx = tid; idx < kExp; idx += 64 * kWavesPerChain) k_state[bh * kExp + idx] = blk[idx];
-      }
+      f32x4* dst = reinterpret_cast<f32x4*>(kv_state + (bh * dv + 64 * eb + 16 * et) * kExp);
+      const f32x4* src = reinterpret_cast<const f32x4*>(blk);
+      for (int idx = threadIdx.x; idx < 16 * kExp / 4; idx += kThreads) dst[idx] = src[idx];
     });
+    // normaliser state = sum of phi(k): the token count, K1/2 and K2/(4 sqrt 2), straight from fp32
+    if constexpr (kNorm) {
+      if (eb == 0) {
+        float* ks = k_state + bh * kExp;
+        if (lane == 0) ks[0] = (float)L;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (col == 0) ks[1 + 4 * grp + r] = K1[r] * 0.5f;
+          ks[1 + kFeat + 16 * (4 * grp + r) + col] = K2[r] * (0.25f / kSqrt2);
+        }
+      }
+    }
   }
 }
+#undef BASED_STAGE_END
 
 template <int MODE>
-__global__ __launch_bounds__(64 * kWavesPerChain, 3) void lin_prefill_mfma_kernel(
+__global__ __launch_bounds__(kThreads, 4) void lin_prefill_mfma_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
     long v_sl, long y_sb, long y_sh, long y_sl, float eps, float* __restrict__ ws, int seg_tokens, int n_seg) {
-  __shared__ __align__(16) __bf16 s_q[kChunk * kFeat];
-  __shared__ __align__(16) __bf16 s_k[kChunk * kFeat];
-  __shared__ __align__(16) __bf16 s_v[kChunk * kVStride];
-  __shared__ __align__(16) unsigned char s_sb[kSbBytes];
-  __shared__ __align__(16) __bf16 s_o[kWavesPerChain * 16 * kOStride];
-#define BASED_CHAIN_ARGS s_q, s_k, s_v, s_sb, s_o, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh, \
+  __shared__ __align__(16) unsigned char lds[kLdsBytes];
+#define BASED_CHAIN_ARGS lds, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh, \
                          k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, ws, seg_tokens, n_seg
   switch (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) {
-    case 0: lin_prefill_chain<0, MODE>(BASED_CHAIN_ARGS); break;
-    case 1: lin_prefill_chain<1, MODE>(BASED_CHAIN_ARGS); break;
-    case 2: lin_prefill_chain<2, MODE>(BASED_CHAIN_ARGS); break;
-    default: lin_prefill_chain<3, MODE>(BASED_CHAIN_ARGS); break;
+    case 0: lin_prefill_reader<0, MODE>(BASED_CHAIN_ARGS); break;
+    case 1: lin_prefill_reader<1, MODE>(BASED_CHAIN_ARGS); break;
+    case 2: lin_prefill_reader<2, MODE>(BASED_CHAIN_ARGS); break;
+    case 3: lin_prefill_reader<3, MODE>(BASED_CHAIN_ARGS); break;
+    case 4: lin_prefill_updater<0, MODE>(BASED_CHAIN_ARGS); break;
+    case 5: lin_prefill_updater<1, MODE>(BASED_CHAIN_ARGS); break;
+    case 6: lin_prefill_updater<2, MODE>(BASED_CHAIN_ARGS); break;
+    default: lin_prefill_updater<3, MODE>(BASED_CHAIN_ARGS); break;
   }
 #undef BASED_CHAIN_ARGS
 }
@@ -694,7 +950,7 @@ extern "C" BASED_API int based_linear_attn_prefill(
                     "linear_attn_prefill: bf16 strides must be multiples of 8 elements (16 bytes)");
     BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
                   "linear_attn_prefill: tensors must be 16-byte aligned");
-    dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(64 * kWavesPerChain);
+    dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(kThreads);
     hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFull>, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
                        q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, (float*)nullptr, 0, 1);
@@ -715,9 +971,9 @@ extern "C" BASED_API int based_linear_attn_prefill(
   return check_launch("linear_attn_prefill");
 }
 
-// Workgroup slots of one full wave of the MFMA prefill kernel on MI355X (256 CUs x 3 resident
+// Workgroup slots of one full wave of the MFMA prefill kernel on MI355X (256 CUs x 2 resident
 // workgroups); segment counts are chosen to fill about one such wave.
-static constexpr int64_t kPrefillSlots = 768;
+static constexpr int64_t kPrefillSlots = 512;
 
 extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, int64_t L, int64_t dv,
                                                         int io_dtype, int64_t* n_seg,
@@ -781,7 +1037,7 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   hipStream_t s = static_cast<hipStream_t>(stream);
   float* ws = static_cast<float*>(workspace);
   const int seg_tokens = (int)(seg_chunks * kChunk);
-  dim3 block(64 * kWavesPerChain);
+  dim3 block(kThreads);
   // pass 1: every segment but the last accumulates its own contribution to the state
   hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)(n_seg - 1)),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,

@@ -188,7 +188,7 @@ def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False,
                                                       ctypes.byref(ws_bytes)))
     if isinstance(split, int) and not isinstance(split, bool) and split > 1:
         n_seg = ctypes.c_int64(split)  # explicit segment count (tests)
-        ws_bytes = ctypes.c_int64(B * H * (dv // 64) * split * 10 * 5 * 64 * 4 * 4)
+        ws_bytes = ctypes.c_int64(B * H * (dv // 64) * split * _lib.PREFILL_SEGMENT_STATE_BYTES)
     args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
             kv_state.data_ptr() if return_state else None, k_state.data_ptr() if return_state else None,
             B, H, L, dv,

@@ -104,11 +104,13 @@ BASED_API int based_linear_attn_prefill(const void* q, const void* k, const void
  * it to accumulation order.
  *
  * based_linear_attn_prefill_plan reports the segment count this library would use for a shape
- * (1 = do not split) and the bytes of device workspace that count needs; the caller allocates
+ * (1 = do not split) and the bytes of device workspace that count needs
+ * (B*H*(dv/64) * n_seg * BASED_PREFILL_SEGMENT_STATE_BYTES); the caller allocates
  * the workspace (16-byte aligned; contents need no initialisation and are scratch afterwards)
  * and passes both to based_linear_attn_prefill_split.  n_seg <= 1 forwards to the unsplit
  * entry point.  bf16, dv in {64, 128} only.
  */
+#define BASED_PREFILL_SEGMENT_STATE_BYTES 43008 /* one (chain, segment) state in the workspace */
 BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, int64_t L, int64_t dv, int io_dtype,
                                              int64_t* n_seg, int64_t* workspace_bytes);
 BASED_API int based_linear_attn_prefill_split(const void* q, const void* k, const void* v, void* y,
@@ -127,7 +129,7 @@ BASED_API int based_linear_attn_prefill_split(const void* q, const void* k, cons
  * (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc).  The
  * per-segment states go to a static device array that is part of the library's code object:
  * BASED_STATIC_SCRATCH_BYTES (64 MiB) per GPU the library runs on, held until the process
- * ends.  B*H*(dv/64) * n_seg * 51,200 bytes must fit (every segment count that
+ * ends.  B*H*(dv/64) * n_seg * BASED_PREFILL_SEGMENT_STATE_BYTES must fit (every segment count that
  * based_linear_attn_prefill_plan returns does); larger requests return BASED_ERR_SHAPE and
  * launch nothing.  The first call on a device looks the array's address up (make it outside
  * a capture).  All calls on one GPU share the array: calls that overlap in time on one GPU

@@ -28,6 +28,12 @@ def test_header_symbols_are_exported_and_bound():
     assert set(_lib.SIGNATURES) == declared
 
 
+def test_header_constants_match_binding():
+    text = open(os.path.join(ROOT, "include", "based_hip.h")).read()
+    m = re.search(r"#define\s+BASED_PREFILL_SEGMENT_STATE_BYTES\s+(\d+)", text)
+    assert m and int(m.group(1)) == _lib.PREFILL_SEGMENT_STATE_BYTES
+
+
 def test_version_and_error_string():
     lib = _lib.lib()
     assert lib.based_hip_version() >= 1

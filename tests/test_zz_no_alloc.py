@@ -32,7 +32,7 @@ def _run(dev, B, H, L, dv, n_seg, seed, static):
     if static:
         _lib.check(lib.based_linear_attn_prefill_split_static(*args, stream))
     else:
-        ws_bytes = B * H * (dv // 64) * n_seg * 51200
+        ws_bytes = B * H * (dv // 64) * n_seg * _lib.PREFILL_SEGMENT_STATE_BYTES
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         _lib.check(lib.based_linear_attn_prefill_split(*args, ws.data_ptr(), ws_bytes, stream))
     torch.cuda.synchronize()
@@ -57,7 +57,7 @@ def test_static_scratch_rejects_oversized_requests(dev):
     lib = _lib.lib()
     buf = torch.zeros(64, dtype=torch.bfloat16, device=dev)
     p = buf.data_ptr()
-    # 4096 chains x 4 segments x 51,200 B = 800 MiB > 64 MiB: refused before anything is launched
+    # 4096 chains x 4 segments x 43,008 B = 672 MiB > 64 MiB: refused before anything is launched
     rc = lib.based_linear_attn_prefill_split_static(p, p, p, p, None, None, 256, 16, 4096, 64,
                                                     0, 0, 16, 0, 0, 16, 0, 0, 64, 0, 0, 64, 1e-12, 0, 4, None)
     assert rc == 1 and b"scratch" in lib.based_hip_last_error()
