@@ -85,13 +85,16 @@ __device__ __forceinline__ int slot_token(int s, int g, int jj) {
 }
 
 constexpr int kWavesPerChain = 4;   // wavefronts cooperating on one (batch, head, channel block)
-// Slot tiles of the state owned by wavefront w: {0,1,2}, {3,4,5}, {6,7}, {8,9}.  The wavefronts
-// with fewer slot tiles own the token tiles with more causal work (see the kernel), and
-// wavefront kNormWave also carries the normaliser state, which balances the MFMA count per
-// wavefront to 46..49 per chunk.
+// Slot tiles of the state owned by updater w, in the order it works through them: {0,1,2},
+// {4,5,3}, {6,7}, {8,9}.  The first two are always the two tiles of one 32-slot slab (their bf16
+// image leaves as one 16-byte piece per lane); updaters 0 and 1 share slab 1.  Updater
+// kNormWave also carries the normaliser state.
 __host__ __device__ constexpr int own_count(int wave) { return wave < 2 ? 3 : 2; }
-__host__ __device__ constexpr int own_tile(int wave, int i) { return (wave < 2 ? 3 * wave : 2 * wave + 2) + i; }
-static_assert(own_tile(3, own_count(3) - 1) == kFTiles - 1, "slot tiles must be covered exactly");
+__host__ __device__ constexpr int own_tile(int wave, int i) {
+  return wave == 0 ? i : wave == 1 ? (i < 2 ? 4 + i : 3) : 2 * wave + 2 + i;
+}
+static_assert(own_tile(3, own_count(3) - 1) == kFTiles - 1 && own_tile(1, 2) == 3 && own_tile(0, 2) == 2 &&
+                  own_tile(2, 0) == 6, "slot tiles must be covered exactly");
 constexpr int kNormWave = 2;
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
@@ -100,7 +103,10 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 // LDS of one workgroup (80,000 B: two workgroups per compute unit).
 //   data ring, 3 slots : the q, k, v rows of a chunk, written by direct global->LDS loads two
 //                        chunks ahead of their use (no registers, HBM latency fully covered).
-//                        q, k: 64 rows x 32 B.  v: 64 rows x 128 B whose eight 16-byte pieces
+//                        q, k: 64 rows x 32 B, the two 16-byte halves of a row swapped when
+//                        bit 2 of the row index is set (column reads of 8 bytes from 16
+//                        consecutive rows then hit 8 distinct bank pairs instead of 4).
+//                        v: 64 rows x 128 B whose eight 16-byte pieces
 //                        are stored at piece index p ^ 2 (row & 3), which makes the transposing
 //                        reads below bank-conflict free without row padding (a direct load
 //                        writes the 64 lanes' pieces back to back, so rows cannot be padded).
@@ -257,6 +263,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
   const bool low_half = grp < 2;  // feature positions 4 grp + c < 8
   const int vt_j = col >> 2;
   const int vt_lane = 128 * (4 * grp + vt_j) + 8 * (col & 3);
+  const int qk_swz = (col >> 2) & 1 ? 2 : 0;  // rows 16 x + col: bit 2 of the row index swaps the halves
   // output: after the lane-group exchange below a lane owns 2 x 8 consecutive channels of its token
   const int out_ch = (grp & 1) * 32 + 4 * (grp & 2);
   using std::integral_constant;
@@ -278,11 +285,12 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
 
       // ---- reads of the first stages ----
       // the 16 raw features are exactly the contraction of a 16x16x16 MFMA: lane <-> (row, features 4 grp ..+3)
-      const s16x4 bq = *reinterpret_cast<const s16x4*>(s_q + (16 * nt + col) * kFeat + 4 * grp);
+      // (feature chunk c of a row sits at 8-byte position c ^ qk_swz of that row)
+      const s16x4 bq = *reinterpret_cast<const s16x4*>(s_q + (16 * nt + col) * kFeat + 4 * (grp ^ qk_swz));
       bf16x4 qx[4];  // q of token 16 nt + col, rotated by 4 grp
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        qx[i] = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + ((4 * grp + 4 * i) & 15));
+        qx[i] = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + 4 * (((grp + i) & 3) ^ qk_swz));
       const unsigned char* k2 = lds + kOffK2 + buf * kK2Bytes;
       const s16x4 k2hi = *reinterpret_cast<const s16x4*>(k2 + lane * 8);
       const s16x4 k2lo = *reinterpret_cast<const s16x4*>(k2 + 512 + lane * 8);
@@ -290,7 +298,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       s16x4 ka[nt + 1];
 #pragma unroll
       for (int mt = 0; mt <= nt; ++mt)
-        ka[mt] = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * grp);
+        ka[mt] = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * (grp ^ qk_swz));
       auto img_load = [&](int sg, bf16x8 (&A)[kCTiles]) {
 #pragma unroll
         for (int et = 0; et < kCTiles; ++et)
@@ -508,11 +516,12 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   const bf16x8 ones8 = __builtin_bit_cast(bf16x8, u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u});
   const int vt_j = col >> 2;
   const int vt_lane = 128 * (4 * grp + vt_j) + 8 * (col & 3);
-  const int kt_lane = 32 * (4 * grp + vt_j) + 8 * (col & 3);
+  const int kt_lane = 32 * (4 * grp + vt_j) + 8 * ((col & 3) ^ (2 * (grp & 1)));  // rows 4 grp + j: bit 2 = grp & 1
 
   // Direct global->LDS loads of a chunk.  The twelve wave-wide loads of a chunk (64 lanes x 16 B
   // each, landing back to back in LDS) are dealt three to an updater: load id 0,1 = q rows 0..31,
-  // 32..63 (lane <-> row id*32 + lane/2, half lane%2); 2,3 = k likewise; 4 + j = v rows 8j..8j+7
+  // 32..63 (lane <-> row id*32 + lane/2, LDS half lane%2 = global half (lane%2) ^ bit 2 of the
+  // row); 2,3 = k likewise; 4 + j = v rows 8j..8j+7
   // (lane <-> row 8j + lane/8, LDS piece lane%8 = global piece (lane%8) ^ 2((lane/8) & 3)).
   // Rows past the end of the sequence are zero-filled instead.
   auto issue_loads = [&](int tc, int slot_index) {
@@ -526,7 +535,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       unsigned char* dst;
       if constexpr (id < 4) {
         row = 32 * (id & 1) + (lane >> 1);
-        src = (id < 2 ? q + (long)(tc + row) * q_sl : k + (long)(tc + row) * k_sl) + 8 * (lane & 1);
+        src = (id < 2 ? q + (long)(tc + row) * q_sl : k + (long)(tc + row) * k_sl) + 8 * ((lane & 1) ^ ((lane >> 3) & 1));
         dst = slot + (id < 2 ? 0 : kDataK) + 1024 * (id & 1);
       } else {
         row = 8 * (id - 4) + (lane >> 3);
@@ -541,17 +550,30 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       }
     });
   };
-  // bf16 image of own slot tile i (and, after the last one, of the normaliser state) into image
-  // buffer `buf`.  img[slab][channel tile][lane] is the 16-byte A operand of the read-out: bytes
-  // 0..7 come from slot tile 2 slab (regs r = 0..3), bytes 8..15 from slot tile 2 slab + 1.
-  auto publish_tile = [&](auto II, int buf) {
-    constexpr int i = decltype(II)::value;
-    constexpr int t = own_tile(w, i);
+  // bf16 image of the own share of the state into image buffer `buf`.  img[slab][channel tile]
+  // [lane] is the 16-byte A operand of the read-out: bytes 0..7 come from slot tile 2 slab (regs
+  // r = 0..3), bytes 8..15 from slot tile 2 slab + 1.  The first two own tiles make up one slab
+  // and leave as whole 16-byte pieces; a third tile fills its half of the shared slab.
+  auto publish_pair = [&](int buf) {
+    constexpr int t = own_tile(w, 0);
+    static_assert(t % 2 == 0 && own_tile(w, 1) == t + 1, "first two own tiles = one slab");
     unsigned char* img = lds + kOffImg + buf * kImgBytes;
 #pragma unroll
     for (int et = 0; et < kCTiles; ++et) {
-      const uint2 w2 = make_uint2(pack_bf16(S[i][et][0], S[i][et][1]), pack_bf16(S[i][et][2], S[i][et][3]));
-      *reinterpret_cast<uint2*>(img + (((t >> 1) * kCTiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
+      const u32x4 w4 = {pack_bf16(S[0][et][0], S[0][et][1]), pack_bf16(S[0][et][2], S[0][et][3]),
+                        pack_bf16(S[1][et][0], S[1][et][1]), pack_bf16(S[1][et][2], S[1][et][3])};
+      *reinterpret_cast<u32x4*>(img + (((t >> 1) * kCTiles + et) * 64 + lane) * 16) = w4;
+    }
+  };
+  auto publish_single = [&](int buf) {
+    if constexpr (kOwn == 3) {
+      constexpr int t = own_tile(w, 2);
+      unsigned char* img = lds + kOffImg + buf * kImgBytes;
+#pragma unroll
+      for (int et = 0; et < kCTiles; ++et) {
+        const uint2 w2 = make_uint2(pack_bf16(S[2][et][0], S[2][et][1]), pack_bf16(S[2][et][2], S[2][et][3]));
+        *reinterpret_cast<uint2*>(img + (((t >> 1) * kCTiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
+      }
     }
   };
   auto publish_norm = [&](int buf) {
@@ -572,7 +594,8 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   if (t_begin < t_end) issue_loads(t_begin, 0);
   if (t_begin + kChunk < t_end) issue_loads(t_begin + kChunk, 1);
   if constexpr (MODE != kModeDelta) {
-    static_for<kOwn>([&](auto II) { publish_tile(II, 0); });
+    publish_pair(0);
+    publish_single(0);
     publish_norm(0);
   }
   // Chunk 0 has landed; chunk 1 may stay in flight when it is a whole chunk (a partial chunk may
@@ -669,16 +692,17 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
         }
         ak = psi_k(integral_constant<int, (i + 1) % kOwn>{});
       }
-      if constexpr (MODE != kModeDelta && s == 1 && i > 0) {
-        if (more1) publish_tile(integral_constant<int, i - 1>{}, buf ^ 1);
+      if constexpr (MODE != kModeDelta && s == 1 && i == 2) {
+        if (more1) publish_pair(buf ^ 1);  // both tiles of the slab are final
       }
-      interleave<4, ((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i > 0) ? 5 : 3)>();
+      interleave<4, ((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i == 2) ? 6 : 3)>();
       BASED_STAGE_END();
     });
     // the rest of the state after this chunk, for the next chunk's readers
     if constexpr (MODE != kModeDelta) {
       if (more1) {
-        publish_tile(integral_constant<int, kOwn - 1>{}, buf ^ 1);
+        if constexpr (kOwn == 2) publish_pair(buf ^ 1);
+        publish_single(buf ^ 1);
         publish_norm(buf ^ 1);
       }
     }
