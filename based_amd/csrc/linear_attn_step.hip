@@ -18,10 +18,6 @@ constexpr int kTabLen = 280;                     // 273 + 3 wrap entries, padded
 constexpr int kRowsPerWave = 16;
 constexpr int kVec4PerWave = kRowsPerWave * kExp / 4;  // 1092
 constexpr int kIters = (kVec4PerWave + kWave - 1) / kWave;  // 18
-// All 18 loads of a wavefront are issued before the first is consumed (18 KB in flight per
-// wavefront); measured on MI355X this beats smaller batches, and plain loads/stores beat
-// non-temporal ones for this read-modify-write stream.
-constexpr int kBatch = kIters;
 
 __device__ __forceinline__ float phi_elem(const float* x, int f) {
   // TaylorExp element f of a 16-vector x: [1 | x/2 | x_i x_j / (4 sqrt 2)], row-major i,j.
@@ -47,6 +43,19 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const long bh = blockIdx.x;
   const int b = (int)(bh / H), h = (int)(bh % H);
+
+  // State rows [16*wave, 16*wave+16) of this (b, h).  All of the wavefront's state is requested
+  // before anything else: the loads depend on nothing but the workgroup's position, so the
+  // HBM round trip runs under the set-up below (feature tables, two barriers).  The state is
+  // touched exactly once per step and the whole batch's state is far larger than any cache:
+  // non-temporal loads and stores keep it from displacing anything.
+  f32x4* base = reinterpret_cast<f32x4*>(kv_state + (bh * dv + (long)kRowsPerWave * wave) * kExp);
+  f32x4 d[kIters];
+#pragma unroll
+  for (int t = 0; t < kIters; ++t) {
+    const int j = t * kWave + lane;
+    if (t < kIters - 1 || j < kVec4PerWave) d[t] = __builtin_nontemporal_load(base + j);
+  }
 
   if (tid < 2 * kFeat) {
     const int which = tid >> 4, i = tid & 15;
@@ -87,54 +96,40 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
     vrow[r] = __builtin_bit_cast(
         float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, s_v[kRowsPerWave * wave + r])));
 
-  f32x4* base = reinterpret_cast<f32x4*>(kv_state + (bh * dv + (long)kRowsPerWave * wave) * kExp);
-
   float acc[kRowsPerWave];
 #pragma unroll
   for (int r = 0; r < kRowsPerWave; ++r) acc[r] = 0.0f;
 
   const int e_lane = 4 * lane;
 #pragma unroll
-  for (int t0 = 0; t0 < kIters; t0 += kBatch) {
-    f32x4 d[kBatch];
+  for (int t = 0; t < kIters; ++t) {
+    const int j = t * kWave + lane;
+    const int rb = (256 * t) / kExp;              // first row touched by this iteration
+    const int bnd = (rb + 1) * kExp - 256 * t;    // local element index where row rb+1 starts
+    const bool two_rows = bnd < 256;
+    if (t < kIters - 1 || j < kVec4PerWave) {
+      const bool lane_hi = two_rows && (e_lane >= bnd);
+      const int f0 = (256 * t - rb * kExp) + e_lane - (lane_hi ? kExp : 0);
+      const int m = f0 & 3;
+      const f32x4 pk = *reinterpret_cast<const f32x4*>(&s_tab[0][m][f0 - m]);
+      const f32x4 pq = *reinterpret_cast<const f32x4*>(&s_tab[1][m][f0 - m]);
+      const float v_lo = vrow[rb];
+      const float v_hi = vrow[rb + 1 < kRowsPerWave ? rb + 1 : rb];
+      f32x4 x = d[t];
+      float s_lo = 0.0f, s_hi = 0.0f;
 #pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const int t = t0 + u;
-      const int j = t * kWave + lane;
-      if (t < kIters - 1 || j < kVec4PerWave) d[u] = base[j];
-    }
-#pragma unroll
-    for (int u = 0; u < kBatch; ++u) {
-      const int t = t0 + u;
-      const int j = t * kWave + lane;
-      const int rb = (256 * t) / kExp;              // first row touched by this iteration
-      const int bnd = (rb + 1) * kExp - 256 * t;    // local element index where row rb+1 starts
-      const bool two_rows = bnd < 256;
-      if (t < kIters - 1 || j < kVec4PerWave) {
-        const bool lane_hi = two_rows && (e_lane >= bnd);
-        const int f0 = (256 * t - rb * kExp) + e_lane - (lane_hi ? kExp : 0);
-        const int m = f0 & 3;
-        const f32x4 pk = *reinterpret_cast<const f32x4*>(&s_tab[0][m][f0 - m]);
-        const f32x4 pq = *reinterpret_cast<const f32x4*>(&s_tab[1][m][f0 - m]);
-        const float v_lo = vrow[rb];
-        const float v_hi = vrow[rb + 1 < kRowsPerWave ? rb + 1 : rb];
-        f32x4 x = d[u];
-        float s_lo = 0.0f, s_hi = 0.0f;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const bool hi = two_rows && (e_lane + c >= bnd);
-          const float nv = __builtin_fmaf(hi ? v_hi : v_lo, pk[c], x[c]);
-          x[c] = nv;
-          const float p = pq[c] * nv;
-          s_lo += hi ? 0.0f : p;
-          s_hi += hi ? p : 0.0f;
-        }
-        base[j] = x;
-        acc[rb] += s_lo;
-        if (two_rows && rb + 1 < kRowsPerWave) acc[rb + 1] += s_hi;
+      for (int c = 0; c < 4; ++c) {
+        const bool hi = two_rows && (e_lane + c >= bnd);
+        const float nv = __builtin_fmaf(hi ? v_hi : v_lo, pk[c], x[c]);
+        x[c] = nv;
+        const float p = pq[c] * nv;
+        s_lo += hi ? 0.0f : p;
+        s_hi += hi ? p : 0.0f;
       }
+      __builtin_nontemporal_store(x, base + j);
+      acc[rb] += s_lo;
+      if (two_rows && rb + 1 < kRowsPerWave) acc[rb + 1] += s_hi;
     }
-    __builtin_amdgcn_sched_barrier(0);  // keep the next batch's loads behind this batch's stores
   }
 
   // Transposing butterfly: 16 per-lane row sums -> lane l holds the total of row l >> 2.

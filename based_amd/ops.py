@@ -26,6 +26,30 @@ def _stream_ptr(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _on_device:
+    """Enters `torch.cuda.device(dev)` only when dev is not already current (entering the context
+    costs microseconds, which matters for single-token steps)."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev: torch.device):
+        self.ctx = None if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
+# Argument checks of the single-token entry points are done once per distinct combination of
+# shapes, strides, dtypes and device (a decode loop presents the same combination every step).
+_CHECKED: dict = {}
+
+
 def _require_cuda(*ts: torch.Tensor) -> None:
     dev = ts[0].device
     for t in ts:
@@ -35,28 +59,42 @@ def _require_cuda(*ts: torch.Tensor) -> None:
             raise ValueError("all tensors must live on the same device")
 
 
-def linear_attn_step(q, k, v, kv_state, k_state, eps: float = 1e-12) -> torch.Tensor:
+def linear_attn_step(q, k, v, kv_state, k_state, eps: float = 1e-12, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One decode step.  q, k: (B, H, 1, 16) raw; v: (B, H, 1, dv); kv_state (B,H,1,dv,273)
-    and k_state (B,H,1,1,273) fp32 contiguous, updated in place.  Returns y (B, H, 1, dv)."""
-    _require_cuda(q, k, v, kv_state, k_state)
-    B, H, l, d = q.shape
-    assert l == 1, f"q.shape is {tuple(q.shape)} but should be ({B}, {H}, 1, {d})"
+    and k_state (B,H,1,1,273) fp32 contiguous, updated in place.  Returns y (B, H, 1, dv)
+    (written into `out` when given)."""
+    key = ("lin_step", q.shape, q.stride(), k.shape, k.stride(), v.shape, v.stride(), kv_state.shape, kv_state.stride(),
+           k_state.shape, k_state.stride(), q.dtype, k.dtype, v.dtype, kv_state.dtype, k_state.dtype, q.device,
+           k.device, v.device, kv_state.device, k_state.device)
+    if key not in _CHECKED:
+        _require_cuda(q, k, v, kv_state, k_state)
+        B, H, l, d = q.shape
+        assert l == 1, f"q.shape is {tuple(q.shape)} but should be ({B}, {H}, 1, {d})"
+        dv = v.shape[-1]
+        if d != FEATURE_DIM or k.shape != q.shape or v.shape[:3] != q.shape[:3]:
+            raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+        if kv_state.dtype != torch.float32 or k_state.dtype != torch.float32:
+            raise ValueError("decode states must be float32")
+        if tuple(kv_state.shape) != (B, H, 1, dv, EXPANDED_DIM) or tuple(k_state.shape) != (B, H, 1, 1, EXPANDED_DIM):
+            raise ValueError(f"bad state shapes {tuple(kv_state.shape)} {tuple(k_state.shape)}")
+        if not (kv_state.is_contiguous() and k_state.is_contiguous()):
+            raise ValueError("decode states must be contiguous")
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ValueError("q, k, v must share a dtype")
+        for t in (q, k, v):
+            if t.stride(-1) != 1:
+                raise ValueError("innermost dimension must be contiguous")
+        _dtype_code(q)
+        _CHECKED[key] = True
+    B, H, _, _ = q.shape
     dv = v.shape[-1]
-    if d != FEATURE_DIM or k.shape != q.shape or v.shape[:3] != q.shape[:3]:
-        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
-    if kv_state.dtype != torch.float32 or k_state.dtype != torch.float32:
-        raise ValueError("decode states must be float32")
-    if tuple(kv_state.shape) != (B, H, 1, dv, EXPANDED_DIM) or tuple(k_state.shape) != (B, H, 1, 1, EXPANDED_DIM):
-        raise ValueError(f"bad state shapes {tuple(kv_state.shape)} {tuple(k_state.shape)}")
-    if not (kv_state.is_contiguous() and k_state.is_contiguous()):
-        raise ValueError("decode states must be contiguous")
-    if not (q.dtype == k.dtype == v.dtype):
-        raise ValueError("q, k, v must share a dtype")
-    for t in (q, k, v):
-        if t.stride(-1) != 1:
-            raise ValueError("innermost dimension must be contiguous")
-    y = torch.empty(B, H, 1, dv, dtype=q.dtype, device=q.device)
-    with torch.cuda.device(q.device):
+    if out is None:
+        y = torch.empty(B, H, 1, dv, dtype=q.dtype, device=q.device)
+    else:
+        y = out
+        if tuple(y.shape) != (B, H, 1, dv) or y.dtype != q.dtype or y.device != q.device or y.stride(-1) != 1:
+            raise ValueError(f"out must be a ({B}, {H}, 1, {dv}) {q.dtype} tensor on {q.device}")
+    with _on_device(q.device):
         _lib.check(_lib.lib().based_linear_attn_step(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), kv_state.data_ptr(), k_state.data_ptr(), y.data_ptr(),
             B, H, dv,
@@ -80,13 +118,14 @@ def _rope_tables(rope, device, need_rows):
     return cos.data_ptr(), sin.data_ptr(), cos.shape[0]
 
 
-def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=None, kv_cache=None) -> torch.Tensor:
+def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=None, kv_cache=None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window causal attention.  q, k, v: (B, L, H, 64) bf16 (any strides with the
     last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i].
     rope: None or (cos, sin) fp32 (n_pos >= L, 32) tables; q and k are then rotated in the kernel
     (non-interleaved rotary over the whole head, positions 0..L-1).
     kv_cache: None or a (B, max_seqlen >= L, 2, H, 64) bf16 cache whose rows 0..L-1 receive the
-    (rotated) k and v."""
+    (rotated) k and v.  out: None or a (B, L, H, 64) tensor (last dim contiguous) to write into."""
     _require_cuda(q, k, v)
     B, L, H, D = q.shape
     if D != 64 or k.shape != q.shape or v.shape != q.shape:
@@ -106,8 +145,13 @@ def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=N
         kc, vc = kv_cache[:, :, 0], kv_cache[:, :, 1]
         kc_ptr, vc_ptr = kc.data_ptr(), vc.data_ptr()
         c_strides, max_seqlen = (kc.stride(0), kc.stride(1), kc.stride(2)), kv_cache.shape[1]
-    o = torch.empty(B, L, H, D, dtype=q.dtype, device=q.device)
-    with torch.cuda.device(q.device):
+    if out is None:
+        o = torch.empty(B, L, H, D, dtype=q.dtype, device=q.device)
+    else:
+        o = out
+        if tuple(o.shape) != (B, L, H, D) or o.dtype != q.dtype or o.device != q.device or o.stride(-1) != 1:
+            raise ValueError(f"out must be a ({B}, {L}, {H}, {D}) {q.dtype} tensor on {q.device}")
+    with _on_device(q.device):
         _lib.check(_lib.lib().based_swa_prefill(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
@@ -117,23 +161,32 @@ def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=N
     return o
 
 
-def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None, rope=None) -> torch.Tensor:
+def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None, rope=None,
+             out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Decode step.  q, k_new, v_new: (B, 1, H, 64) bf16; kv_cache (B, max_seqlen, 2, H, 64)
     bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.
     pos: int (same for the whole batch) or an int32 device tensor of B positions.
-    rope: None or (cos, sin) tables as for swa_prefill: q and k_new are rotated at `pos` first."""
-    _require_cuda(q, k_new, v_new, kv_cache)
-    B, one, H, D = q.shape
-    if one != 1 or D != 64 or k_new.shape != q.shape or v_new.shape != q.shape:
-        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k_new.shape)} v{tuple(v_new.shape)}")
-    if kv_cache.dim() != 5 or kv_cache.shape[0] < B or kv_cache.shape[2] != 2 or tuple(kv_cache.shape[3:]) != (H, D):
-        raise ValueError(f"bad cache shape {tuple(kv_cache.shape)}")
-    if kv_cache.dtype != q.dtype or kv_cache.stride(-1) != 1:
-        raise ValueError("cache must share q's dtype and have a contiguous last dim")
-    for t in (q, k_new, v_new):
-        if t.stride(-1) != 1:
-            raise ValueError("innermost dimension must be contiguous")
-    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    rope: None or (cos, sin) tables as for swa_prefill: q and k_new are rotated at `pos` first.
+    out: None or a (B, 1, H, 64) tensor (last dim contiguous) to write into."""
+    key = ("swa_step", q.shape, q.stride(), k_new.shape, k_new.stride(), v_new.shape, v_new.stride(), kv_cache.shape,
+           kv_cache.stride(), q.dtype, k_new.dtype, v_new.dtype, kv_cache.dtype, q.device, k_new.device, v_new.device,
+           kv_cache.device)
+    if key not in _CHECKED:
+        _require_cuda(q, k_new, v_new, kv_cache)
+        B, one, H, D = q.shape
+        if one != 1 or D != 64 or k_new.shape != q.shape or v_new.shape != q.shape:
+            raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k_new.shape)} v{tuple(v_new.shape)}")
+        if kv_cache.dim() != 5 or kv_cache.shape[0] < B or kv_cache.shape[2] != 2 or tuple(kv_cache.shape[3:]) != (H, D):
+            raise ValueError(f"bad cache shape {tuple(kv_cache.shape)}")
+        if kv_cache.dtype != q.dtype or kv_cache.stride(-1) != 1:
+            raise ValueError("cache must share q's dtype and have a contiguous last dim")
+        for t in (q, k_new, v_new):
+            if t.stride(-1) != 1:
+                raise ValueError("innermost dimension must be contiguous")
+        _dtype_code(q)
+        _CHECKED[key] = True
+    B, _, H, D = q.shape
+    scale = 0.125 if scale is None else float(scale)  # 1 / sqrt(64)
     if isinstance(pos, torch.Tensor):
         if pos.dtype != torch.int32 or not pos.is_cuda or pos.numel() < B or not pos.is_contiguous():
             raise ValueError("cache_seqlens must be a contiguous int32 device tensor with B entries")
@@ -142,15 +195,22 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
     else:
         seq_ptr, pos_host = None, int(pos)
         cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, pos_host + 1)
-    o = torch.empty(B, 1, H, D, dtype=q.dtype, device=q.device)
-    kc, vc = kv_cache[:, :, 0], kv_cache[:, :, 1]
-    with torch.cuda.device(q.device):
+    if out is None:
+        o = torch.empty(B, 1, H, D, dtype=q.dtype, device=q.device)
+    else:
+        o = out
+        if tuple(o.shape) != (B, 1, H, D) or o.dtype != q.dtype or o.device != q.device or o.stride(-1) != 1:
+            raise ValueError(f"out must be a ({B}, 1, {H}, {D}) {q.dtype} tensor on {q.device}")
+    c_sb, c_st, _, c_sh, _ = kv_cache.stride()
+    kc_ptr = kv_cache.data_ptr()
+    vc_ptr = kc_ptr + kv_cache.stride(2) * kv_cache.element_size()
+    with _on_device(q.device):
         _lib.check(_lib.lib().based_swa_step(
-            q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc.data_ptr(), vc.data_ptr(), o.data_ptr(),
+            q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
             seq_ptr, pos_host, B, H, kv_cache.shape[1],
             q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
             v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
-            kc.stride(0), kc.stride(1), kc.stride(2),
+            c_sb, c_st, c_sh,
             int(w_left), scale, cos_ptr, sin_ptr, n_pos, _dtype_code(q), _stream_ptr(q)))
     return o
 
@@ -195,7 +255,7 @@ def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
             v.stride(0), v.stride(1), v.stride(2), y.stride(0), y.stride(1), y.stride(2),
             float(eps), _dtype_code(q))
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if n_seg.value > 1:
             # scratch for the per-segment states; torch's caching allocator makes this cheap
             ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q.device)
@@ -235,7 +295,7 @@ def gated_conv_prefill(u, weight, bias=None, state=None) -> torch.Tensor:
             raise ValueError(f"state must be a contiguous ({B}, {D}, {K}) tensor, got {tuple(state.shape)}")
         state_code = _dtype_code(state)
     y = torch.empty(B, L, D, dtype=u.dtype, device=u.device)
-    with torch.cuda.device(u.device):
+    with _on_device(u.device):
         _lib.check(_lib.lib().based_gated_conv_prefill(
             u.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(),
             state.data_ptr() if state is not None else None, B, L, D, K,
@@ -268,7 +328,7 @@ def gated_conv_step(u, state, weight, bias=None) -> torch.Tensor:
         _require_cuda(u, bias)
         bias = bias.contiguous()
     y = torch.empty(B, D, dtype=u.dtype, device=u.device)
-    with torch.cuda.device(u.device):
+    with _on_device(u.device):
         _lib.check(_lib.lib().based_gated_conv_step(
             u2d.data_ptr(), state.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
             y.data_ptr(), B, D, K, u2d.stride(0), y.stride(0), _dtype_code(u), _dtype_code(state), _stream_ptr(u)))
@@ -304,7 +364,7 @@ def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool 
     y = torch.empty(rows, D, dtype=x.dtype, device=x.device)
     out = torch.empty(rows, D, dtype=res_dtype, device=x.device) if want_residual else None
     res_code = _lib.BASED_F32 if res_dtype == torch.float32 else _lib.BASED_BF16
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _lib.check(_lib.lib().based_add_rms_norm(
             x2.data_ptr(), r2.data_ptr() if r2 is not None else None, weight.data_ptr(), y.data_ptr(),
             out.data_ptr() if out is not None else None, rows, D, x2.stride(0),
@@ -324,7 +384,7 @@ def swiglu(u) -> torch.Tensor:
     if u2.stride(-1) != 1:
         u2 = u2.contiguous()
     out = torch.empty(u2.shape[0], F, dtype=u.dtype, device=u.device)
-    with torch.cuda.device(u.device):
+    with _on_device(u.device):
         _lib.check(_lib.lib().based_swiglu(u2.data_ptr(), out.data_ptr(), u2.shape[0], F, u2.stride(0), out.stride(0),
                                            _dtype_code(u), _stream_ptr(u)))
     return out.view(*u.shape[:-1], F)

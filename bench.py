@@ -7,7 +7,9 @@ Headline workload (`value`): the recurrent decode step of Taylor linear attentio
 B=128, H=16, dv=64 — fp32 kv_state (128,16,1,64,273) + k_state, initialised from a seeded
 512-token prefill, bf16 q/k/v ~ N(0,1), K consecutive single-token steps.  One "step" is
 one kernel launch over the whole batch; value = B / time-per-step (tokens/s, one layer).
-Inputs and state are resident in HBM before the timed region.
+Inputs and state are resident in HBM before the timed region.  The HBM-bound workloads are
+timed cold (rotating over several independent state / input sets, working set well beyond the
+256 MB last-level cache) and warm (one set); `value` and `roofline` use the slower of the two.
 
 The same JSON line also carries, as secondary objects, the linear-attention prefill at
 L=4096 (tokens/s and fraction of bf16 MFMA peak) and the sliding-window attention prefill +
@@ -69,7 +71,12 @@ def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0):
     return e0.elapsed_time(e1) / steps, wall
 
 
-def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512):
+def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4):
+    """Recurrent decode step.  Timed twice: COLD over `n_sets` independent (kv_state, k_state) sets
+    visited in turn (n_sets x 145 MB at B=128, dv=64: more than the 256 MB last-level cache, and what
+    the linear-attention layers of a stack do per token: every layer has its own state), and WARM
+    on one set updated in place every step (145 MB: may be served from the last-level cache).
+    The roofline figure is the lower of the two."""
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(0)
     # state from a seeded prefill (same kernels; q only shapes the outputs, not the state)
@@ -77,6 +84,7 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512)
     vp = torch.randn(B, H, prefill_len, dv, generator=g).bfloat16().to(dev)
     _, kv_state, k_state = ops.linear_attn_prefill(kp, kp, vp, return_state=True)
     del kp, vp
+    states = [(kv_state, k_state)] + [(kv_state.clone(), k_state.clone()) for _ in range(n_sets - 1)]
     n_in = 8  # distinct pre-generated inputs cycled through the steps
     qs = [torch.randn(B, H, 1, 16, generator=g).bfloat16().to(dev) for _ in range(n_in)]
     ks = [torch.randn(B, H, 1, 16, generator=g).bfloat16().to(dev) for _ in range(n_in)]
@@ -87,30 +95,42 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512)
     lib = _lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
     args = [(qs[i].data_ptr(), ks[i].data_ptr(), vs[i].data_ptr()) for i in range(n_in)]
+    st_ptrs = [(a.data_ptr(), b.data_ptr()) for a, b in states]
     it = [0]
 
-    def step():
-        a = args[it[0] % n_in]
-        it[0] += 1
-        rc = lib.based_linear_attn_step(a[0], a[1], a[2], kv_state.data_ptr(), k_state.data_ptr(), y.data_ptr(),
-                                        B, H, dv, H * 16, 16, H * 16, 16, H * dv, dv, H * dv, dv,
-                                        1e-12, 0, stream)
-        if rc:
-            _lib.check(rc)
+    def make_step(sets):
+        def step():
+            a = args[it[0] % n_in]
+            st = st_ptrs[it[0] % sets]
+            it[0] += 1
+            rc = lib.based_linear_attn_step(a[0], a[1], a[2], st[0], st[1], y.data_ptr(),
+                                            B, H, dv, H * 16, 16, H * 16, 16, H * dv, dv, H * dv, dv,
+                                            1e-12, 0, stream)
+            if rc:
+                _lib.check(rc)
+        return step
 
-    ms, wall = _events_ms(torch, step, steps, warmup)
+    ms_cold, wall = _events_ms(torch, make_step(n_sets), steps, warmup)
+    ms_warm, _ = _events_ms(torch, make_step(1), steps, warmup)
     bytes_per_launch = B * H * (2 * D_EXP * dv * 4 + 2 * D_EXP * 4 + (2 * 16 + 2 * dv) * 2)
+    ms = max(ms_cold, ms_warm)
     gbs = bytes_per_launch / (ms * 1e-3) / 1e9
-    assert torch.isfinite(y.float()).all() and torch.isfinite(kv_state).all()
+    assert torch.isfinite(y.float()).all() and all(torch.isfinite(a).all() for a, _ in states)
     return {
         "tok_s": B / (ms * 1e-3),
         "ms": ms,
         "wall_ms": wall,
+        "cold": {"ms": round(ms_cold, 5), "GBps": round(bytes_per_launch / (ms_cold * 1e-3) / 1e9, 1), "state_sets": n_sets,
+                 "working_set_MB": round(n_sets * (kv_state.numel() + k_state.numel()) * 4 / 1e6, 1)},
+        "warm": {"ms": round(ms_warm, 5), "GBps": round(bytes_per_launch / (ms_warm * 1e-3) / 1e9, 1), "state_sets": 1,
+                 "working_set_MB": round((kv_state.numel() + k_state.numel()) * 4 / 1e6, 1)},
         "roofline": {"kernel": "lin_step_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else None,
-                     "algorithmic_bytes_per_launch": bytes_per_launch},
-        "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, bf16 q/k/v",
+                     "algorithmic_bytes_per_launch": bytes_per_launch,
+                     "timed": "the slower of cold (rotating state sets) and warm (one set)"},
+        "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, "
+                    f"bf16 q/k/v, {n_sets} independent state sets visited in turn",
     }
 
 
@@ -135,29 +155,49 @@ def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
     }
 
 
-def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256):
+def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_sets=4):
+    """Sliding-window prefill + decode.  The prefill is timed COLD over `n_sets` different packed
+    qkv tensors and outputs visited in turn (n_sets x 268 MB of traffic: beyond the 256 MB
+    last-level cache) and WARM on one; the roofline figure is the lower of the two."""
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(2)
-    qkv = torch.randn(B, L, 3, H, 64, generator=g).bfloat16().to(dev)
-    ms, _ = _events_ms(torch, lambda: ops.swa_prefill(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=64), steps, warmup)
+    qkvs = [torch.randn(B, L, 3, H, 64, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
+    outs = [torch.empty(B, L, H, 64, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+    qkv = qkvs[0]
+    it = [0]
+
+    def make_pf(sets):
+        def pf():
+            x, o = qkvs[it[0] % sets], outs[it[0] % sets]
+            it[0] += 1
+            ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=64, out=o)
+        return pf
+
+    ms_cold, _ = _events_ms(torch, make_pf(n_sets), steps, warmup)
+    ms_warm, _ = _events_ms(torch, make_pf(1), steps, warmup)
+    ms = max(ms_cold, ms_warm)
     byts = B * L * H * 4 * 64 * 2
     gbs = byts / (ms * 1e-3) / 1e9
     cache = torch.zeros(B, L + decode_steps, 2, H, 64, dtype=torch.bfloat16, device=dev)
     cache[:, :L] = qkv[:, :, 1:]
     qn = torch.randn(B, 1, 3, H, 64, generator=g).bfloat16().to(dev)
+    o1 = torch.empty(B, 1, H, 64, dtype=torch.bfloat16, device=dev)
     pos = [L]
 
     def dstep():
-        ops.swa_step(qn[:, :, 0], qn[:, :, 1], qn[:, :, 2], cache, pos[0], w_left=64)
+        ops.swa_step(qn[:, :, 0], qn[:, :, 1], qn[:, :, 2], cache, pos[0], w_left=64, out=o1)
         pos[0] = L + (pos[0] + 1 - L) % decode_steps
 
     dms, _ = _events_ms(torch, dstep, decode_steps, 8)
     return {
         "prefill_tok_s": B * L / (ms * 1e-3), "prefill_ms": ms, "decode_tok_s": B / (dms * 1e-3), "decode_us": dms * 1e3,
         "B": B, "L": L, "window": 64,
+        "cold": {"ms": round(ms_cold, 5), "GBps": round(byts / (ms_cold * 1e-3) / 1e9, 1), "input_sets": n_sets},
+        "warm": {"ms": round(ms_warm, 5), "GBps": round(byts / (ms_warm * 1e-3) / 1e9, 1), "input_sets": 1},
         "roofline": {"kernel": "swa_prefill_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES["swa_prefill_kernel"], "algorithmic_bytes_per_launch": byts},
+                     "traffic": MEASURED_TRAFFIC_BYTES["swa_prefill_kernel"], "algorithmic_bytes_per_launch": byts,
+                     "timed": "the slower of cold (rotating inputs) and warm (one input)"},
     }
 
 
@@ -287,7 +327,7 @@ def main():
     ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "copy"], default=None,
                     help="one workload only; 'copy' is a plain 256 MiB device copy used to calibrate the "
                          "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
-    ap.add_argument("--prefill-batches", default="1,8,48,96",
+    ap.add_argument("--prefill-batches", default="1,8,32,96",
                     help="comma-separated batch sizes of the L=4096 prefill lines")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -321,7 +361,8 @@ def main():
         d = bench_decode(torch, ops, args.steps, args.warmup)
         out.update({"value": round(d["tok_s"], 1), "ms_per_step": round(d["ms"], 5),
                     "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
-                    "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5)})
+                    "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5),
+                    "decode_cold": d["cold"], "decode_warm": d["warm"]})
     if args.only in (None, "prefill"):
         pre = [bench_prefill(torch, ops, 30, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
@@ -331,7 +372,7 @@ def main():
         d5 = bench_decode(torch, ops, 64, 8, B=64, dv=128, prefill_len=256)
         out["long_context"] = {"prefill": {k: (round(v, 3) if isinstance(v, float) else v) for k, v in c5.items()},
                                "decode": {"tok_s": round(d5["tok_s"], 1), "ms": round(d5["ms"], 5), "B": 64, "dv": 128,
-                                          "roofline": d5["roofline"]}}
+                                          "cold": d5["cold"], "warm": d5["warm"], "roofline": d5["roofline"]}}
     if args.only in (None, "swa"):
         s = bench_swa(torch, ops, 20, 3)
         out["swa"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in s.items()}
