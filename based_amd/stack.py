@@ -18,6 +18,7 @@ from typing import Optional
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from . import ops
 
@@ -57,12 +58,39 @@ class StackConfig(SimpleNamespace):
             n_embd=1024, n_layer=27, n_head=16, n_inner=None, vocab_size=50277, pad_vocab_size_multiple=8,
             layer_norm_epsilon=1e-5, rms_norm=True, residual_in_fp32=True, initializer_range=0.02,
             tie_word_embeddings=True, activation_function="swiglu", mlp_fc1_bias=False, mlp_fc2_bias=False,
+            mlp_type="base", ff_mult=2,
             qkv_proj_bias=False, out_proj_bias=False, rotary_emb_fraction=0.0, rotary_emb_base=10000.0,
             rotary_emb_interleaved=False, scale_attn_weights=True, max_position_embeddings=0,
             mixer=None, alt_mixer=None, alt_mixer_layers=None, alt_mixer_2=None, alt_mixer_2_layers=None,
         )
         defaults.update(kw)
         super().__init__(**defaults)
+
+    # What the reference assumes for a key that a config dictionary does not carry: transformers'
+    # GPT2Config constructor defaults plus the getattr defaults of based/models/gpt.py:100-113,
+    # 206-208, 254, 262, 352, 359, 529, 745.  They differ from the defaults above (which describe
+    # the released Based configurations): a config.json written by the reference's training code
+    # that omits a key must mean here what it means there.
+    REFERENCE_DEFAULTS = dict(
+        n_embd=768, n_layer=12, n_head=12, n_inner=None, vocab_size=50257, pad_vocab_size_multiple=1,
+        layer_norm_epsilon=1e-5, rms_norm=False, residual_in_fp32=False, initializer_range=0.02,
+        tie_word_embeddings=True, activation_function="gelu_new", mlp_fc1_bias=True, mlp_fc2_bias=True,
+        mlp_type="base", ff_mult=2, qkv_proj_bias=True, out_proj_bias=True, rotary_emb_fraction=0.0,
+        rotary_emb_base=10000.0, rotary_emb_interleaved=False, scale_attn_weights=True,
+        max_position_embeddings=0, n_positions=1024,
+    )
+
+    @classmethod
+    def from_reference_dict(cls, d: dict) -> "StackConfig":
+        """Config from a dictionary in the reference's format (the content of a checkpoint's
+        config.json, or the keyword arguments its tests pass to GPT2MixerConfig), missing keys
+        filled with the reference's defaults.  GPT2Config's `n_positions` feeds
+        `max_position_embeddings` (its attribute map), as the reference's model reads it."""
+        cfg = dict(cls.REFERENCE_DEFAULTS)
+        cfg.update(d)
+        if "max_position_embeddings" not in d:
+            cfg["max_position_embeddings"] = cfg["n_positions"]
+        return cls(**cfg)
 
     @property
     def hidden_size(self):
@@ -134,19 +162,43 @@ class RMSNorm(nn.Module):
         return ops.add_rms_norm(x, None, self.weight, self.eps, want_residual=False)[0]
 
 
-class GatedMlp(nn.Module):
-    """SwiGLU MLP: fc2(y * silu(gate)), y, gate = fc1(x).chunk(2) (mlp.py:141-151)."""
+_GATE_ACTIVATIONS = {"glu": torch.sigmoid, "swiglu": F.silu, "geglu": F.gelu}
 
-    def __init__(self, in_features, hidden_features=None, bias1=False, bias2=False, multiple_of=256,
-                 device=None, dtype=None):
+
+class GatedMlp(nn.Module):
+    """Gated MLP of based/models/mlp.py:99-157.  Layout 'base': fc2(y * act(gate)) with
+    y, gate = fc1(x).chunk(2).  Layout 'alt' (the NeoX-style MLP of the reference's test
+    configuration): fc2(act(fc1(x)) * fc3(x)) with a hidden size derived from ff_mult.
+    activation: "swiglu" (silu; the released models), "geglu" (gelu) or "glu" (sigmoid),
+    chosen as in gpt.py:238-243.  The released combination (base + swiglu) gates in one HIP
+    kernel; the others are two element-wise torch operations."""
+
+    def __init__(self, in_features, hidden_features=None, activation="swiglu", bias1=False, bias2=False,
+                 multiple_of=256, mlp_type="base", ff_mult=2, device=None, dtype=None):
         super().__init__()
-        hidden_features = hidden_features if hidden_features is not None else int(8 * in_features / 3)
-        hidden_features = (hidden_features + multiple_of - 1) // multiple_of * multiple_of
-        self.fc1 = nn.Linear(in_features, 2 * hidden_features, bias=bias1, device=device, dtype=dtype)
-        self.fc2 = nn.Linear(hidden_features, in_features, bias=bias2, device=device, dtype=dtype)
+        if activation not in _GATE_ACTIVATIONS:
+            raise NotImplementedError(f"activation_function {activation!r}: only gated MLPs (glu / swiglu / geglu)")
+        fk = {"device": device, "dtype": dtype}
+        self.activation = activation
+        self.mlp_type = mlp_type
+        if mlp_type == "base":
+            hidden_features = hidden_features if hidden_features is not None else int(8 * in_features / 3)
+            hidden_features = (hidden_features + multiple_of - 1) // multiple_of * multiple_of
+            self.fc1 = nn.Linear(in_features, 2 * hidden_features, bias=bias1, **fk)
+        else:
+            hidden_features = int(2 * in_features * ff_mult / 3)
+            hidden_features = (hidden_features + multiple_of - 1) // multiple_of * multiple_of
+            self.fc1 = nn.Linear(in_features, hidden_features, bias=bias1, **fk)
+            self.fc3 = nn.Linear(in_features, hidden_features, bias=bias1, **fk)
+        self.fc2 = nn.Linear(hidden_features, in_features, bias=bias2, **fk)
 
     def forward(self, x):
-        return self.fc2(ops.swiglu(self.fc1(x)))
+        if self.mlp_type != "base":
+            return self.fc2(_GATE_ACTIVATIONS[self.activation](self.fc1(x)) * self.fc3(x))
+        if self.activation == "swiglu":
+            return self.fc2(ops.swiglu(self.fc1(x)))
+        y, gate = self.fc1(x).chunk(2, dim=-1)
+        return self.fc2(y * _GATE_ACTIVATIONS[self.activation](gate))
 
 
 class Block(nn.Module):
@@ -207,8 +259,9 @@ class GPTModel(nn.Module):
         if not config.rms_norm:
             raise NotImplementedError("the block glue kernel implements RMSNorm (rms_norm: True in the released configs)")
         norm_cls = partial(RMSNorm, eps=config.layer_norm_epsilon, **fk)
-        mlp_cls = partial(GatedMlp, hidden_features=config.n_inner, bias1=config.mlp_fc1_bias,
-                          bias2=config.mlp_fc2_bias, **fk)
+        mlp_cls = partial(GatedMlp, hidden_features=config.n_inner, activation=config.activation_function,
+                          bias1=config.mlp_fc1_bias, bias2=config.mlp_fc2_bias, mlp_type=config.mlp_type,
+                          ff_mult=config.ff_mult, **fk)
         self.layers = nn.ModuleList([
             Block(config.hidden_size, create_mixer_cls(config, layer_idx=i, **fk), mlp_cls, norm_cls,
                   residual_in_fp32=config.residual_in_fp32, layer_idx=i)
@@ -267,7 +320,7 @@ class GPTLMHeadModel(nn.Module, GenerationMixin):
         import re
 
         with open(os.path.join(directory, "config.json")) as f:
-            config = StackConfig(**json.load(f))
+            config = StackConfig.from_reference_dict(json.load(f))
         model = cls(config, device=device, dtype=dtype)
         st_path = os.path.join(directory, "model.safetensors")
         if os.path.exists(st_path):
@@ -281,6 +334,28 @@ class GPTLMHeadModel(nn.Module, GenerationMixin):
             state["lm_head.weight"] = state["transformer.embeddings.word_embeddings.weight"]
         model.load_state_dict(state, strict=strict)
         return model
+
+    def load_state_dict(self, state_dict, strict=True, **kwargs):
+        """Also accepts checkpoints written with the older order of the layers in a block (norm
+        after the mixer / MLP, a leading `transformer.ln_0`): their norm parameters are moved to
+        the current prenorm slots exactly as the reference does (gpt.py:829-853); norms without
+        a bias (RMSNorm) simply have no bias entries to move."""
+        if "transformer.ln_0.weight" in state_dict:
+            state_dict = dict(state_dict)
+            n_layers = len(self.transformer.layers)
+
+            def move(src, dst):
+                for suffix in ("weight", "bias"):
+                    if f"{src}.{suffix}" in state_dict:
+                        state_dict[f"{dst}.{suffix}"] = state_dict.pop(f"{src}.{suffix}")
+
+            move(f"transformer.layers.{n_layers - 1}.norm2", "transformer.ln_f")
+            for l in reversed(range(n_layers)):
+                move(f"transformer.layers.{l}.norm1", f"transformer.layers.{l}.norm2")
+                if l > 0:
+                    move(f"transformer.layers.{l - 1}.norm2", f"transformer.layers.{l}.norm1")
+            move("transformer.ln_0", "transformer.layers.0.norm1")
+        return super().load_state_dict(state_dict, strict=strict, **kwargs)
 
     def forward(self, input_ids, position_ids=None, inference_params=None, num_last_tokens=0, stream=None, **kwargs):
         assert input_ids.ndim == 2, f"Expected `input_ids` to have shape [b, slen], but got shape {input_ids.shape}"

@@ -33,6 +33,14 @@ tests/test_oracle.py):
                           agreement with THAT library is "parity unpinned".
   gated_short_conv(_step) F.conv1d(groups=D, padding=K-1)[..., :L] + F.silu, per-element
                           brute force, step == parallel                   -> pinned
+  add_rms_norm            closed form on hand-made rows, the cast BEFORE the norm (a bf16
+                          sum rounded first), the fp32 residual stream     -> pinned
+  gated_mlp               F.glu / explicit products for the four (activation, layout)
+                          combinations                                      -> pinned
+  stack_forward           composition of the functions above in the order of
+                          block.py:134-163 and gpt.py:622-736; checked against a
+                          hand-unrolled one-layer case and against nn.Module building
+                          blocks (nn.Linear, nn.Embedding, F.conv1d, SDPA) -> pinned
 """
 from __future__ import annotations
 
@@ -260,3 +268,90 @@ def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool 
     r = x if residual is None else x + residual
     y = rms_norm(r.to(x.dtype), weight, eps)
     return y, (r.float() if residual_in_fp32 else r)
+
+
+# ----------------------------------------------------------------------------------------------
+# Model assembly (only what the stack-level parity tests need), CPU, any float dtype
+# ----------------------------------------------------------------------------------------------
+def gated_mlp(x, fc1_w, fc2_w, fc3_w=None, activation: str = "swiglu", fc1_b=None, fc2_b=None, fc3_b=None):
+    """GatedMlp.forward (based/models/mlp.py:141-157).  Layout 'base' (fc3_w is None):
+    y, gate = fc1(x).chunk(2); fc2(y * act(gate)), with F.glu for the sigmoid case.  Layout
+    'alt' (fc3_w given): fc2(act(fc1(x)) * fc3(x)).  act: glu -> sigmoid, swiglu -> silu,
+    geglu -> gelu (based/models/gpt.py:238-243)."""
+    act = {"glu": torch.sigmoid, "swiglu": F.silu, "geglu": F.gelu}[activation]
+    if fc3_w is None:
+        y, gate = F.linear(x, fc1_w, fc1_b).chunk(2, dim=-1)
+        return F.linear(y * act(gate), fc2_w, fc2_b)
+    return F.linear(act(F.linear(x, fc1_w, fc1_b)) * F.linear(x, fc3_w, fc3_b), fc2_w, fc2_b)
+
+
+def mixer_kind(config, layer_idx: int) -> tuple:
+    """(kind, spec) of a layer's mixer following create_mixer_cls (based/models/gpt.py:64-96):
+    alt_mixer_2 wins over alt_mixer wins over mixer; kind from the `_target_` string."""
+    spec = config["mixer"]
+    if config.get("alt_mixer_2_layers") is not None and layer_idx in config["alt_mixer_2_layers"]:
+        spec = config["alt_mixer_2"]
+    elif config.get("alt_mixer_layers") is not None and layer_idx in config["alt_mixer_layers"]:
+        spec = config["alt_mixer"]
+    target = spec["_target_"]
+    kind = "linear" if "linear_attention" in target else "slide" if "slide" in target else "conv"
+    return kind, spec
+
+
+def stack_forward(input_ids, sd: dict, config: dict, dtype=torch.float32):
+    """Parallel forward of the Based stack: embeddings (+ learned positions) ->
+    [add + RMSNorm -> mixer -> add + RMSNorm -> gated MLP] x n_layer -> add + final RMSNorm ->
+    LM head (GPTModel.forward gpt.py:622-736, Block.forward block.py:134-163, dropout-free,
+    prenorm, residual stream in fp32 when residual_in_fp32).  `sd` is a state dict with the
+    reference's parameter names; `config` a plain dict with the reference's keys.  Activations are
+    kept in `dtype` between the operations exactly where the model would hold them in its own
+    dtype (every projection output is rounded to `dtype`); the mixers' inner arithmetic is fp32 on
+    those rounded inputs.  With dtype=float32 this is the exact-arithmetic statement of the model;
+    with dtype=bfloat16 it shows how far a bf16 model may sit from it through rounding alone."""
+    g = lambda name: sd[name].to(dtype) if name in sd else None
+    n_embd, n_head, eps = config["n_embd"], config["n_head"], config.get("layer_norm_epsilon", 1e-5)
+    res_fp32 = config.get("residual_in_fp32", False)
+    B, L = input_ids.shape
+    hidden = F.embedding(input_ids, g("transformer.embeddings.word_embeddings.weight"))
+    if config.get("max_position_embeddings", 0) > 0:
+        hidden = hidden + g("transformer.embeddings.position_embeddings.weight")[:L]
+    residual = None
+    for i in range(config["n_layer"]):
+        pre = f"transformer.layers.{i}."
+        hidden, residual = add_rms_norm(hidden, residual, g(pre + "norm1.weight"), eps, res_fp32)
+        kind, spec = mixer_kind(config, i)
+        m = pre + "mixer."
+        if kind == "conv":
+            u = F.linear(hidden, g(m + "in_proj.weight"), g(m + "in_proj.bias"))
+            y = gated_short_conv(u, g(m + "conv.conv.weight")[:, 0], g(m + "conv.conv.bias"))
+            hidden = F.linear(y, g(m + "out_proj.weight"), g(m + "out_proj.bias"))
+        elif kind == "linear":
+            H = spec.get("num_heads", 16)
+            fd = spec.get("feature_dim", 16)
+            q = F.linear(hidden, g(m + "proj_q.weight")).view(B, L, H, fd).transpose(1, 2)
+            k = F.linear(hidden, g(m + "proj_k.weight")).view(B, L, H, fd).transpose(1, 2)
+            v = F.linear(hidden, g(m + "proj_v.weight")).view(B, L, H, -1).transpose(1, 2)
+            # fp32 arithmetic on the (dtype-rounded) projections, like the kernels (module header, F9)
+            y = linear_attn_quadratic(q.float(), k.float(), v.float(), eps=spec.get("eps", 1e-12))
+            y = y.transpose(1, 2).reshape(B, L, -1)
+            hidden = F.linear(y.to(dtype), g(m + "out_proj.weight"))
+        else:
+            hd = n_embd // n_head
+            qkv = F.linear(hidden, g(m + "Wqkv.weight"), g(m + "Wqkv.bias")).view(B, L, 3, n_head, hd)
+            q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+            rot = int(config.get("rotary_emb_fraction", 0.0) * hd)
+            if rot > 0:
+                assert rot == hd, "only whole-head rotary is restated"
+                pos = torch.arange(L)
+                q = rotary_embedding(q, pos, config.get("rotary_emb_base", 10000.0))
+                k = rotary_embedding(k, pos, config.get("rotary_emb_base", 10000.0))
+            scale = hd ** -0.5 if config.get("scale_attn_weights", True) else 1.0
+            o = sliding_window_attn(q, k, v, w_left=spec.get("window_size", 128) // 2, scale=scale)
+            hidden = F.linear(o.reshape(B, L, n_embd).to(dtype), g(m + "out_proj.weight"), g(m + "out_proj.bias"))
+        hidden, residual = add_rms_norm(hidden, residual, g(pre + "norm2.weight"), eps, res_fp32)
+        p = pre + "mlp."
+        hidden = gated_mlp(hidden, g(p + "fc1.weight"), g(p + "fc2.weight"), g(p + "fc3.weight"),
+                           config.get("activation_function", "swiglu"), g(p + "fc1.bias"), g(p + "fc2.bias"),
+                           g(p + "fc3.bias"))
+    hidden, _ = add_rms_norm(hidden, residual, g("transformer.ln_f.weight"), eps, res_fp32)
+    return F.linear(hidden, g("lm_head.weight"))

@@ -131,15 +131,37 @@ def test_config4_full_stack_generation(dev):
     out = model.generate(input_ids=ids, max_length=P + T, return_dict_in_generate=True, output_scores=True, top_k=1)
     assert out.sequences.shape == (B, P + T) and len(out.scores) == T
     seqs = out.sequences.clone()
-    # 27 bf16 layers deep, element-wise tolerances of the 2-layer reference test are too tight for
-    # the worst of 4 x 50k logits; the bar here is rel-L2 of the logit vectors (and the
-    # element-wise bound of the reference's test on 99.9 % of the entries).
+    # the reference's own assertion (atol 5e-2, rtol 1e-2 on every logit) at three positions
     with torch.inference_mode():
         for i in (0, 63, T - 1):
             ref = model(input_ids=seqs[:, : P + i]).logits[:, -1].float()
             got = out.scores[i].float()
-            err = rel_l2(got, ref)
-            ok = ((got - ref).abs() <= 5e-2 + 1e-2 * ref.abs()).float().mean().item()
-            print(f"position {i}: rel-L2 {err:.4f}, within reference tolerance {ok:.5f}", flush=True)
-            assert err < 3e-2, f"position {i}: rel-L2 {err}"
-            assert ok > 0.999, f"position {i}: only {ok} of the logits within atol 5e-2 / rtol 1e-2"
+            print(f"position {i}: rel-L2 {rel_l2(got, ref):.4f}, max |diff| {float((got - ref).abs().max()):.4f}", flush=True)
+            assert torch.allclose(got, ref, atol=5e-2, rtol=1e-2), f"position {i}"
+
+
+def test_config4_stack_against_oracle_composition(dev):
+    """The 27-layer shape (all three mixer kinds, SwiGLU MLPs, fp32 residual stream, tied head)
+    against the oracle composition on the CPU, on a short prompt (the CPU statement is quadratic in
+    the length).  27 bf16 layers deep every GEMM output is rounded, so the element-wise bound of
+    the 2-layer reference test does not apply against exact arithmetic; the bar is that the GPU
+    model sits as close to the fp32 truth as the SAME composition evaluated with bf16 activations
+    on the CPU does (rounding alone), and closer than 4e-2 in rel-L2."""
+    from based_amd.stack import GPTLMHeadModel, based_360m_config
+    from oracle import based_oracle as O
+
+    torch.manual_seed(0)
+    cfg = based_360m_config(rotary_emb_fraction=1.0)
+    model = GPTLMHeadModel(cfg, device=dev, dtype=torch.bfloat16).eval()
+    g = torch.Generator(device="cpu").manual_seed(5)
+    ids = torch.randint(0, 50277, (1, 160), generator=g)
+    with torch.inference_mode():
+        got = model(ids.to(dev)).logits[:, -8:].float().cpu()
+    sd = {k: v.detach().cpu() for k, v in model.state_dict().items()}
+    exact = O.stack_forward(ids, sd, vars(cfg), dtype=torch.float32)[:, -8:]
+    rounded = O.stack_forward(ids, sd, vars(cfg), dtype=torch.bfloat16)[:, -8:].float()
+    e_gpu, e_cpu = rel_l2(got, exact), rel_l2(rounded, exact)
+    print(f"27-layer stack: rel-L2 to the fp32 statement: GPU bf16 {e_gpu:.4f}, CPU bf16 composition {e_cpu:.4f}; "
+          f"GPU vs CPU bf16 {rel_l2(got, rounded):.4f}", flush=True)
+    assert e_gpu < 4e-2
+    assert e_gpu < 1.5 * e_cpu + 2e-3

@@ -159,3 +159,55 @@ def test_local_checkpoint_round_trip(tmp_path):
     assert a.keys() == b.keys()
     assert all(torch.equal(a[k], b[k]) for k in a)
     assert dst.lm_head.weight is dst.transformer.embeddings.word_embeddings.weight
+
+
+def test_reference_config_defaults():
+    """A config dictionary in the reference's format means here what it means there: missing keys
+    take transformers' GPT2Config defaults and the getattr defaults of based/models/gpt.py."""
+    from based_amd.stack import StackConfig
+
+    c = StackConfig.from_reference_dict({"n_embd": 256, "n_head": 16, "rms_norm": True})
+    assert (c.residual_in_fp32, c.mlp_fc1_bias, c.mlp_fc2_bias, c.qkv_proj_bias, c.out_proj_bias) == (False, True, True, True, True)
+    assert c.vocab_size == 50257 and c.pad_vocab_size_multiple == 1 and c.n_layer == 12
+    assert c.max_position_embeddings == 1024 and c.mlp_type == "base" and c.activation_function == "gelu_new"
+    c = StackConfig.from_reference_dict({"max_position_embeddings": 0, "residual_in_fp32": True})
+    assert c.max_position_embeddings == 0 and c.residual_in_fp32 is True
+
+
+def test_old_layer_order_checkpoints_are_remapped():
+    """Checkpoints written with the earlier order of the layers in a block (gpt.py:829-853):
+    ln_0 -> layers.0.norm1, layers.l.norm1 -> layers.l.norm2, layers.l.norm2 -> layers.(l+1).norm1,
+    last norm2 -> ln_f."""
+    cfg = based_360m_config(n_embd=64, n_head=1, n_layer=3, n_inner=128, vocab_size=32,
+                            alt_mixer_layers=[], alt_mixer_2_layers=[])
+    torch.manual_seed(2)
+    model = GPTLMHeadModel(cfg)
+    sd = {k: v.clone() for k, v in model.state_dict().items()}
+    norms = {}
+    for name in ["transformer.ln_f"] + [f"transformer.layers.{l}.norm{j}" for l in range(3) for j in (1, 2)]:
+        norms[name] = torch.randn(64)
+        sd[name + ".weight"] = norms[name]
+    # the same parameters filed under the old names
+    old = dict(sd)
+    old["transformer.ln_0.weight"] = old.pop("transformer.layers.0.norm1.weight")
+    for l in range(3):
+        old[f"transformer.layers.{l}.norm1.weight"] = sd[f"transformer.layers.{l}.norm2.weight"]
+        nxt = f"transformer.layers.{l + 1}.norm1.weight" if l < 2 else "transformer.ln_f.weight"
+        old[f"transformer.layers.{l}.norm2.weight"] = sd[nxt]
+    del old["transformer.ln_f.weight"]
+    model.load_state_dict(old)
+    got = model.state_dict()
+    for name, w in norms.items():
+        assert torch.equal(got[name + ".weight"], w), name
+
+
+def test_gated_mlp_variants_construct_like_the_reference():
+    from based_amd.stack import GatedMlp
+
+    alt = GatedMlp(256, hidden_features=2816, activation="geglu", mlp_type="alt", ff_mult=2)
+    assert set(dict(alt.named_parameters())) == {"fc1.weight", "fc3.weight", "fc2.weight"}
+    assert alt.fc1.weight.shape == (512, 256) and alt.fc2.weight.shape == (256, 512)   # int(2*256*2/3) -> 512
+    base = GatedMlp(1024, hidden_features=2048)
+    assert base.fc1.weight.shape == (4096, 1024) and base.fc2.weight.shape == (1024, 2048)
+    with pytest.raises(NotImplementedError):
+        GatedMlp(64, activation="gelu_new")

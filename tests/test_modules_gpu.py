@@ -81,7 +81,7 @@ def _small_stack(dev, rotary=0.0):
         alt_mixer={"_target_": "based.models.mixers.linear_attention.LinearAttention", "l_max": 2048,
                    "feature_map": {"_target_": "based.models.mixers.linear_attention.TaylorExp", "input_dim": 16},
                    "feature_dim": 16, "num_heads": 4},
-        alt_mixer_layers=[1], alt_mixer_2_layers=[2], initializer_range=0.1)
+        alt_mixer_layers=[1], alt_mixer_2_layers=[2])
     torch.manual_seed(3)
     model = GPTLMHeadModel(cfg, device=dev, dtype=torch.bfloat16)
     model.eval()
@@ -94,7 +94,7 @@ def test_generation_cached_equals_parallel(dev, prefill_size, rotary):
     """3-layer stack (BaseConv, LinearAttention, SlidingAttention), greedy generation with the
     cache vs a fresh parallel forward over every prefix."""
     model = _small_stack(dev, rotary)
-    n_new = 24
+    n_new = 64
     torch.manual_seed(0)
     input_ids = torch.randint(1, 1000, (4, prefill_size), dtype=torch.long, device=dev)
     out = model.generate(input_ids=input_ids, max_length=prefill_size + n_new, return_dict_in_generate=True,
@@ -105,16 +105,9 @@ def test_generation_cached_equals_parallel(dev, prefill_size, rotary):
     with torch.inference_mode():
         for i in range(n_new):
             ref = model(input_ids=seqs[:, : prefill_size + i]).logits[:, -1]
-            # The reference's test bounds every logit by atol 5e-2 / rtol 1e-2.  The worst of the
-            # 4000 logits of this randomly initialised stack sits right at that bound (bf16 GEMMs
-            # of different shapes in the cached and the parallel pass), so the bound is asked of
-            # 99.9 % of them, twice the bound of all, and rel-L2 of the whole vector.
-            got, want = scores[:, i].float(), ref.float()
-            diff = (got - want).abs()
-            bound = ATOL_BF16 + RTOL_BF16 * want.abs()
-            assert (diff <= bound).float().mean().item() >= 0.999, f"position {i}"
-            assert bool((diff <= 2 * bound).all()), f"position {i}: max abs diff {float(diff.max())}"
-            assert rel_l2(got, want) < 2e-2, f"position {i}"
+            # the reference's own assertion (based/tests/test_generation.py:169-173), on every logit
+            assert torch.allclose(ref, scores[:, i], atol=ATOL_BF16, rtol=RTOL_BF16), f"position {i}"
+            assert torch.equal(seqs[:, prefill_size + i], ref.argmax(dim=-1)), f"position {i}"
 
 
 def test_graph_decode_equals_eager(dev):

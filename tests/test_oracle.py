@@ -283,3 +283,139 @@ def test_rotary_embedding_properties():
         w = 10000.0 ** (-2.0 * i / D)
         z = complex(float(x[b, l, h, i]), float(x[b, l, h, i + D // 2])) * complex(math.cos(l * w), math.sin(l * w))
         assert abs(float(rx[b, l, h, i]) - z.real) < 1e-5 and abs(float(rx[b, l, h, i + D // 2]) - z.imag) < 1e-5
+
+
+def test_add_rms_norm_closed_form_cast_order_and_fp32_stream():
+    """The prenorm glue (block.py:134-139): (i) closed form on hand-made rows; (ii) the sum is cast to
+    the activation dtype BEFORE the norm (a bf16 activation plus an fp32 residual is normalised from
+    the bf16-rounded sum); (iii) the residual stream that is handed on is the UNROUNDED fp32 sum."""
+    # (i) r = [3, 4] + [0, 0]: mean(r^2) = 12.5, y = r / sqrt(12.5 + eps) * w
+    x = torch.tensor([[3.0, 4.0]])
+    w = torch.tensor([2.0, 0.5])
+    y, r = O.add_rms_norm(x, None, w, eps=0.0, residual_in_fp32=True)
+    assert torch.allclose(y, torch.tensor([[3.0 / math.sqrt(12.5) * 2.0, 4.0 / math.sqrt(12.5) * 0.5]]), atol=1e-6)
+    assert torch.equal(r, x)
+    y, r = O.add_rms_norm(x, torch.tensor([[1.0, -4.0]]), w, eps=0.0)
+    assert torch.allclose(y, torch.tensor([[4.0 / math.sqrt(8.0) * 2.0, 0.0]]), atol=1e-6) and torch.equal(r, torch.tensor([[4.0, 0.0]]))
+    # eps enters under the root
+    y, _ = O.add_rms_norm(torch.tensor([[0.0, 0.0]]), None, w, eps=1e-5)
+    assert torch.equal(y, torch.zeros(1, 2))
+    y, _ = O.add_rms_norm(torch.tensor([[1e-3, 0.0]]), None, torch.ones(2), eps=1e-5)
+    assert abs(float(y[0, 0]) - 1e-3 / math.sqrt(0.5e-6 + 1e-5)) < 1e-6
+    # (ii) + (iii): x bf16, residual fp32 with bits below bf16 resolution
+    xb = torch.tensor([[1.0, 2.0, -3.0, 0.5]], dtype=torch.bfloat16)
+    res = torch.tensor([[0.001953125 * 0.37, 0.00390625 * 0.41, 0.0078125 * 0.3, 1.0 / 1024 * 0.45]])  # sub-ulp parts
+    wb = torch.ones(4, dtype=torch.bfloat16)
+    y, r = O.add_rms_norm(xb, res, wb, eps=1e-5, residual_in_fp32=True)
+    exact_sum = xb.float() + res
+    assert r.dtype == torch.float32 and torch.equal(r, exact_sum)           # stream: exact fp32 sum
+    rounded = exact_sum.to(torch.bfloat16)
+    assert not torch.equal(rounded.float(), exact_sum)                        # the case is discriminating
+    expect = (rounded.float() * torch.rsqrt(rounded.float().square().mean(-1, keepdim=True) + 1e-5)).to(torch.bfloat16)
+    assert y.dtype == torch.bfloat16 and torch.equal(y, expect)              # norm of the ROUNDED sum
+    # without an fp32 stream the sum itself is what torch promotion gives, handed on as is
+    y2, r2 = O.add_rms_norm(xb, res.to(torch.bfloat16), wb, eps=1e-5, residual_in_fp32=False)
+    assert r2.dtype == torch.bfloat16
+
+
+def test_gated_mlp_layouts():
+    """mlp.py:141-157: F.glu for the sigmoid gate, y * act(gate) for base, act(fc1) * fc3 for alt."""
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(3, 5, 8, generator=g)
+    w1, w2 = torch.randn(12, 8, generator=g), torch.randn(8, 6, generator=g)
+    h = x @ w1.T
+    assert torch.allclose(O.gated_mlp(x, w1, w2, activation="glu"), F.glu(h, dim=-1) @ w2.T, atol=1e-5)
+    assert torch.allclose(O.gated_mlp(x, w1, w2, activation="swiglu"), O.swiglu_mlp(x, w1, w2), atol=1e-6)
+    y, gate = h[..., :6], h[..., 6:]
+    assert torch.allclose(O.gated_mlp(x, w1, w2, activation="geglu"), (y * 0.5 * gate * (1 + torch.erf(gate / math.sqrt(2)))) @ w2.T, atol=1e-5)
+    w1a, w3a, w2a = torch.randn(6, 8, generator=g), torch.randn(6, 8, generator=g), torch.randn(8, 6, generator=g)
+    a = x @ w1a.T
+    ref = ((0.5 * a * (1 + torch.erf(a / math.sqrt(2)))) * (x @ w3a.T)) @ w2a.T
+    assert torch.allclose(O.gated_mlp(x, w1a, w2a, w3a, activation="geglu"), ref, atol=1e-5)
+    b1, b2 = torch.randn(12, generator=g), torch.randn(8, generator=g)
+    assert torch.allclose(O.gated_mlp(x, w1, w2, activation="swiglu", fc1_b=b1, fc2_b=b2),
+                          ((h + b1)[..., :6] * F.silu((h + b1)[..., 6:])) @ w2.T + b2, atol=1e-5)
+
+
+def _tiny_stack_config(**over):
+    cfg = dict(
+        n_embd=128, n_head=2, n_layer=3, n_inner=256, vocab_size=96, pad_vocab_size_multiple=8, rms_norm=True,
+        residual_in_fp32=True, activation_function="swiglu", mlp_type="base", layer_norm_epsilon=1e-5,
+        mlp_fc1_bias=False, mlp_fc2_bias=False, qkv_proj_bias=False, out_proj_bias=False, max_position_embeddings=0,
+        rotary_emb_fraction=0.0, scale_attn_weights=True,
+        mixer={"_target_": "based.models.mixers.convolution.BaseConv", "l_max": 64, "use_bias": True, "expand_proj": 4,
+               "kernel_size": 3},
+        alt_mixer={"_target_": "based.models.mixers.linear_attention.LinearAttention", "l_max": 64,
+                   "feature_map": {"_target_": "based.models.mixers.linear_attention.TaylorExp", "input_dim": 16},
+                   "feature_dim": 16, "num_heads": 2},
+        alt_mixer_layers=[1],
+        alt_mixer_2={"_target_": "based.models.mixers.slide_attention.SlidingAttention", "window_size": 128,
+                     "num_heads": 2, "causal": True},
+        alt_mixer_2_layers=[2],
+    )
+    cfg.update(over)
+    return cfg
+
+
+def test_stack_forward_against_hand_unrolled_modules():
+    """The composition (block.py:134-163, gpt.py:622-736) against the same stack unrolled by hand
+    from torch building blocks that share no code with the oracle's functions: nn.Embedding,
+    nn.Linear, nn.Conv1d (depthwise, padding K-1, truncated), F.scaled_dot_product_attention for
+    a window that covers the sequence, and the Taylor weights 1 + s + s^2/2 written out."""
+    import torch.nn as nn
+
+    from based_amd.stack import GPTLMHeadModel, StackConfig
+
+    torch.manual_seed(3)
+    cfg = _tiny_stack_config(rotary_emb_fraction=0.0, max_position_embeddings=32)
+    model = GPTLMHeadModel(StackConfig(**cfg))            # only used as a container of random weights
+    sd = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    for k in sd:                                          # make every norm weight non-trivial
+        if "norm" in k or "ln_f" in k:
+            sd[k] = 1.0 + 0.1 * torch.randn_like(sd[k])
+    B, L, D, H = 2, 20, 128, 2
+    ids = torch.randint(0, 96, (B, L))
+    got = O.stack_forward(ids, sd, cfg)
+
+    def rms(x, w):
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5) * w
+
+    emb = nn.Embedding.from_pretrained(sd["transformer.embeddings.word_embeddings.weight"])
+    h = emb(ids) + sd["transformer.embeddings.position_embeddings.weight"][:L]
+    res = None
+    for i in range(3):
+        pre = f"transformer.layers.{i}."
+        res = h if res is None else h + res
+        x = rms(res, sd[pre + "norm1.weight"])
+        m = pre + "mixer."
+        if i == 0:
+            u = x @ sd[m + "in_proj.weight"].T + sd[m + "in_proj.bias"]
+            conv = nn.Conv1d(256, 256, 3, groups=256, padding=2, bias=False)
+            conv.weight.data.copy_(sd[m + "conv.conv.weight"])
+            c = conv(u[..., :256].transpose(1, 2))[..., :L].transpose(1, 2)
+            h = (F.silu(c) * u[..., 256:]) @ sd[m + "out_proj.weight"].T + sd[m + "out_proj.bias"]
+        elif i == 1:
+            q = (x @ sd[m + "proj_q.weight"].T).view(B, L, H, 16).transpose(1, 2)
+            k = (x @ sd[m + "proj_k.weight"].T).view(B, L, H, 16).transpose(1, 2)
+            v = (x @ sd[m + "proj_v.weight"].T).view(B, L, H, 64).transpose(1, 2)
+            s = q @ k.transpose(-1, -2) / 4.0
+            a = torch.tril(1 + s + s * s / 2)
+            y = (a @ v) / (a.sum(-1, keepdim=True) + 1e-12)
+            h = y.transpose(1, 2).reshape(B, L, D) @ sd[m + "out_proj.weight"].T
+        else:
+            qkv = (x @ sd[m + "Wqkv.weight"].T).view(B, L, 3, H, 64)
+            o = F.scaled_dot_product_attention(qkv[:, :, 0].transpose(1, 2), qkv[:, :, 1].transpose(1, 2),
+                                               qkv[:, :, 2].transpose(1, 2), is_causal=True)   # window 64 >= L
+            h = o.transpose(1, 2).reshape(B, L, D) @ sd[m + "out_proj.weight"].T
+        res = h + res
+        x = rms(res, sd[pre + "norm2.weight"])
+        yv, gate = (x @ sd[pre + "mlp.fc1.weight"].T).chunk(2, -1)
+        h = (yv * F.silu(gate)) @ sd[pre + "mlp.fc2.weight"].T
+    x = rms(h + res, sd["transformer.ln_f.weight"])
+    ref = x @ sd["lm_head.weight"].T
+    assert got.shape == ref.shape == (B, L, 96)
+    assert torch.allclose(got, ref, atol=2e-5, rtol=1e-5)
+    # causality of the whole stack: changing the last token leaves earlier logits alone
+    ids2 = ids.clone()
+    ids2[:, -1] = (ids2[:, -1] + 1) % 96
+    assert torch.equal(O.stack_forward(ids2, sd, cfg)[:, :-1], got[:, :-1])

@@ -1,0 +1,154 @@
+"""Stack-level parity on the GPU.
+
+(1) A tiny BaseConv + LinearAttention + SlidingAttention stack against the ORACLE composition
+    (oracle.stack_forward: fp32 on the CPU, an independent statement of block.py:134-163 +
+    gpt.py:622-736 + mlp.py:141-157): prefill logits and the logits of every cached decode step,
+    held to the reference's own bound on EVERY logit (atol 5e-2 / rtol 1e-2 for bf16, atol 1e-3 /
+    rtol 3e-4 for fp32; based/tests/test_generation.py:106-115).
+(2) The reference's test configurations as written (test_generation.py:7-34,47-69: n_embd 256,
+    16 heads of dim 16, 2 layers, learned positions, NeoX-style geglu MLP, default init,
+    batch 4, prefill 1 and 128, 64 generated tokens, fp32 and bf16): cached logits against a fresh
+    parallel forward over every prefix, torch.allclose on all logits at the reference's
+    tolerances, plus the oracle composition as the independent arbiter.
+"""
+import pytest
+import torch
+
+from oracle import based_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+ATOL = {torch.float32: 1e-3, torch.bfloat16: 5e-2}   # test_generation.py:106-115
+RTOL = {torch.float32: 3e-4, torch.bfloat16: 1e-2}
+
+
+def _tiny_cfg(**over):
+    cfg = dict(
+        n_embd=256, n_head=4, n_layer=3, n_inner=512, vocab_size=1000, pad_vocab_size_multiple=8, rms_norm=True,
+        residual_in_fp32=True, activation_function="swiglu", mlp_type="base", layer_norm_epsilon=1e-5,
+        mlp_fc1_bias=False, mlp_fc2_bias=False, qkv_proj_bias=False, out_proj_bias=False, max_position_embeddings=0,
+        rotary_emb_fraction=0.0, scale_attn_weights=True, initializer_range=0.02,
+        mixer={"_target_": "based.models.mixers.convolution.BaseConv", "l_max": 2048, "use_bias": True, "expand_proj": 4,
+               "kernel_size": 3},
+        alt_mixer={"_target_": "based.models.mixers.linear_attention.LinearAttention", "l_max": 2048,
+                   "feature_map": {"_target_": "based.models.mixers.linear_attention.TaylorExp", "input_dim": 16},
+                   "feature_dim": 16, "num_heads": 4},
+        alt_mixer_layers=[1],
+        alt_mixer_2={"_target_": "based.models.mixers.slide_attention.SlidingAttention", "window_size": 128,
+                     "num_heads": 4, "causal": True},
+        alt_mixer_2_layers=[2],
+    )
+    cfg.update(over)
+    return cfg
+
+
+def _build(cfg, dev, dtype, seed=3):
+    from based_amd.stack import GPTLMHeadModel, StackConfig
+
+    torch.manual_seed(seed)
+    model = GPTLMHeadModel(StackConfig(**cfg), device=dev, dtype=dtype).eval()
+    with torch.no_grad():  # non-trivial norm weights, so that a misplaced norm shows
+        for name, p in model.named_parameters():
+            if "norm" in name or "ln_f" in name:
+                p.copy_(1.0 + 0.1 * torch.randn_like(p))
+    # the oracle sees exactly the parameters the device holds (bf16-rounded for a bf16 model), in fp32
+    sd = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    return model, sd
+
+
+def _allclose_all(got, want, dtype, what):
+    got, want = got.float().cpu(), want.float().cpu()
+    diff = (got - want).abs()
+    bound = ATOL[dtype] + RTOL[dtype] * want.abs()
+    worst = float((diff - bound).max())
+    assert worst <= 0, f"{what}: a logit exceeds atol {ATOL[dtype]} / rtol {RTOL[dtype]} by {worst:.3e} (max |diff| {float(diff.max()):.3e})"
+
+
+@pytest.mark.parametrize("rotary,window", [(0.0, 128), (1.0, 128), (1.0, 34)])
+def test_tiny_stack_matches_oracle_composition_bf16(dev, rotary, window):
+    cfg = _tiny_cfg(rotary_emb_fraction=rotary)
+    cfg["alt_mixer_2"] = dict(cfg["alt_mixer_2"], window_size=window)
+    model, sd = _build(cfg, dev, torch.bfloat16)
+    B, P, n_new = 2, 70, 16
+    torch.manual_seed(0)
+    ids = torch.randint(1, 1000, (B, P), dtype=torch.long, device=dev)
+    print(f"stack vs oracle bf16: rotary={rotary} window={window}", flush=True)
+    with torch.inference_mode():
+        logits = model(ids).logits
+    _allclose_all(logits, O.stack_forward(ids.cpu(), sd, cfg), torch.bfloat16, "prefill logits")
+    out = model.generate(input_ids=ids, max_length=P + n_new, return_dict_in_generate=True, output_scores=True, top_k=1)
+    seqs = out.sequences.cpu()
+    for i, sc in enumerate(out.scores):
+        ref = O.stack_forward(seqs[:, : P + i], sd, cfg)[:, -1]
+        _allclose_all(sc, ref, torch.bfloat16, f"cached decode step {i}")
+
+
+def test_tiny_stack_matches_oracle_composition_fp32(dev):
+    """fp32 model (BaseConv + LinearAttention; the window mixer computes in bf16 like the reference's
+    flash path and is left out here), fp32 tolerances."""
+    cfg = _tiny_cfg(n_layer=2, alt_mixer_2_layers=[])
+    model, sd = _build(cfg, dev, torch.float32)
+    B, P, n_new = 2, 40, 16
+    torch.manual_seed(1)
+    ids = torch.randint(1, 1000, (B, P), dtype=torch.long, device=dev)
+    with torch.inference_mode():
+        logits = model(ids).logits
+    _allclose_all(logits, O.stack_forward(ids.cpu(), sd, cfg), torch.float32, "prefill logits")
+    out = model.generate(input_ids=ids, max_length=P + n_new, return_dict_in_generate=True, output_scores=True, top_k=1)
+    seqs = out.sequences.cpu()
+    for i, sc in enumerate(out.scores):
+        _allclose_all(sc, O.stack_forward(seqs[:, : P + i], sd, cfg)[:, -1], torch.float32, f"cached decode step {i}")
+
+
+# ---------------------------------------------------------------------------------------------
+# the reference's own test configurations (based/tests/test_generation.py:7-34, 47-69)
+# ---------------------------------------------------------------------------------------------
+BASE_CONFIG = {
+    "n_embd": 256, "special_initializer": True, "n_head": 16, "n_layer": 2, "rms_norm": True, "fused_mlp": False,
+    "attn_pdrop": 0, "embd_pdrop": 0, "n_positions": 2048, "resid_pdrop": 0, "mlp_fc1_bias": False,
+    "mlp_fc2_bias": False, "fused_bias_fc": True, "out_proj_bias": False, "qkv_proj_bias": False,
+    "use_flash_attn": False, "residual_in_fp32": True, "activation_function": "geglu", "fused_dropout_add_ln": True,
+    "max_position_embeddings": 2048, "pad_vocab_size_multiple": 8, "reorder_and_upcast_attn": False,
+    "scale_attn_by_inverse_layer_idx": False, "n_inner": 1408 * 2, "mlp_type": "alt",
+}
+REFERENCE_CONFIGS = {
+    "base_conv": {"mixer": {"_target_": "based.models.mixers.convolution.BaseConv", "kernel_size": 3, "l_max": 2048},
+                  **BASE_CONFIG},
+    "linear_attn": {"feature_dim": 16,
+                    "mixer": {"_target_": "based.models.mixers.linear_attention.LinearAttention",
+                              "feature_map": {"_target_": "based.models.mixers.linear_attention.TaylorExp", "input_dim": 16},
+                              "num_heads": 16},
+                    **BASE_CONFIG},
+}
+
+
+@pytest.mark.parametrize("config", ["base_conv", "linear_attn"])
+@pytest.mark.parametrize("prefill_size", [1, 128])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_reference_generation_configs_as_written(dev, config, prefill_size, dtype):
+    from based_amd.stack import GPTLMHeadModel, StackConfig
+
+    cfg = REFERENCE_CONFIGS[config]
+    batch_size, n_generated_tokens = 4, 64
+    print(f"reference config {config} prefill {prefill_size} {dtype}", flush=True)
+    torch.manual_seed(0)
+    model = GPTLMHeadModel(StackConfig.from_reference_dict(cfg)).to(device=dev, dtype=dtype).eval()
+    torch.manual_seed(0)
+    input_ids = torch.randint(1, 1000, (batch_size, prefill_size), dtype=torch.long, device=dev)
+    out = model.generate(input_ids=input_ids, max_length=prefill_size + n_generated_tokens,
+                         return_dict_in_generate=True, output_scores=True, eos_token_id=None, top_k=1, cg=False)
+    scores = torch.stack(out.scores, dim=1)
+    seqs = out.sequences.clone()
+    atol, rtol = ATOL[dtype], RTOL[dtype]
+    sd = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    full_cfg = vars(StackConfig.from_reference_dict(cfg))
+    with torch.inference_mode():
+        for i in range(n_generated_tokens):
+            scores_ref = model(input_ids=seqs[:, : prefill_size + i]).logits
+            # the reference's assertions, on all logits
+            assert torch.allclose(scores_ref[:, -1], scores[:, i], atol=atol, rtol=rtol), f"position {i}"
+            assert torch.equal(seqs[:, prefill_size + i], scores_ref[:, -1].argmax(dim=-1)), f"position {i}"
+            if i % 16 == 0:  # and both against the independent fp32 statement of the same stack
+                want = O.stack_forward(seqs[:, : prefill_size + i].cpu(), sd, full_cfg)[:, -1]
+                _allclose_all(scores[:, i], want, dtype, f"cached step {i} vs oracle")
+                _allclose_all(scores_ref[:, -1], want, dtype, f"parallel step {i} vs oracle")
