@@ -1,9 +1,10 @@
 // Sliding-window causal softmax attention for gfx950: prefill (MFMA) and decode step.
 //
 // Prefill.  One workgroup of four wavefronts covers 64 consecutive queries of one
-// (batch, head); wavefront w owns queries [q0+16w, q0+16w+16) and the 80 keys
-// [n0-64, n0+16) they can see (window <= 64 to the left plus the causal diagonal).
-//   S^T = K Q^T   : 5 key tiles x 2 MFMA 16x16x32 (head dim 64); the workgroup's 128 K rows are
+// (batch, head); wavefront w owns queries [q0+16w, q0+16w+16) and the keys
+// [n0-64(NB-1), n0+16) they can see: NB = 2 staged blocks of 64 rows for a window of up to 64 to
+// the left (80 keys, 5 tiles), NB = 3 for up to 128 (144 keys, 9 tiles), plus the causal diagonal.
+//   S^T = K Q^T   : 5 or 9 key tiles x 2 MFMA 16x16x32 (head dim 64); the workgroup's K rows are
 //                   staged once in LDS (a lane's operand = 8 consecutive bf16 of one row).
 //   softmax       : S^T leaves the MFMA with lane <-> query and registers <-> keys, so the
 //                   row max / row sum are in-lane loops plus two cross-lane steps.
@@ -12,11 +13,13 @@
 //                   <-> channel, registers <-> keys) is the one operand that needs a
 //                   transpose: V rows are staged as they come and read with the transposing
 //                   LDS load.  Outputs leave through LDS as full 128-byte rows.
-// Whole-window softmax in one pass: 80 keys fit in registers, so no online rescaling.
+// Whole-window softmax in one pass: 80 (144) keys fit in registers, so no online rescaling.
 //
 // Decode.  One workgroup of four wavefronts per (batch, head) against the last w_left+1 rows of
 // a linear cache, with every load issued up front (one memory round trip per step).
 #include "common.hpp"
+
+#include <atomic>
 
 namespace based {
 
@@ -66,20 +69,24 @@ template <> struct SwaRows<true> {
 // attention of the reference (slide_attention.py:346-355,553-556).
 // kc_out / vc_out (optional): the (rotated) K rows and the V rows of this call are also written
 // to a KV cache, the job of _update_kv_cache (slide_attention.py:255-281).
-template <bool ROPE>
-__global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
+template <bool ROPE, int NB>
+__global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
     int w_left, float scale_log2e, const float* __restrict__ rope_cos, const float* __restrict__ rope_sin,
     __bf16* __restrict__ kc_out, __bf16* __restrict__ vc_out, long c_sb, long c_st, long c_sh) {
-  // Two blocks of 64 K rows and 64 V rows: one holds the current tile's own keys, the other the
-  // 64 keys to its left.  Moving on by one tile, "own" becomes "left" without a copy and the
-  // old left block takes the next tile's rows.
-  __shared__ __align__(16) __bf16 s_k[2 * kQTile * kKStride];
-  __shared__ __align__(16) __bf16 s_v[2 * kQTile * kVStride];
-  __shared__ __align__(16) __bf16 s_q[ROPE ? kQTile * kKStride : 8];  // rotated queries (ROPE only)
-  static_assert(kOStride == kKStride, "output staging reuses whole K rows of the left block");
+  // A ring of NB blocks of 64 K rows and 64 V rows: one holds the current tile's own keys, the
+  // others the 64 (NB - 1) keys to its left.  Moving on by one tile, "own" becomes "left" without
+  // a copy and the oldest block takes the next tile's rows.
+  constexpr int NT = 4 * (NB - 1) + 1;   // key tiles of 16 a wavefront sees
+  constexpr int NS = (NT + 1) / 2;       // key slabs of 32 in the second product (last one half empty)
+  // (dynamic LDS: the three-block ring with rotated queries is past the 64 KB static limit)
+  extern __shared__ __align__(16) unsigned char swa_lds[];
+  __bf16* const s_k = reinterpret_cast<__bf16*>(swa_lds);
+  __bf16* const s_v = s_k + NB * kQTile * kKStride;
+  __bf16* const s_q = s_v + NB * kQTile * kVStride;  // rotated queries (ROPE only)
+  static_assert(kOStride == kKStride, "output staging reuses whole K rows of the oldest block");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -175,12 +182,14 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
   SwaRows<ROPE> pre;
   bf16x8 bq[2], bq_next[2];
   {
-    // first tile: own rows in block 0, the 64 keys to the left in block 1 (one round trip)
-    SwaRows<ROPE> left;
-    load_rows(q0 - kQTile, left, false);
+    // first tile: own rows in block 0, the keys 64 a to the left in block NB - a (one round trip)
+    SwaRows<ROPE> left[NB - 1];
+#pragma unroll
+    for (int a = 1; a < NB; ++a) load_rows(q0 - a * kQTile, left[a - 1], false);
     load_rows(q0, pre, true);
     if constexpr (!ROPE) load_q(q0, bq);
-    store_rows(1, q0 - kQTile, left, false);
+#pragma unroll
+    for (int a = 1; a < NB; ++a) store_rows(NB - a, q0 - a * kQTile, left[a - 1], false);
     store_rows(0, q0, pre, true);
   }
   if (tile_begin + 1 < tile_end) {  // the next tile's rows travel while this one is computed
@@ -188,12 +197,17 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
     if constexpr (!ROPE) load_q(q0 + kQTile, bq_next);
   }
 
-  for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile) {
-    const int own = (tile - tile_begin) & 1;  // block with keys [q0, q0+64); 1 - own has [q0-64, q0)
+  int own = 0;  // ring block with keys [q0, q0+64); block own + 1 (mod NB) is the oldest
+  for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile, own = own + 1 == NB ? 0 : own + 1) {
+    const int oldest = own + 1 == NB ? 0 : own + 1;
     const int n0 = q0 + 16 * wave;            // first query of this wavefront
     const int n = n0 + col;                   // this lane's query
-    // staged key index x (0..127 <-> key q0 - 64 + x) -> row of the ring
-    auto ring_row = [&](int x) { return ((x < kQTile ? 1 - own : own) * kQTile) + (x & (kQTile - 1)); };
+    // staged key index x (0..64 NB - 1 <-> key q0 - 64 (NB - 1) + x) -> row of the ring
+    auto ring_row = [&](int x) {
+      int blk = oldest + (x >> 6);
+      blk = blk >= NB ? blk - NB : blk;
+      return blk * kQTile + (x & (kQTile - 1));
+    };
     __syncthreads();  // the staged rows are visible
     if constexpr (ROPE) {
 #pragma unroll
@@ -202,10 +216,10 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
     }
 
     // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
-    // wavefront w sees staged keys 16 w .. 16 w + 79 (tile i = keys 16 w + 16 i ..)
-    f32x4 st[5];
+    // wavefront w sees staged keys 16 w .. 16 w + 16 NT - 1 (tile i = keys 16 w + 16 i ..)
+    f32x4 st[NT];
 #pragma unroll
-    for (int i = 0; i < 5; ++i) {
+    for (int i = 0; i < NT; ++i) {
       const __bf16* row = s_k + (ring_row(16 * wave + 16 * i) + col) * kKStride + 8 * grp;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -217,10 +231,10 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
     // ---- masked softmax over keys; lane holds keys 16 i + 4 grp + r of query n ----
     float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 5; ++i)
+    for (int i = 0; i < NT; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int key = n0 - 64 + 16 * i + 4 * grp + r;
+        const int key = n0 - 64 * (NB - 1) + 16 * i + 4 * grp + r;
         const bool keep = key >= 0 && key <= n && key >= n - w_left;
         const float sc = keep ? st[i][r] * scale_log2e : -INFINITY;
         st[i][r] = sc;
@@ -230,7 +244,7 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 5; ++i)
+    for (int i = 0; i < NT; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float p = __builtin_amdgcn_exp2f(st[i][r] - mx);  // exp2(-inf) = 0 for masked keys
@@ -240,7 +254,7 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
 
-    // ---- O^T = V^T P^T: 4 channel tiles x 3 key slabs of 32 (last slab half empty) ----
+    // ---- O^T = V^T P^T: 4 channel tiles x NS key slabs of 32 (last slab half empty) ----
     // V^T operand tiles come from the row-major V rows with the transposing 64-bit LDS read:
     // in each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
     // loaded, so source lane 4j + a fetches channels 4a..4a+3 of key j of the group's four.
@@ -249,12 +263,12 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
 #pragma unroll
     for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent for s = 2)
+    for (int s = 0; s < NS; ++s) {
+      // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent in the last slab)
       u32x4 pb;
       pb[0] = pack_bf16(st[2 * s][0], st[2 * s][1]);
       pb[1] = pack_bf16(st[2 * s][2], st[2 * s][3]);
-      if (s < 2) {
+      if (s < NS - 1) {
         pb[2] = pack_bf16(st[2 * s + 1][0], st[2 * s + 1][1]);
         pb[3] = pack_bf16(st[2 * s + 1][2], st[2 * s + 1][3]);
       } else {
@@ -263,12 +277,12 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
       }
       const bf16x8 bp = __builtin_bit_cast(bf16x8, pb);
       const __bf16* lo_rows = s_v + ring_row(16 * wave + 32 * s) * kVStride + vt_off;
-      const __bf16* hi_rows = s_v + ring_row((16 * wave + 32 * s + 16) & (2 * kQTile - 1)) * kVStride + vt_off;
+      const __bf16* hi_rows = s_v + ring_row(s < NS - 1 ? 16 * wave + 32 * s + 16 : 0) * kVStride + vt_off;
 #pragma unroll
       for (int et = 0; et < 4; ++et) {
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + 16 * et));
         s16x4 hi = {0, 0, 0, 0};
-        if (s < 2)
+        if (s < NS - 1)
           hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + 16 * et));
         const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
@@ -277,8 +291,8 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
 
     // ---- normalise; stage the 16 x 64 tile in LDS so each lane stores 16 contiguous bytes ----
     const float inv = 1.0f / sum;
-    __syncthreads();  // every wavefront is done with the left block
-    __bf16* so = s_k + ((1 - own) * kQTile + 16 * wave) * kKStride;
+    __syncthreads();  // every wavefront is done with the oldest block
+    __bf16* so = s_k + (oldest * kQTile + 16 * wave) * kKStride;
 #pragma unroll
     for (int et = 0; et < 4; ++et) {
       const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
@@ -295,9 +309,9 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
       if (n0 + row < L) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(o + (long)(n0 + row) * o_sl + 8 * (lane & 7)));
     }
 
-    // ---- the left block takes the next tile's rows (this wavefront's own 16 rows of it) ----
+    // ---- the oldest block takes the next tile's rows (this wavefront's own 16 rows of it) ----
     if (tile + 1 < tile_end) {
-      store_rows(1 - own, q0 + kQTile, pre, true);
+      store_rows(oldest, q0 + kQTile, pre, true);
       if constexpr (!ROPE) {
         bq[0] = bq_next[0];
         bq[1] = bq_next[1];
@@ -317,10 +331,12 @@ __global__ __launch_bounds__(256, ROPE ? 3 : 4) void swa_prefill_kernel(
 }
 
 // One workgroup of four wavefronts per (b, h).  Keys lo..pos, lo = max(0, pos - w_left): at most
-// 64 cached rows plus the new token.  Every global load of the step (K rows for the scores,
-// V rows for the output) is issued before anything is waited on, so the step costs one memory
-// round trip: thread t scores key t/4 over channels 16 (t%4)..+16, and accumulates channel t%64
-// over the keys congruent to t/64 mod 4.
+// 64 KB cached rows plus the new token (KB = 1 for windows of up to 64 to the left, 2 for up to
+// 128).  Every global load of the step (K rows for the scores, V rows for the output) is issued
+// before anything is waited on, so the step costs one memory round trip: thread t scores keys
+// t/4 (+64) over channels 16 (t%4)..+16, and accumulates channel t%64 over the keys congruent to
+// t/64 mod 4.
+template <int KB>
 __global__ __launch_bounds__(256) void swa_step_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k_new, const __bf16* __restrict__ v_new,
     __bf16* __restrict__ kcache, __bf16* __restrict__ vcache, __bf16* __restrict__ o,
@@ -328,7 +344,8 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
     long q_sh, long kn_sb, long kn_sh, long vn_sb, long vn_sh, long o_sb, long o_sh, long c_sb,
     long c_st, long c_sh, int w_left, float scale_log2e, const float* __restrict__ rope_cos,
     const float* __restrict__ rope_sin, int rope_len) {
-  __shared__ float s_p[80];          // scores, then weights; entry 64 is the new token
+  constexpr int kCached = 64 * KB;   // most cached rows a step reads
+  __shared__ float s_p[kCached + 16];  // scores, then weights; entry kCached is the new token
   __shared__ float s_part[4][kHeadDim];
   __shared__ __align__(16) float s_qrot[4][kHeadDim];  // rotated query, one private copy per wavefront
   const int tid = threadIdx.x;
@@ -349,15 +366,19 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
   __bf16* kc = kcache + b * c_sb + h * c_sh;
   __bf16* vc = vcache + b * c_sb + h * c_sh;
   const int lo = pos - w_left > 0 ? pos - w_left : 0;
-  const int ncached = pos - lo;  // 0..64 rows of the cache, then the new token itself
+  const int ncached = pos - lo;  // 0..kCached rows of the cache, then the new token itself
 
   // ---- issue every load of the step ----
-  const int kj = tid >> 2, kq4 = tid & 3;  // key and channel quarter for the scores
-  bf16x8 kx[2] = {{0, 0, 0, 0, 0, 0, 0, 0}, {0, 0, 0, 0, 0, 0, 0, 0}};
-  if (kj < ncached) {
-    const bf16x8* row = reinterpret_cast<const bf16x8*>(kc + (long)(lo + kj) * c_st + 16 * kq4);
-    kx[0] = row[0];
-    kx[1] = row[1];
+  const int kj = tid >> 2, kq4 = tid & 3;  // key (and key + 64) and channel quarter for the scores
+  bf16x8 kx[KB][2];
+#pragma unroll
+  for (int g = 0; g < KB; ++g) {
+    kx[g][0] = kx[g][1] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if (kj + 64 * g < ncached) {
+      const bf16x8* row = reinterpret_cast<const bf16x8*>(kc + (long)(lo + kj + 64 * g) * c_st + 16 * kq4);
+      kx[g][0] = row[0];
+      kx[g][1] = row[1];
+    }
   }
   const bf16x8* qrow = reinterpret_cast<const bf16x8*>(q + b * q_sb + h * q_sh + 16 * kq4);
   const bf16x8 qx[2] = {qrow[0], qrow[1]};
@@ -366,16 +387,17 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
     cs = rope_cos[(long)pos * (kHeadDim / 2) + (lane & 31)];
     sn = rope_sin[(long)pos * (kHeadDim / 2) + (lane & 31)];
   }
-  float vv[17];
+  constexpr int kPerWave = kCached / 4;  // keys of this wavefront: j = wave, wave + 4, ...
+  float vv[kPerWave];
 #pragma unroll
-  for (int u = 0; u < 17; ++u) {
-    const int j = 4 * u + wave;  // keys of this wavefront: j = wave, wave + 4, ...
+  for (int u = 0; u < kPerWave; ++u) {
+    const int j = 4 * u + wave;
     vv[u] = j < ncached ? to_f32(vc[(long)(lo + j) * c_st + lane]) : 0.f;
   }
   float kn = to_f32(k_new[b * kn_sb + h * kn_sh + lane]);
   const float vn = to_f32(v_new[b * vn_sb + h * vn_sh + lane]);
   float ql = to_f32(q[b * q_sb + h * q_sh + lane]);
-  // this wavefront's slice of the query for the scores: 16 channels from 16 kq4
+  // this thread's slice of the query for the scores: 16 channels from 16 kq4
   float qf[16];
 #pragma unroll
   for (int c = 0; c < 2; ++c)
@@ -408,36 +430,49 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
   }
 
   // ---- scores ----
-  float part = 0.f;
 #pragma unroll
-  for (int c = 0; c < 2; ++c)
+  for (int g = 0; g < KB; ++g) {
+    float part = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) part = __builtin_fmaf(to_f32(kx[c][i]), qf[8 * c + i], part);
-  part += __shfl_xor(part, 1, 64);
-  part += __shfl_xor(part, 2, 64);
-  if (kq4 == 0) s_p[kj] = kj < ncached ? part * scale_log2e : -INFINITY;
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) part = __builtin_fmaf(to_f32(kx[g][c][i]), qf[8 * c + i], part);
+    part += __shfl_xor(part, 1, 64);
+    part += __shfl_xor(part, 2, 64);
+    if (kq4 == 0) s_p[kj + 64 * g] = kj + 64 * g < ncached ? part * scale_log2e : -INFINITY;
+  }
   if (wave == 0) {
     const float self = wave_sum(ql * kn);
-    if (lane == 0) s_p[64] = self * scale_log2e;
+    if (lane == 0) s_p[kCached] = self * scale_log2e;
   }
   __syncthreads();
 
-  // ---- softmax over the 65 entries (every wavefront redundantly: no second barrier) ----
-  const float s0 = s_p[lane];
-  const float s1 = s_p[64];
-  float mx = fmaxf(s0, s1);
+  // ---- softmax over the kCached + 1 entries (every wavefront redundantly: no second barrier) ----
+  float sc[KB], pw[KB];
+  const float s1 = s_p[kCached];
+  float mx = s1;
+#pragma unroll
+  for (int g = 0; g < KB; ++g) {
+    sc[g] = s_p[lane + 64 * g];
+    mx = fmaxf(mx, sc[g]);
+  }
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-  const float p0 = __builtin_amdgcn_exp2f(s0 - mx);
   const float p1 = __builtin_amdgcn_exp2f(s1 - mx);
-  const float denom = wave_sum(p0) + p1;
+  float psum = 0.f;
+#pragma unroll
+  for (int g = 0; g < KB; ++g) {
+    pw[g] = __builtin_amdgcn_exp2f(sc[g] - mx);
+    psum += pw[g];
+  }
+  const float denom = wave_sum(psum) + p1;
 
   // ---- output: channel = lane, this wavefront's keys ----
   float acc = wave == 0 ? p1 * vn : 0.f;
 #pragma unroll
-  for (int u = 0; u < 17; ++u) {
+  for (int u = 0; u < kPerWave; ++u) {
     const int j = 4 * u + wave;
-    const float p = __shfl(p0, j & 63, 64);
+    const float p = __shfl(pw[u >> 4], j & 63, 64);  // key j sits in group j / 64 = u / 16
     acc = __builtin_fmaf(j < ncached ? p : 0.f, vv[u], acc);
   }
   s_part[wave][lane] = acc;
@@ -449,6 +484,12 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
 }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static size_t swa_prefill_lds_bytes(int nb, bool rope) {
+  return sizeof(__bf16) * ((size_t)nb * kQTile * (kKStride + kVStride) + (rope ? kQTile * kKStride : 0));
+}
+constexpr int kMaxDevices = 64;
+static std::atomic<bool> g_big_lds_allowed[kMaxDevices];  // only one variant (rotary, three blocks) needs it
 
 }  // namespace based
 
@@ -482,8 +523,8 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   }
   BASED_REQUIRE(B >= 0 && H > 0 && L >= 0, BASED_ERR_ARG, "swa_prefill: bad sizes");
   BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_prefill: only bf16 is supported");
-  BASED_REQUIRE(w_left >= 0 && w_left <= 64, BASED_ERR_SHAPE,
-                "swa_prefill: left window %d unsupported (0..64)", w_left);
+  BASED_REQUIRE(w_left >= 0 && w_left <= 128, BASED_ERR_SHAPE,
+                "swa_prefill: left window %d unsupported (0..128)", w_left);
   BASED_REQUIRE(H < 65536 && B < 65536 && L < (1ll << 31) - 64, BASED_ERR_SHAPE,
                 "swa_prefill: grid too large");
   const int64_t strides[] = {q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl, o_sh};
@@ -501,8 +542,24 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
   const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
   dim3 grid((unsigned)(B * H * runs_per_seq)), block(256);
-  auto kern = rope_cos ? swa_prefill_kernel<true> : swa_prefill_kernel<false>;
-  hipLaunchKernelGGL(kern, grid, block, 0, static_cast<hipStream_t>(stream),
+  const int nb = w_left > 64 ? 3 : 2;
+  auto kern = nb == 3 ? (rope_cos ? swa_prefill_kernel<true, 3> : swa_prefill_kernel<false, 3>)
+                      : (rope_cos ? swa_prefill_kernel<true, 2> : swa_prefill_kernel<false, 2>);
+  const size_t lds = swa_prefill_lds_bytes(nb, rope_cos != nullptr);
+  if (lds > 64 * 1024) {
+    // above the default cap a kernel has to be told once per device that it may ask for more
+    int dev = 0;
+    BASED_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, BASED_ERR_LAUNCH,
+                  "swa_prefill: cannot identify the current device");
+    if (!g_big_lds_allowed[dev].load(std::memory_order_acquire)) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      BASED_REQUIRE(e == hipSuccess, BASED_ERR_LAUNCH, "swa_prefill: cannot raise the LDS limit to %zu bytes: %s", lds,
+                    hipGetErrorString(e));
+      g_big_lds_allowed[dev].store(true, std::memory_order_release);
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, block, lds, static_cast<hipStream_t>(stream),
                      (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o, (int)H, (int)L,
                      (int)n_tiles, (int)run_tiles, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb,
                      o_sl, o_sh, w_left, scale * 1.4426950408889634f, rope_cos, rope_sin,
@@ -533,8 +590,8 @@ extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const 
   }
   BASED_REQUIRE(B >= 0 && H > 0 && max_seqlen > 0, BASED_ERR_ARG, "swa_step: bad sizes");
   BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_step: only bf16 is supported");
-  BASED_REQUIRE(w_left >= 0 && w_left <= 64, BASED_ERR_SHAPE,
-                "swa_step: left window %d unsupported (0..64)", w_left);
+  BASED_REQUIRE(w_left >= 0 && w_left <= 128, BASED_ERR_SHAPE,
+                "swa_step: left window %d unsupported (0..128)", w_left);
   BASED_REQUIRE(max_seqlen < (1ll << 31) && B * H < (1ll << 31), BASED_ERR_SHAPE, "swa_step: sizes too large");
   if (!cache_seqlens)
     BASED_REQUIRE(pos_host >= 0 && pos_host < max_seqlen, BASED_ERR_ARG,
@@ -545,7 +602,7 @@ extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const 
   BASED_REQUIRE(aligned16(kcache) && aligned16(q), BASED_ERR_ALIGN,
                 "swa_step: kcache and q must be 16-byte aligned");
   if (B == 0) return BASED_OK;
-  hipLaunchKernelGGL(swa_step_kernel, dim3((unsigned)(B * H)), dim3(256), 0,
+  hipLaunchKernelGGL(w_left > 64 ? swa_step_kernel<2> : swa_step_kernel<1>, dim3((unsigned)(B * H)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), (const __bf16*)q, (const __bf16*)k_new,
                      (const __bf16*)v_new, (__bf16*)kcache, (__bf16*)vcache, (__bf16*)o, cache_seqlens,
                      (int)pos_host, (int)H, (int)max_seqlen, q_sb, q_sh, kn_sb, kn_sh, vn_sb, vn_sh,

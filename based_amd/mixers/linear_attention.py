@@ -73,9 +73,12 @@ class LinearAttention(nn.Module):
         self.layer_idx = layer_idx
         self.d_model = d_model
         self.l_max = l_max
-        self.eps = eps
-        # Accepted for config compatibility; there is exactly one implementation here.
+        # Accepted for config compatibility; there is exactly one implementation here.  The one
+        # thing the name changes is the regulariser of the denominator: the reference's "fla_*"
+        # paths use 1e-6 instead of `eps`, in the parallel kernel they call and in the recurrent
+        # step (linear_attention.py:199-212,245-249); so does this module.
         self.parallel_implementation = parallel_implementation
+        self.eps = 1e-6 if "fla" in parallel_implementation else eps
 
         self.num_heads = num_heads
         self.head_dim = self.d_model // self.num_heads if head_dim is None else head_dim

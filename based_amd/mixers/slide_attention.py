@@ -115,8 +115,8 @@ class SlidingAttention(nn.Module):
         self.return_residual = return_residual
         self.checkpointing = checkpointing
         self.window = (window_size // 2, 0)
-        if self.window[0] > 64:
-            raise NotImplementedError(f"left window {self.window[0]} > 64 is not built into the kernels")
+        if self.window[0] > 128:
+            raise NotImplementedError(f"left window {self.window[0]} > 128 is not built into the kernels")
 
         self.num_heads = num_heads
         self.num_heads_kv = num_heads

@@ -106,9 +106,11 @@ class StackConfig(SimpleNamespace):
 
 
 def based_360m_config(**overrides) -> StackConfig:
-    """Shape of the released Based-360m: BaseConv everywhere except Taylor linear attention at
-    layers {1,6,11,16,21} and sliding-window attention at {2,7,12,17,22}
-    (train/configs/experiment/reference/based-360m.yaml:53-65), window 64 to the left."""
+    """The 360M-scale benchmark stack: the layer plan of the released Based-360m (BaseConv everywhere
+    except Taylor linear attention at layers {1,6,11,16,21} and sliding-window attention at
+    {2,7,12,17,22}; train/configs/experiment/reference/based-360m.yaml:53-65) with window_size 128,
+    i.e. 64 keys to the left, and no rotary.  The released checkpoint itself uses window_size 256
+    and rotary over the whole head: `based_360m_released_config`."""
     cfg = dict(
         n_embd=1024, n_layer=27, n_head=16, n_inner=2048, vocab_size=50277,
         mixer={"_target_": "based.models.mixers.convolution.BaseConv", "l_max": 2048, "use_bias": True,
@@ -121,6 +123,19 @@ def based_360m_config(**overrides) -> StackConfig:
                      "num_heads": 16, "causal": True},
         alt_mixer_2_layers=[2, 7, 12, 17, 22],
     )
+    cfg.update(overrides)
+    return StackConfig(**cfg)
+
+
+def based_360m_released_config(**overrides) -> StackConfig:
+    """The model section of train/configs/experiment/reference/based-360m.yaml:49-115 as written:
+    window_size 256 (128 keys to the left), rotary_emb_fraction 1, parallel_implementation
+    "fla_parallel" on the linear-attention layers, everything else as `based_360m_config`."""
+    cfg = vars(based_360m_config())
+    cfg = {k: (dict(v) if isinstance(v, dict) else v) for k, v in cfg.items()}
+    cfg["alt_mixer"]["parallel_implementation"] = "fla_parallel"
+    cfg["alt_mixer_2"]["window_size"] = 256
+    cfg.update(rotary_emb_fraction=1, n_positions=2048, max_position_embeddings=0)
     cfg.update(overrides)
     return StackConfig(**cfg)
 

@@ -155,7 +155,8 @@ BASED_API int based_linear_attn_prefill_split_static(const void* q, const void* 
  * 206-213.  Query i attends keys j in [i - w_left, i].
  *
  * q, k, v, o : element (b,l,h,c) at p[b*sb + l*sl + h*sh + c], c < 64 contiguous.
- * head dim is 64; 0 <= w_left <= 64 (pass window_size // 2 of the module).  bf16 only.
+ * head dim is 64; 0 <= w_left <= 128 (pass window_size // 2 of the module; the released
+ * checkpoints use 128).  bf16 only.
  *
  * rope_cos, rope_sin : NULL, or fp32 tables (rope_len, 32) of cos / sin(position * inv_freq[i]):
  *   q and k are rotated inside the kernel (non-interleaved rotary over the whole head:

@@ -332,7 +332,9 @@ def stack_forward(input_ids, sd: dict, config: dict, dtype=torch.float32):
             k = F.linear(hidden, g(m + "proj_k.weight")).view(B, L, H, fd).transpose(1, 2)
             v = F.linear(hidden, g(m + "proj_v.weight")).view(B, L, H, -1).transpose(1, 2)
             # fp32 arithmetic on the (dtype-rounded) projections, like the kernels (module header, F9)
-            y = linear_attn_quadratic(q.float(), k.float(), v.float(), eps=spec.get("eps", 1e-12))
+            # the reference's "fla_*" implementations regularise with 1e-6 (linear_attention.py:199-212,245-249)
+            lin_eps = 1e-6 if "fla" in spec.get("parallel_implementation", "") else spec.get("eps", 1e-12)
+            y = linear_attn_quadratic(q.float(), k.float(), v.float(), eps=lin_eps)
             y = y.transpose(1, 2).reshape(B, L, -1)
             hidden = F.linear(y.to(dtype), g(m + "out_proj.weight"))
         else:

@@ -53,7 +53,7 @@ def test_argument_validation_without_gpu():
     rc = lib.based_linear_attn_step(p, p, p, p, p, p, 1, 1, 40, 0, 0, 0, 0, 0, 0, 0, 0, 1e-12, 0, None)
     assert rc == 1
     # window too wide -> BASED_ERR_SHAPE
-    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 65, 0.125, None, None, 0, None, None, 0, 0, 0, 0, 0, None)
+    rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 129, 0.125, None, None, 0, None, None, 0, 0, 0, 0, 0, None)
     assert rc == 1
     # fp32 is not a sliding-window element type -> BASED_ERR_DTYPE (2)
     rc = lib.based_swa_prefill(p, p, p, p, 1, 1, 8, 0, 64, 64, 0, 64, 64, 0, 64, 64, 0, 64, 64, 64, 0.125, None, None, 0, None, None, 0, 0, 0, 0, 1, None)

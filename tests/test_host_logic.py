@@ -44,8 +44,9 @@ def test_sliding_attention_parameters_and_cache():
     assert m.allocate_inference_cache(3, 77).shape == (3, 77, 2, 16, 64)
     with pytest.raises(NotImplementedError):
         SlidingAttention(embed_dim=1024, num_heads=16, num_heads_kv=4)
+    assert SlidingAttention(embed_dim=1024, num_heads=16, window_size=256).window == (128, 0)   # the released configs
     with pytest.raises(NotImplementedError):
-        SlidingAttention(embed_dim=1024, num_heads=16, window_size=256)
+        SlidingAttention(embed_dim=1024, num_heads=16, window_size=258)
     with pytest.raises(NotImplementedError):
         SlidingAttention(embed_dim=512, num_heads=16)
 

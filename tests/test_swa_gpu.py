@@ -16,7 +16,10 @@ def _qkv(B, L, H, seed, scale=1.0):
 
 
 @pytest.mark.parametrize("B,L,H,w", [(2, 256, 3, 64), (1, 1, 2, 64), (1, 65, 1, 64), (1, 100, 2, 64),
-                                     (1, 130, 2, 17), (2, 64, 2, 0), (1, 333, 4, 64), (1, 1024, 16, 64)])
+                                     (1, 130, 2, 17), (2, 64, 2, 0), (1, 333, 4, 64), (1, 1024, 16, 64),
+                                     # left windows past 64 (three staged key blocks); lengths either side of 128/129/256
+                                     (1, 128, 2, 128), (1, 129, 2, 128), (2, 130, 2, 128), (1, 256, 3, 128), (1, 257, 2, 128),
+                                     (1, 300, 2, 65), (1, 200, 2, 100), (1, 1, 1, 128), (1, 700, 16, 128), (2, 2048, 4, 128)])
 def test_prefill_matches_oracle(dev, B, L, H, w):
     from based_amd import ops
 
@@ -31,6 +34,29 @@ def test_prefill_matches_oracle(dev, B, L, H, w):
     assert rel_l2(out.float(), ref.float()) < TOL
 
 
+@pytest.mark.parametrize("w", [0, 1, 63, 64, 65, 100, 127, 128])
+def test_window_edges_are_exact(dev, w):
+    """q = 0 makes every visible key weigh the same, so the output is the plain mean of the V rows in
+    [i - w, i]: one key too many or too few moves it by 1/(w+1) of a row, far above this bound."""
+    from based_amd import ops
+
+    B, L, H = 1, 400, 2
+    qkv = _qkv(B, L, H, seed=7)
+    qkv[:, :, 0] = 0
+    v = qkv[:, :, 2].float()
+    ref = torch.stack([v[:, max(0, i - w): i + 1].mean(dim=1) for i in range(L)], dim=1)
+    qd = qkv.to(dev)
+    out = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w)
+    assert rel_l2(out.float(), ref) < 3e-3
+    # and the decode step at positions around the window width
+    cache = torch.zeros(B, L, 2, H, 64, dtype=torch.bfloat16, device=dev)
+    cache[:, :, 0] = qd[:, :, 1]
+    cache[:, :, 1] = qd[:, :, 2]
+    for t in sorted({0, 1, max(w - 1, 0), w, w + 1, w + 2, 2 * w + 1, L - 1}):
+        o = ops.swa_step(qd[:, t:t + 1, 0], qd[:, t:t + 1, 1], qd[:, t:t + 1, 2], cache, t, w_left=w)
+        assert rel_l2(o.float(), ref[:, t:t + 1]) < 3e-3, f"step at {t}"
+
+
 def test_prefill_large_scores(dev):
     """Scores with a wide dynamic range (|s| up to ~60): softmax must stay finite."""
     from based_amd import ops
@@ -43,7 +69,8 @@ def test_prefill_large_scores(dev):
     assert rel_l2(out.float(), ref.float()) < TOL
 
 
-@pytest.mark.parametrize("P,T,w", [(0, 70, 64), (60, 12, 64), (200, 5, 64), (10, 10, 7)])
+@pytest.mark.parametrize("P,T,w", [(0, 70, 64), (60, 12, 64), (200, 5, 64), (10, 10, 7), (0, 140, 128), (120, 20, 128),
+                                   (250, 10, 128), (60, 80, 100), (60, 10, 65)])
 def test_decode_matches_prefill_oracle(dev, P, T, w):
     """Decode steps after a P-token prefill equal the parallel oracle at each position
     (the reference's own cached == uncached invariant)."""
@@ -79,10 +106,12 @@ def test_rejects(dev):
         ops.swa_prefill(x, x, x)  # head dim 32
     y = torch.zeros(1, 4, 2, 64, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
-        ops.swa_prefill(y, y, y, w_left=65)
+        ops.swa_prefill(y, y, y, w_left=129)
     cache = torch.zeros(1, 8, 2, 2, 64, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         ops.swa_step(y[:, :1], y[:, :1], y[:, :1], cache, 8)  # position outside the cache
+    with pytest.raises(ValueError):
+        ops.swa_step(y[:, :1], y[:, :1], y[:, :1], cache, 2, w_left=129)
 
 
 def _rope_tables(n_pos, dev):
@@ -91,7 +120,8 @@ def _rope_tables(n_pos, dev):
     return ang.cos().contiguous().to(dev), ang.sin().contiguous().to(dev)
 
 
-@pytest.mark.parametrize("B,L,H,w", [(2, 256, 3, 64), (1, 1, 2, 64), (1, 100, 2, 64), (1, 333, 4, 20), (1, 1024, 8, 64)])
+@pytest.mark.parametrize("B,L,H,w", [(2, 256, 3, 64), (1, 1, 2, 64), (1, 100, 2, 64), (1, 333, 4, 20), (1, 1024, 8, 64),
+                                     (2, 257, 3, 128), (1, 129, 2, 128), (1, 1024, 8, 128), (1, 333, 4, 90)])
 def test_prefill_with_rotary_and_cache_output(dev, B, L, H, w):
     """Rotary inside the kernel == rotating q, k first (oracle RoPE, rounded to bf16 like the
     reference's rotated tensors); the optional cache output holds the rotated k and v."""
@@ -121,7 +151,7 @@ def test_prefill_with_rotary_and_cache_output(dev, B, L, H, w):
     assert torch.equal(cache2.cpu()[:, :L], qkv[:, :, 1:])
 
 
-@pytest.mark.parametrize("P,T,w", [(0, 70, 64), (130, 6, 64), (10, 10, 7)])
+@pytest.mark.parametrize("P,T,w", [(0, 70, 64), (130, 6, 64), (10, 10, 7), (0, 135, 128), (200, 8, 128), (100, 40, 128)])
 def test_decode_with_rotary_matches_parallel(dev, P, T, w):
     """Prefill P tokens into the cache with in-kernel rotary, then rotary decode steps (host and
     device positions): every step equals the parallel oracle on the rotated sequence."""
