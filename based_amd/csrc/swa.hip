@@ -126,10 +126,10 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
       r.kp[i] = r.vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
       if constexpr (ROPE) r.qp[i] = z4;
       if (key >= 0 && key < L) {
-        r.kp[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(k + (long)key * k_sl + piece_ch(i)));
-        r.vp[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(v + (long)key * v_sl + piece_ch(i)));
+        r.kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + piece_ch(i));
+        r.vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + piece_ch(i));
         if constexpr (ROPE)
-          if (with_q) r.qp[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(q + (long)key * q_sl + piece_ch(i)));
+          if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q + (long)key * q_sl + piece_ch(i));
       }
     }
     if constexpr (ROPE) {
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
 #pragma unroll
     for (int ds = 0; ds < 2; ++ds) {
       bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (n < L) x = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp));
+      if (n < L) x = *reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp);
       bq[ds] = x;
     }
   };

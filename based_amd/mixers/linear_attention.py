@@ -13,6 +13,7 @@ import math
 
 import torch
 import torch.nn as nn
+import torch.nn.functional as F
 
 from .. import ops
 from ..generation import InferenceParams
@@ -98,7 +99,14 @@ class LinearAttention(nn.Module):
     def forward(self, hidden_states: torch.Tensor, inference_params: InferenceParams = None, *args, **kwargs):
         """hidden_states (b, l, d_model) -> (b, l, d_model)."""
         b, l, _ = hidden_states.size()
-        q, k, v = self.proj_q(hidden_states), self.proj_k(hidden_states), self.proj_v(hidden_states)
+        if l == 1 and inference_params is not None and not torch.is_grad_enabled():
+            # a decode step is bound by launches, not by arithmetic: one GEMM over the stacked
+            # projection weights instead of three
+            nq = self.feature_dim * self.num_heads
+            qkv = F.linear(hidden_states, self._stacked_qkv_weight())
+            q, k, v = qkv[..., :nq], qkv[..., nq:2 * nq], qkv[..., 2 * nq:]
+        else:
+            q, k, v = self.proj_q(hidden_states), self.proj_k(hidden_states), self.proj_v(hidden_states)
         q = q.view(b, l, self.num_heads, self.feature_dim).transpose(1, 2)
         k = k.view(b, l, self.num_heads, self.feature_dim).transpose(1, 2)
         v = v.view(b, l, self.num_heads, self.head_dim).transpose(1, 2)
@@ -118,6 +126,17 @@ class LinearAttention(nn.Module):
         else:
             inference_params.key_value_memory_dict[self.layer_idx] = (kv_state, k_state)
         return y
+
+    def _stacked_qkv_weight(self) -> torch.Tensor:
+        """[proj_q; proj_k; proj_v] weights as one matrix, rebuilt whenever one of them has been
+        written to or replaced (tensor version counters and storage addresses are the key)."""
+        ws = (self.proj_q.weight, self.proj_k.weight, self.proj_v.weight)
+        key = tuple((w.data_ptr(), w._version) for w in ws)
+        cached = getattr(self, "_qkv_cache", None)
+        if cached is None or cached[0] != key:
+            cached = (key, torch.cat([w.detach() for w in ws], dim=0))
+            self._qkv_cache = cached
+        return cached[1]
 
     def parallel_forward(self, x: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
         """q, k: (b, h, l, 16) raw; v: (b, h, l, head_dim).  Returns out_proj(y), plus the decode

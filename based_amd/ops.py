@@ -22,7 +22,15 @@ def _dtype_code(t: torch.Tensor) -> int:
     raise ValueError(f"unsupported dtype {t.dtype} (bfloat16 or float32)")
 
 
+# torch's current stream on a device as a raw hipStream_t.  The private accessor skips building a
+# Stream object (several microseconds per call, which a single-token step notices); where a torch
+# build lacks it the public route is taken.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(t: torch.Tensor) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
@@ -339,24 +347,33 @@ def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool 
     """Prenorm block glue in one launch: r = x + residual (r = x when residual is None),
     y = rms_norm(r cast to x.dtype) * weight, and r itself (fp32 when residual_in_fp32, else
     x.dtype).  x: (..., D) with contiguous rows; returns (y, r) with r None if not wanted."""
-    _require_cuda(x, weight)
     D = x.shape[-1]
-    if weight.shape != (D,) or weight.dtype != x.dtype:
-        raise ValueError(f"weight must be ({D},) of {x.dtype}, got {tuple(weight.shape)} {weight.dtype}")
-    x2 = x.reshape(-1, D)
+    key = ("add_rms_norm", x.shape, x.stride(), x.dtype, x.device, weight.shape, weight.dtype, weight.device,
+           None if residual is None else (residual.shape, residual.stride(), residual.dtype, residual.device))
+    if key not in _CHECKED:
+        _require_cuda(x, weight)
+        if weight.shape != (D,) or weight.dtype != x.dtype or not weight.is_contiguous():
+            raise ValueError(f"weight must be a contiguous ({D},) of {x.dtype}, got {tuple(weight.shape)} {weight.dtype}")
+        if residual is not None:
+            _require_cuda(x, residual)
+            if residual.shape != x.shape:
+                raise ValueError(f"residual {tuple(residual.shape)} does not match x {tuple(x.shape)}")
+            if x.dtype == torch.float32 and residual.dtype != torch.float32:
+                raise ValueError("fp32 activations need an fp32 residual stream")
+            if residual.dtype not in (torch.float32, torch.bfloat16):
+                raise ValueError(f"unsupported residual dtype {residual.dtype}")
+        _dtype_code(x)
+        _CHECKED[key] = True
+    x2 = x if x.dim() == 2 else x.reshape(-1, D)
     if x2.stride(-1) != 1:
         x2 = x2.contiguous()
     rows = x2.shape[0]
     res_dtype = torch.float32 if residual_in_fp32 else x.dtype
     r2 = None
     if residual is not None:
-        _require_cuda(x, residual)
-        if residual.shape != x.shape:
-            raise ValueError(f"residual {tuple(residual.shape)} does not match x {tuple(x.shape)}")
-        if residual.dtype != res_dtype:
-            # a residual stream of another dtype (first block with residual_in_fp32=False, ...)
-            res_dtype = residual.dtype
-        r2 = residual.reshape(-1, D)
+        # a residual stream of another dtype (first block with residual_in_fp32=False, ...) keeps its own
+        res_dtype = residual.dtype
+        r2 = residual if residual.dim() == 2 else residual.reshape(-1, D)
         if r2.stride(-1) != 1:
             r2 = r2.contiguous()
     if x.dtype == torch.float32 and res_dtype != torch.float32:
@@ -368,7 +385,7 @@ def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool 
         _lib.check(_lib.lib().based_add_rms_norm(
             x2.data_ptr(), r2.data_ptr() if r2 is not None else None, weight.data_ptr(), y.data_ptr(),
             out.data_ptr() if out is not None else None, rows, D, x2.stride(0),
-            r2.stride(0) if r2 is not None else 0, y.stride(0), out.stride(0) if out is not None else 0,
+            r2.stride(0) if r2 is not None else 0, D, D if out is not None else 0,
             float(eps), _dtype_code(x), res_code, _stream_ptr(x)))
     return y.view(x.shape), (out.view(x.shape) if out is not None else None)
 

@@ -183,9 +183,10 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     qn = torch.randn(B, 1, 3, H, 64, generator=g).bfloat16().to(dev)
     o1 = torch.empty(B, 1, H, 64, dtype=torch.bfloat16, device=dev)
     pos = [L]
+    q1, k1, v1 = qn[:, :, 0], qn[:, :, 1], qn[:, :, 2]
 
     def dstep():
-        ops.swa_step(qn[:, :, 0], qn[:, :, 1], qn[:, :, 2], cache, pos[0], w_left=64, out=o1)
+        ops.swa_step(q1, k1, v1, cache, pos[0], w_left=64, out=o1)
         pos[0] = L + (pos[0] + 1 - L) % decode_steps
 
     dms, _ = _events_ms(torch, dstep, decode_steps, 8)
