@@ -1,19 +1,27 @@
 // Sliding-window causal softmax attention for gfx950: prefill (MFMA) and decode step.
 //
-// Prefill.  One workgroup of four wavefronts covers 64 consecutive queries of one
-// (batch, head); wavefront w owns queries [q0+16w, q0+16w+16) and the keys
-// [n0-64(NB-1), n0+16) they can see: NB = 2 staged blocks of 64 rows for a window of up to 64 to
-// the left (80 keys, 5 tiles), NB = 3 for up to 128 (144 keys, 9 tiles), plus the causal diagonal.
-//   S^T = K Q^T   : 5 or 9 key tiles x 2 MFMA 16x16x32 (head dim 64); the workgroup's K rows are
-//                   staged once in LDS (a lane's operand = 8 consecutive bf16 of one row).
+// Prefill.  Four wavefronts cover 64 consecutive queries of one (batch, head); wavefront w owns
+// queries [q0+16w, q0+16w+16) and the keys [n0-64(NB-1), n0+16) they can see: NB = 2 staged
+// blocks of 64 rows for a window of up to 64 to the left (80 keys, 5 tiles), NB = 3 for up to 128
+// (144 keys, 9 tiles), plus the causal diagonal.
+//   S^T = K Q^T   : 5 or 9 key tiles x 2 MFMA 16x16x32 (head dim 64); the K rows are staged once
+//                   in LDS (a lane's operand = 8 consecutive bf16 of one row).
 //   softmax       : S^T leaves the MFMA with lane <-> query and registers <-> keys, so the
 //                   row max / row sum are in-lane loops plus two cross-lane steps.
 //   O^T = V^T P^T : the accumulator layout of S^T is already the B-operand layout for a
 //                   product contracted over keys, so P never leaves registers.  V^T (lane
 //                   <-> channel, registers <-> keys) is the one operand that needs a
 //                   transpose: V rows are staged as they come and read with the transposing
-//                   LDS load.  Outputs leave through LDS as full 128-byte rows.
+//                   LDS load.  Outputs go out from registers: two lane groups trade channel
+//                   tiles with a row swap, after which every lane stores 2 x 16 contiguous bytes.
 // Whole-window softmax in one pass: 80 (144) keys fit in registers, so no online rescaling.
+// A workgroup holds G such wavefront quartets, one per head of G heads that are neighbours in
+// memory (G = 2 when the head stride is 64 elements): their rows of one token are one contiguous
+// 128 G-byte piece, and HBM serves pieces of 256 bytes measurably better than pieces of 128
+// (a plain streaming kernel with this access pattern: 4.4 TB/s at 128 bytes, 4.9 at 256).
+// LDS rows are 128 bytes, unpadded; the 16-byte pieces of a row are XOR-swizzled by the row
+// number so that the operand reads (16 rows x 16 bytes, or 8 rows x 32 bytes for the transposing
+// read) fall on distinct banks.
 //
 // Decode.  One workgroup of four wavefronts per (batch, head) against the last w_left+1 rows of
 // a linear cache, with every load issued up front (one memory round trip per step).
@@ -24,14 +32,20 @@
 namespace based {
 
 constexpr int kHeadDim = 64;
-constexpr int kQTile = 64;          // queries per workgroup
-constexpr int kKStride = 72;        // bf16 per K row in LDS (144 B: 16 rows x 16 B reads hit 64 distinct banks)
-constexpr int kVStride = 80;        // bf16 per V row in LDS (160 B: conflict-free transposing reads)
-constexpr int kOStride = 72;        // bf16 per row of a wavefront's output staging tile
+constexpr int kQTile = 64;          // queries per wavefront quartet
+constexpr int kRowBytes = 128;      // a K, V or Q row in LDS
 
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+// 16-byte piece p (0..7) of LDS row r sits at piece p ^ swizzle(r).
+//   K and Q rows are read as MFMA operands, 16 consecutive rows x one piece each: rows r and r+1
+//   differ in the bank half (128-byte rows), rows of the same parity need 8 different pieces.
+//   V rows are read by the transposing load, 8 consecutive rows x two neighbouring pieces each:
+//   rows of the same parity need 4 different piece pairs.
+__device__ __forceinline__ int swz_k(int row) { return (row >> 1) & 7; }
+__device__ __forceinline__ int swz_v(int row) { return ((row >> 1) & 3) << 1; }
 
 // bf16 pair (x1 at channel c < 32, x2 at channel c + 32) -> rotated pair, rounded to bf16
 __device__ __forceinline__ void rope_rotate8(u32x4& lo, u32x4& hi, const f32x4 (&cs)[2], const f32x4 (&sn)[2]) {
@@ -56,80 +70,90 @@ __device__ __forceinline__ void rope_rotate8(u32x4& lo, u32x4& hi, const f32x4 (
 }
 
 // One tile's worth of rows on their way from global memory to LDS (register prefetch).
-template <bool ROPE> struct SwaRows {
-  u32x4 kp[2], vp[2];
+struct SwaRows {
+  u32x4 kp[2], vp[2], qp[2];  // qp: only when the queries go through LDS
+  f32x4 cs[2], sn[2];         // rotary factors (ROPE only)
 };
-template <> struct SwaRows<true> {
-  u32x4 kp[2], vp[2], qp[2];
-  f32x4 cs[2], sn[2];
-};
+
+constexpr int swa_head_lds_bytes(int nb) { return (2 * nb + 1) * kQTile * kRowBytes; }
 
 // ROPE: q and k are rotated on their way into LDS (non-interleaved rotary over the whole head,
 // cos/sin tables of 32 frequencies per position), as flash-attn's rotary layer does before the
 // attention of the reference (slide_attention.py:346-355,553-556).
 // kc_out / vc_out (optional): the (rotated) K rows and the V rows of this call are also written
 // to a KV cache, the job of _update_kv_cache (slide_attention.py:255-281).
-template <bool ROPE, int NB>
-__global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill_kernel(
+// G > 1 needs q_sh == k_sh == v_sh == o_sh == c_sh == 64 and H % G == 0 (checked by the launcher).
+template <bool ROPE, int NB, int G>
+__global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4))) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
     int w_left, float scale_log2e, const float* __restrict__ rope_cos, const float* __restrict__ rope_sin,
     __bf16* __restrict__ kc_out, __bf16* __restrict__ vc_out, long c_sb, long c_st, long c_sh) {
-  // A ring of NB blocks of 64 K rows and 64 V rows: one holds the current tile's own keys, the
-  // others the 64 (NB - 1) keys to its left.  Moving on by one tile, "own" becomes "left" without
-  // a copy and the oldest block takes the next tile's rows.
+  // Per head: a ring of NB blocks of 64 K rows, the same of V rows, and (ROPE) the 64 rotated
+  // queries.  One block holds the current tile's own keys, the others the 64 (NB - 1) keys to its
+  // left.  Moving on by one tile, "own" becomes "left" without a copy and the oldest block takes
+  // the next tile's rows.
   constexpr int NT = 4 * (NB - 1) + 1;   // key tiles of 16 a wavefront sees
   constexpr int NS = (NT + 1) / 2;       // key slabs of 32 in the second product (last one half empty)
-  // (dynamic LDS: the three-block ring with rotated queries is past the 64 KB static limit)
+  constexpr int kHeadBytes = swa_head_lds_bytes(NB);
+  constexpr int kOffV = NB * kQTile * kRowBytes;
+  constexpr int kOffQ = 2 * kOffV;
   extern __shared__ __align__(16) unsigned char swa_lds[];
-  __bf16* const s_k = reinterpret_cast<__bf16*>(swa_lds);
-  __bf16* const s_v = s_k + NB * kQTile * kKStride;
-  __bf16* const s_q = s_v + NB * kQTile * kVStride;  // rotated queries (ROPE only)
-  static_assert(kOStride == kKStride, "output staging reuses whole K rows of the oldest block");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wq = wave & 3;     // which 16 of the tile's 64 queries
+  const int hsel = wave >> 2;  // which of the workgroup's G heads
   const int col = lane & 15;   // query (B operand / accumulator column), or row of an A tile
   const int grp = lane >> 4;   // 0..3: which 8 contraction slots / which 4 accumulator rows
 
-  // work item: a run of up to run_tiles consecutive query tiles of one (batch, head)
+  // work item: a run of up to run_tiles consecutive query tiles of G neighbouring heads of one batch entry
   const int runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
   const int run = (int)(blockIdx.x % runs_per_seq);
-  const long bh = blockIdx.x / runs_per_seq;
-  const int h = (int)(bh % H), b = (int)(bh / H);
+  const long bhg = blockIdx.x / runs_per_seq;
+  const int hg = (int)(bhg % (H / G)), b = (int)(bhg / (H / G));
   const int tile_begin = run * run_tiles;
   const int tile_end = tile_begin + run_tiles < n_tiles ? tile_begin + run_tiles : n_tiles;
 
-  q += b * q_sb + h * q_sh;
-  k += b * k_sb + h * k_sh;
-  v += b * v_sb + h * v_sh;
-  o += b * o_sb + h * o_sh;
-  if (kc_out != nullptr) {
-    kc_out += b * c_sb + h * c_sh;
-    vc_out += b * c_sb + h * c_sh;
-  }
+  // rows are moved by lane-dependent heads (head0 + mv_head); the products are per wavefront (head0 + hsel)
+  const long head0 = (long)hg * G;
+  unsigned char* const my = swa_lds + hsel * kHeadBytes;
 
-  // Pieces (row of a 64-row block, first channel) moved by this thread, 16 bytes each.  A
-  // wavefront only ever writes block rows 16 wave .. 16 wave + 15, the rows that double as its
-  // output staging tile.  Plain: rows 16 wave + 8 i + lane / 8, channels 8 (lane % 8).
-  // ROPE: one row, 16 wave + lane / 4, and the two channel groups 8 (lane % 4) + 32 i that the
-  // rotation pairs up.
-  auto piece_row = [&](int i) { return ROPE ? 16 * wave + (lane >> 2) : 16 * wave + 8 * i + (lane >> 3); };
-  auto piece_ch = [&](int i) { return ROPE ? 8 * (lane & 3) + 32 * i : 8 * (lane & 7); };
-  auto load_rows = [&](int key0, SwaRows<ROPE>& r, bool with_q) {
+  // Pieces (row of a 64-row block, 16-byte piece, head) moved by this thread.  The G wavefronts
+  // with the same wq move the rows 16 wq .. 16 wq + 15 of all G heads between them, every load
+  // instruction covering whole 128 G-byte pieces of memory.
+  //   plain: instruction i of 2 moves 8/G rows x G heads x 8 pieces
+  //   ROPE : one row per 4 G lanes, pieces p and p + 4 (the channel pairs of the rotation)
+  const int mv_head = ROPE ? (lane >> 2) % G : (lane >> 3) % G;
+  auto piece_row = [&](int i) {
+    return ROPE ? 16 * wq + (16 / G) * hsel + lane / (4 * G) : 16 * wq + (16 / G) * hsel + (8 / G) * i + lane / (8 * G);
+  };
+  auto piece_idx = [&](int i) { return ROPE ? (lane & 3) + 4 * i : (lane & 7); };
+  const __bf16* const q_mv = q + b * q_sb + (head0 + mv_head) * q_sh;
+  const __bf16* const k_mv = k + b * k_sb + (head0 + mv_head) * k_sh;
+  const __bf16* const v_mv = v + b * v_sb + (head0 + mv_head) * v_sh;
+  __bf16* kc_mv = nullptr;
+  __bf16* vc_mv = nullptr;
+  if (kc_out != nullptr) {
+    kc_mv = kc_out + b * c_sb + (head0 + mv_head) * c_sh;
+    vc_mv = vc_out + b * c_sb + (head0 + mv_head) * c_sh;
+  }
+  unsigned char* const mv_lds = swa_lds + mv_head * kHeadBytes;
+  __bf16* const o_my = o + b * o_sb + (head0 + hsel) * o_sh;
+
+  auto load_rows = [&](int key0, SwaRows& r, bool with_q) {
     const u32x4 z4 = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int key = key0 + piece_row(i);
       r.kp[i] = r.vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
-      if constexpr (ROPE) r.qp[i] = z4;
+      r.qp[i] = z4;
       if (key >= 0 && key < L) {
-        r.kp[i] = *reinterpret_cast<const u32x4*>(k + (long)key * k_sl + piece_ch(i));
-        r.vp[i] = *reinterpret_cast<const u32x4*>(v + (long)key * v_sl + piece_ch(i));
-        if constexpr (ROPE)
-          if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q + (long)key * q_sl + piece_ch(i));
+        r.kp[i] = *reinterpret_cast<const u32x4*>(k_mv + (long)key * k_sl + 8 * piece_idx(i));
+        r.vp[i] = *reinterpret_cast<const u32x4*>(v_mv + (long)key * v_sl + 8 * piece_idx(i));
+        if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q_mv + (long)key * q_sl + 8 * piece_idx(i));
       }
     }
     if constexpr (ROPE) {
@@ -148,59 +172,54 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
     }
   };
   // own_rows: the rows are the tile's own keys (they also carry its queries and go to the cache)
-  auto store_rows = [&](int blk, int key0, SwaRows<ROPE>& r, bool own_rows) {
+  auto store_rows = [&](int blk, int key0, SwaRows& r, bool own_rows) {
     if constexpr (ROPE) {
       rope_rotate8(r.kp[0], r.kp[1], r.cs, r.sn);
       if (own_rows) rope_rotate8(r.qp[0], r.qp[1], r.cs, r.sn);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      const int row = blk * kQTile + piece_row(i);
-      *reinterpret_cast<u32x4*>(s_k + row * kKStride + piece_ch(i)) = r.kp[i];
-      *reinterpret_cast<u32x4*>(s_v + row * kVStride + piece_ch(i)) = r.vp[i];
-      if constexpr (ROPE)
-        if (own_rows) *reinterpret_cast<u32x4*>(s_q + piece_row(i) * kKStride + piece_ch(i)) = r.qp[i];
-      const int key = key0 + piece_row(i);
-      if (own_rows && kc_out != nullptr && key < L) {
-        *reinterpret_cast<u32x4*>(kc_out + (long)key * c_st + piece_ch(i)) = r.kp[i];
-        *reinterpret_cast<u32x4*>(vc_out + (long)key * c_st + piece_ch(i)) = r.vp[i];
+      const int lrow = piece_row(i);
+      const int row = blk * kQTile + lrow;
+      const int pc = piece_idx(i);
+      *reinterpret_cast<u32x4*>(mv_lds + row * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.kp[i];
+      *reinterpret_cast<u32x4*>(mv_lds + kOffV + row * kRowBytes + ((pc ^ swz_v(lrow)) << 4)) = r.vp[i];
+      if (own_rows) *reinterpret_cast<u32x4*>(mv_lds + kOffQ + lrow * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.qp[i];
+      const int key = key0 + lrow;
+      if (own_rows && kc_mv != nullptr && key < L) {
+        *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
+        *reinterpret_cast<u32x4*>(vc_mv + (long)key * c_st + 8 * pc) = r.vp[i];
       }
     }
   };
-  // Q operand of this wavefront's 16 queries, straight from global memory (plain variant)
-  auto load_q = [&](int q0, bf16x8 (&bq)[2]) {
-    const int n = q0 + 16 * wave + col;
-#pragma unroll
-    for (int ds = 0; ds < 2; ++ds) {
-      bf16x8 x = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (n < L) x = *reinterpret_cast<const bf16x8*>(q + (long)n * q_sl + 32 * ds + 8 * grp);
-      bq[ds] = x;
-    }
-  };
-
   int q0 = tile_begin * kQTile;
-  SwaRows<ROPE> pre;
-  bf16x8 bq[2], bq_next[2];
+  SwaRows pre;
   {
     // first tile: own rows in block 0, the keys 64 a to the left in block NB - a (one round trip)
-    SwaRows<ROPE> left[NB - 1];
+    SwaRows left[NB - 1];
 #pragma unroll
     for (int a = 1; a < NB; ++a) load_rows(q0 - a * kQTile, left[a - 1], false);
     load_rows(q0, pre, true);
-    if constexpr (!ROPE) load_q(q0, bq);
 #pragma unroll
     for (int a = 1; a < NB; ++a) store_rows(NB - a, q0 - a * kQTile, left[a - 1], false);
     store_rows(0, q0, pre, true);
   }
   if (tile_begin + 1 < tile_end) {  // the next tile's rows travel while this one is computed
     load_rows(q0 + kQTile, pre, true);
-    if constexpr (!ROPE) load_q(q0 + kQTile, bq_next);
   }
+
+  // lane-constant parts of the operand addresses (rows of a tile start at multiples of 16)
+  const int k_lane = col * kRowBytes;                  // + ((4 ds + grp) ^ swz_k(col)) << 4
+  const int k_sw = swz_k(col);
+  const int vt_row = 4 * grp + (col >> 2);             // row of a 16-row tile this lane fetches for the transposing read
+  const int v_lane = vt_row * kRowBytes + 8 * (col & 1);
+  const int v_sw = swz_v(vt_row);
+  const int v_half = (col & 3) >> 1;                   // piece 2 et + v_half
 
   int own = 0;  // ring block with keys [q0, q0+64); block own + 1 (mod NB) is the oldest
   for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile, own = own + 1 == NB ? 0 : own + 1) {
     const int oldest = own + 1 == NB ? 0 : own + 1;
-    const int n0 = q0 + 16 * wave;            // first query of this wavefront
+    const int n0 = q0 + 16 * wq;              // first query of this wavefront
     const int n = n0 + col;                   // this lane's query
     // staged key index x (0..64 NB - 1 <-> key q0 - 64 (NB - 1) + x) -> row of the ring
     auto ring_row = [&](int x) {
@@ -209,22 +228,23 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
       return blk * kQTile + (x & (kQTile - 1));
     };
     __syncthreads();  // the staged rows are visible
-    if constexpr (ROPE) {
+    unsigned char* const q_rows = my + kOffQ + 16 * wq * kRowBytes;  // this wavefront's 16 query rows
+    bf16x8 bq[2];
 #pragma unroll
-      for (int ds = 0; ds < 2; ++ds)
-        bq[ds] = *reinterpret_cast<const bf16x8*>(s_q + (16 * wave + col) * kKStride + 32 * ds + 8 * grp);
-    }
+    for (int ds = 0; ds < 2; ++ds)
+      bq[ds] = *reinterpret_cast<const bf16x8*>(q_rows + k_lane + (((4 * ds + grp) ^ k_sw) << 4));
 
     // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
     // wavefront w sees staged keys 16 w .. 16 w + 16 NT - 1 (tile i = keys 16 w + 16 i ..)
     f32x4 st[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-      const __bf16* row = s_k + (ring_row(16 * wave + 16 * i) + col) * kKStride + 8 * grp;
+      const unsigned char* row = my + ring_row(16 * wq + 16 * i) * kRowBytes + k_lane;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ds = 0; ds < 2; ++ds)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(row + 32 * ds), bq[ds], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *reinterpret_cast<const bf16x8*>(row + (((4 * ds + grp) ^ k_sw) << 4)), bq[ds], acc, 0, 0, 0);
       st[i] = acc;
     }
 
@@ -258,7 +278,6 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
     // V^T operand tiles come from the row-major V rows with the transposing 64-bit LDS read:
     // in each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
     // loaded, so source lane 4j + a fetches channels 4a..4a+3 of key j of the group's four.
-    const int vt_off = (4 * grp + (col >> 2)) * kVStride + 4 * (col & 3);
     f32x4 ot[4];
 #pragma unroll
     for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -276,28 +295,29 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
         pb[3] = 0u;
       }
       const bf16x8 bp = __builtin_bit_cast(bf16x8, pb);
-      const __bf16* lo_rows = s_v + ring_row(16 * wave + 32 * s) * kVStride + vt_off;
-      const __bf16* hi_rows = s_v + ring_row(s < NS - 1 ? 16 * wave + 32 * s + 16 : 0) * kVStride + vt_off;
+      const unsigned char* lo_rows = my + kOffV + ring_row(16 * wq + 32 * s) * kRowBytes + v_lane;
+      const unsigned char* hi_rows = my + kOffV + ring_row(s < NS - 1 ? 16 * wq + 32 * s + 16 : 0) * kRowBytes + v_lane;
 #pragma unroll
       for (int et = 0; et < 4; ++et) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + 16 * et));
+        const int pc = ((2 * et + v_half) ^ v_sw) << 4;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + pc));
         s16x4 hi = {0, 0, 0, 0};
         if (s < NS - 1)
-          hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + 16 * et));
+          hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + pc));
         const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
       }
     }
 
-    // ---- normalise; stage the 16 x 64 tile in LDS so each lane stores 16 contiguous bytes ----
+    // ---- normalise; the 16 x 64 tile goes through the wavefront's own query rows (read above, not
+    // needed again, and rewritten only after the barrier below) so that every lane stores 16
+    // bytes of a full 128-byte row ----
     const float inv = 1.0f / sum;
-    __syncthreads();  // every wavefront is done with the oldest block
-    __bf16* so = s_k + (oldest * kQTile + 16 * wave) * kKStride;
 #pragma unroll
     for (int et = 0; et < 4; ++et) {
       const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
       const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
-      *reinterpret_cast<uint2*>(so + col * kOStride + 16 * et + 4 * grp) = make_uint2(w0, w1);
+      *reinterpret_cast<uint2*>(q_rows + k_lane + (((2 * et + (grp >> 1)) ^ k_sw) << 4) + 8 * (grp & 1)) = make_uint2(w0, w1);
     }
     // the tile is re-read below in another lane layout: order the wavefront's own LDS accesses
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -305,26 +325,21 @@ __global__ __launch_bounds__(256, NB == 3 ? 2 : (ROPE ? 3 : 4)) void swa_prefill
 #pragma unroll
     for (int hlf = 0; hlf < 2; ++hlf) {
       const int row = 8 * hlf + (lane >> 3);
-      const u32x4 w4 = *reinterpret_cast<const u32x4*>(so + row * kOStride + 8 * (lane & 7));
-      if (n0 + row < L) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(o + (long)(n0 + row) * o_sl + 8 * (lane & 7)));
+      const u32x4 w4 = *reinterpret_cast<const u32x4*>(q_rows + row * kRowBytes + (((lane & 7) ^ swz_k(row)) << 4));
+      if (n0 + row < L) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(o_my + (long)(n0 + row) * o_sl + 8 * (lane & 7)));
     }
 
-    // ---- the oldest block takes the next tile's rows (this wavefront's own 16 rows of it) ----
+    // ---- the oldest block takes the next tile's rows ----
     if (tile + 1 < tile_end) {
+      __syncthreads();  // every wavefront is done with the oldest block
       store_rows(oldest, q0 + kQTile, pre, true);
-      if constexpr (!ROPE) {
-        bq[0] = bq_next[0];
-        bq[1] = bq_next[1];
-      }
       if (tile + 2 < tile_end) {
         load_rows(q0 + 2 * kQTile, pre, true);
-        // Measured: letting these loads overlap the next tile's compute is SLOWER (B=32:
-        // 264 us vs 247 us).  With 1024 workgroups resident, one more tile in flight per
-        // workgroup (24 MB in total) only lengthens the HBM queues; waiting here keeps the
-        // request stream of a workgroup in bursts of one tile, and the other workgroups of
-        // the compute unit cover the latency.
+        // Measured: letting these loads overlap the next tile's compute is SLOWER.  With every
+        // compute unit full of workgroups, one more tile in flight per workgroup only lengthens
+        // the HBM queues; waiting here keeps the request stream of a workgroup in bursts of one
+        // tile, and the other workgroups of the compute unit cover the latency.
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (!ROPE) load_q(q0 + 2 * kQTile, bq_next);
       }
     }
   }
@@ -485,11 +500,9 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-static size_t swa_prefill_lds_bytes(int nb, bool rope) {
-  return sizeof(__bf16) * ((size_t)nb * kQTile * (kKStride + kVStride) + (rope ? kQTile * kKStride : 0));
-}
 constexpr int kMaxDevices = 64;
-static std::atomic<bool> g_big_lds_allowed[kMaxDevices];  // only one variant (rotary, three blocks) needs it
+// kernels asking for more than 64 KB of LDS have to be told once per device that they may
+static std::atomic<bool> g_big_lds_allowed[kMaxDevices][2 /*ROPE*/][2 /*NB - 2*/][2 /*G - 1*/];
 
 }  // namespace based
 
@@ -541,22 +554,33 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   int64_t run_tiles = B * H * n_tiles / 1024;
   run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
   const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
-  dim3 grid((unsigned)(B * H * runs_per_seq)), block(256);
+  // Two heads per workgroup when they are neighbours in every tensor (the packed qkv layout) and
+  // the ring is the two-block one; the three-block ring keeps one head per workgroup (LDS).
+  const bool rope = rope_cos != nullptr;
   const int nb = w_left > 64 ? 3 : 2;
-  auto kern = nb == 3 ? (rope_cos ? swa_prefill_kernel<true, 3> : swa_prefill_kernel<false, 3>)
-                      : (rope_cos ? swa_prefill_kernel<true, 2> : swa_prefill_kernel<false, 2>);
-  const size_t lds = swa_prefill_lds_bytes(nb, rope_cos != nullptr);
+  const bool pair = nb == 2 && H % 2 == 0 && q_sh == 64 && k_sh == 64 && v_sh == 64 && o_sh == 64 &&
+                    (!kcache_out || c_sh == 64);
+  const int g = pair ? 2 : 1;
+  dim3 grid((unsigned)(B * (H / g) * runs_per_seq)), block(256 * g);
+  using Kern = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int, int, int, int, long, long, long, long,
+                        long, long, long, long, long, long, long, long, int, float, const float*, const float*, __bf16*,
+                        __bf16*, long, long, long);
+  Kern kern;
+  if (nb == 3) kern = rope ? swa_prefill_kernel<true, 3, 1> : swa_prefill_kernel<false, 3, 1>;
+  else if (g == 2) kern = rope ? swa_prefill_kernel<true, 2, 2> : swa_prefill_kernel<false, 2, 2>;
+  else kern = rope ? swa_prefill_kernel<true, 2, 1> : swa_prefill_kernel<false, 2, 1>;
+  const size_t lds = (size_t)g * swa_head_lds_bytes(nb);
   if (lds > 64 * 1024) {
-    // above the default cap a kernel has to be told once per device that it may ask for more
     int dev = 0;
     BASED_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, BASED_ERR_LAUNCH,
                   "swa_prefill: cannot identify the current device");
-    if (!g_big_lds_allowed[dev].load(std::memory_order_acquire)) {
+    std::atomic<bool>& allowed = g_big_lds_allowed[dev][rope][nb - 2][g - 1];
+    if (!allowed.load(std::memory_order_acquire)) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       BASED_REQUIRE(e == hipSuccess, BASED_ERR_LAUNCH, "swa_prefill: cannot raise the LDS limit to %zu bytes: %s", lds,
                     hipGetErrorString(e));
-      g_big_lds_allowed[dev].store(true, std::memory_order_release);
+      allowed.store(true, std::memory_order_release);
     }
   }
   hipLaunchKernelGGL(kern, grid, block, lds, static_cast<hipStream_t>(stream),
