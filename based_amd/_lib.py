@@ -56,6 +56,9 @@ SIGNATURES = {
         C.c_int,
         [_P, _P, _P, _P, _P] + [_I64] * 2 + [C.c_int] + [_I64] * 2 + [C.c_int, C.c_int, _P],
     ),
+    "based_probe_stream_qkv": (C.c_int, [_P, _P, _I64, _I64, _I64, C.c_int, _P]),
+    "based_probe_rmw": (C.c_int, [_P, _I64, _P]),
+    "based_probe_copy": (C.c_int, [_P, _P, _I64, _P]),
     "based_add_rms_norm": (
         C.c_int,
         [_P, _P, _P, _P, _P] + [_I64] * 6 + [C.c_float, C.c_int, C.c_int, _P],

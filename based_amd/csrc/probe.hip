@@ -1,0 +1,114 @@
+// Measurement probes: plain streaming kernels with the memory access patterns of the hot kernels
+// and no arithmetic to speak of.  What they reach on a given machine is the ceiling the real
+// kernels are measured against next to the published HBM figure (the benchmark reports both).
+//   stream_qkv : reads a packed (B, L, 3, H, 64) bf16 tensor and writes a (B, L, H, 64) one the way
+//                the window-attention prefill does: a workgroup walks a run of tokens of G
+//                neighbouring heads, every load instruction covering whole 128 G-byte pieces.
+//   rmw        : reads and rewrites a float buffer in 16-byte pieces, lane-contiguous, like the
+//                state update of the recurrent decode step.
+//   copy       : plain 16-byte-per-lane copy of known size; the calibration kernel for the
+//                profiler's HBM byte counters.
+#include "common.hpp"
+
+namespace based {
+
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+
+template <int G>
+__global__ __launch_bounds__(256) void probe_stream_qkv_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ o,
+                                                               int B, int H, int L, int runs) {
+  // 16-byte pieces: a token row of x holds 3*H*8 of them, one of o H*8
+  const int t = threadIdx.x;
+  const int groups = H / G;
+  int id = blockIdx.x;
+  const int run = id % runs;
+  id /= runs;
+  const int hg = id % groups, b = id / groups;
+  if (b >= B) return;
+  constexpr int kTokPerIter = 64 / G;   // 64 rows of 128 bytes per tensor and iteration, as one attention tile
+  const int toks = (L + runs - 1) / runs;
+  for (int t0 = run * toks; t0 < (run + 1) * toks && t0 < L; t0 += kTokPerIter) {
+    u32x4 a[2][3];
+    size_t oidx[2];
+    bool live[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int p = t + 256 * i;
+      const int tok = t0 + p / (8 * G), rem = p % (8 * G);
+      const int head = hg * G + rem / 8, c = rem % 8;
+      live[i] = tok < L && tok < (run + 1) * toks;
+      oidx[i] = ((size_t)b * L + tok) * H * 8 + head * 8 + c;
+#pragma unroll
+      for (int s = 0; s < 3; ++s) {
+        a[i][s] = u32x4{0, 0, 0, 0};
+        if (live[i]) a[i][s] = x[(((size_t)b * L + tok) * 3 + s) * H * 8 + head * 8 + c];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (live[i]) __builtin_nontemporal_store(a[i][0] ^ a[i][1] ^ a[i][2], o + oidx[i]);
+  }
+}
+
+template <bool WRITE>
+__global__ __launch_bounds__(256) void probe_rw_kernel(u32x4* dst, const u32x4* src, size_t n16) {
+  // grid-stride over 16-byte pieces, four in flight per lane
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += 4 * stride) {
+    u32x4 a[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      a[u] = u32x4{0, 0, 0, 0};
+      if (i + u * stride < n16) a[u] = __builtin_nontemporal_load(src + i + u * stride);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * stride < n16) __builtin_nontemporal_store(WRITE ? a[u] : a[u] + u32x4{1, 1, 1, 1}, dst + i + u * stride);
+  }
+}
+
+static bool probe_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace based
+
+extern "C" BASED_API int based_probe_stream_qkv(const void* qkv, void* o, int64_t B, int64_t H, int64_t L,
+                                                int heads_per_group, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(qkv && o, BASED_ERR_ARG, "probe_stream_qkv: null pointer argument");
+  BASED_REQUIRE(B > 0 && H > 0 && L > 0 && B < 65536 && H < 65536 && L < (1ll << 30), BASED_ERR_ARG,
+                "probe_stream_qkv: bad sizes");
+  BASED_REQUIRE(heads_per_group == 1 || heads_per_group == 2 || heads_per_group == 4, BASED_ERR_SHAPE,
+                "probe_stream_qkv: heads per group must be 1, 2 or 4");
+  BASED_REQUIRE(H % heads_per_group == 0, BASED_ERR_SHAPE, "probe_stream_qkv: H must be a multiple of the group");
+  BASED_REQUIRE(probe_aligned16(qkv) && probe_aligned16(o), BASED_ERR_ALIGN, "probe_stream_qkv: 16-byte alignment");
+  // as the attention launcher: runs long enough to leave about 1024 x 256 threads in flight
+  const int64_t n_tiles = (L + 63) / 64;
+  int64_t run_tiles = B * H * n_tiles / 1024;
+  run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
+  const int64_t runs = (n_tiles + run_tiles - 1) / run_tiles * heads_per_group;
+  const int64_t grid = B * (H / heads_per_group) * runs;
+  BASED_REQUIRE(grid < (1ll << 31), BASED_ERR_SHAPE, "probe_stream_qkv: grid too large");
+  auto kern = heads_per_group == 1 ? probe_stream_qkv_kernel<1>
+                                   : (heads_per_group == 2 ? probe_stream_qkv_kernel<2> : probe_stream_qkv_kernel<4>);
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     (const u32x4*)qkv, (u32x4*)o, (int)B, (int)H, (int)L, (int)runs);
+  return check_launch("probe_stream_qkv");
+}
+
+extern "C" BASED_API int based_probe_rmw(void* buf, int64_t bytes, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(buf && bytes > 0 && bytes % 16 == 0, BASED_ERR_ARG, "probe_rmw: need a buffer of a multiple of 16 bytes");
+  BASED_REQUIRE(probe_aligned16(buf), BASED_ERR_ALIGN, "probe_rmw: 16-byte alignment");
+  hipLaunchKernelGGL(probe_rw_kernel<false>, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     (u32x4*)buf, (const u32x4*)buf, (size_t)(bytes / 16));
+  return check_launch("probe_rmw");
+}
+
+extern "C" BASED_API int based_probe_copy(void* dst, const void* src, int64_t bytes, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(dst && src && bytes > 0 && bytes % 16 == 0, BASED_ERR_ARG, "probe_copy: need buffers of a multiple of 16 bytes");
+  BASED_REQUIRE(probe_aligned16(dst) && probe_aligned16(src), BASED_ERR_ALIGN, "probe_copy: 16-byte alignment");
+  hipLaunchKernelGGL(probe_rw_kernel<true>, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     (u32x4*)dst, (const u32x4*)src, (size_t)(bytes / 16));
+  return check_launch("probe_copy");
+}

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Based sequence-mixer hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|stack|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|stack|copy|machine]
 
 Headline workload (`value`): the recurrent decode step of Taylor linear attention at
 B=128, H=16, dv=64 — fp32 kv_state (128,16,1,64,273) + k_state, initialised from a seeded
@@ -202,6 +202,54 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     }
 
 
+def bench_machine(torch, steps=20, warmup=4, n_sets=4):
+    """What this machine's memory delivers for the access patterns of the HBM-bound kernels, measured
+    with the library's probe kernels (no arithmetic) over rotating buffers beyond the last-level
+    cache: the ceiling next to which the 8 TB/s figure should be read."""
+    from based_amd import _lib
+
+    lib = _lib.lib()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream().cuda_stream
+    out = {}
+    # state-update pattern: 145 MB read and rewritten in place per launch, like the B=128 decode step
+    n = 128 * 16 * (273 * 64 + 273) * 4 // 16 * 16
+    bufs = [torch.zeros(n, dtype=torch.uint8, device=dev) for _ in range(n_sets)]
+    it = [0]
+
+    def rmw():
+        b = bufs[it[0] % n_sets]
+        it[0] += 1
+        _lib.check(lib.based_probe_rmw(b.data_ptr(), n, stream))
+
+    ms, _ = _events_ms(torch, rmw, steps, warmup)
+    out["rmw_cold_GBps"] = round(2 * n / (ms * 1e-3) / 1e9, 1)
+    srcs = [torch.ones(n, dtype=torch.uint8, device=dev) for _ in range(n_sets)]
+
+    def cp():
+        i = it[0] % n_sets
+        it[0] += 1
+        _lib.check(lib.based_probe_copy(bufs[i].data_ptr(), srcs[i].data_ptr(), n, stream))
+
+    ms, _ = _events_ms(torch, cp, steps, warmup)
+    out["copy_cold_GBps"] = round(2 * n / (ms * 1e-3) / 1e9, 1)
+    del bufs, srcs
+    # packed-qkv pattern of the window attention (B=8, H=16, L=4096), 1 / 2 / 4 heads per workgroup
+    B, H, L = 8, 16, 4096
+    xs = [torch.ones(B, L, 3, H, 64, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+    os_ = [torch.empty(B, L, H, 64, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+    for g in (1, 2, 4):
+        def st():
+            i = it[0] % n_sets
+            it[0] += 1
+            _lib.check(lib.based_probe_stream_qkv(xs[i].data_ptr(), os_[i].data_ptr(), B, H, L, g, stream))
+
+        ms, _ = _events_ms(torch, st, steps, warmup)
+        out[f"stream_qkv_cold_GBps_{g}_heads"] = round(B * L * H * 512 / (ms * 1e-3) / 1e9, 1)
+    out["note"] = ("probe kernels of the library over %d rotating buffer sets; GB/s of bytes read + written" % n_sets)
+    return out
+
+
 def bench_conv(torch, ops, steps, warmup, B=4, L=2048, D=2048, K=3, decode_B=128):
     """Gated short convolution at the shape of the 27-layer configuration (d_inner = 2048)."""
     dev = torch.device("cuda:0")
@@ -325,9 +373,10 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "copy"], default=None,
-                    help="one workload only; 'copy' is a plain 256 MiB device copy used to calibrate the "
-                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "copy", "machine"], default=None,
+                    help="one workload only; 'copy' is a plain 256 MiB device copy (the library's copy probe) used to "
+                         "calibrate the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run; 'machine' the memory "
+                         "probes alone")
     ap.add_argument("--prefill-batches", default="1,8,32,96",
                     help="comma-separated batch sizes of the L=4096 prefill lines")
     args = ap.parse_args()
@@ -344,12 +393,20 @@ def main():
     from based_amd import ops
 
     if args.only == "copy":
+        from based_amd import _lib
+
         n = 256 * 1024 * 1024
         src = torch.empty(n, dtype=torch.uint8, device="cuda:0").fill_(1)
         dst = torch.empty_like(src)
-        ms, _ = _events_ms(torch, lambda: dst.copy_(src), args.steps, args.warmup)
-        print(json.dumps({"workload": "plain device copy", "bytes_read": n, "bytes_written": n, "ms": round(ms, 5),
-                          "GBps": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
+        stream = torch.cuda.current_stream().cuda_stream
+        ms, _ = _events_ms(torch, lambda: _lib.check(_lib.lib().based_probe_copy(dst.data_ptr(), src.data_ptr(), n, stream)),
+                           args.steps, args.warmup)
+        assert bool((dst == 1).all())
+        print(json.dumps({"workload": "plain device copy (probe_rw_kernel)", "bytes_read": n, "bytes_written": n,
+                          "ms": round(ms, 5), "GBps": round(2 * n / (ms * 1e-3) / 1e9, 1)}))
+        return
+    if args.only == "machine":
+        print(json.dumps({"machine": bench_machine(torch)}))
         return
 
     out = {
@@ -399,6 +456,8 @@ def main():
         out.update({"value": round(out["swa"]["prefill_tok_s"], 1), "ms_per_step": out["swa"]["prefill_ms"], "dtype": "bf16",
                     "config": {"workload": "configs[2]: sliding-window prefill B=8 H=16 L=4096 w=64"},
                     "roofline": out["swa"]["roofline"]})
+    if args.only is None:
+        out["machine"] = bench_machine(torch)
     if not args.no_cpu and args.only in (None, "decode"):
         out["cpu_baseline"] = cpu_baseline_decode(torch)
     if not args.no_cpu and args.only is None:
