@@ -3,11 +3,11 @@
 // Kernels behind the entry points:
 //
 //  * lin_prefill_mfma_kernel (bf16 in/out): chunked scan, 64 tokens per chunk, one workgroup
-//    of FOUR wavefronts per (batch, head, 64-channel block).  The running state stays in MFMA
-//    accumulators for the length of the sequence, split by feature slots over the four
-//    wavefronts; a bf16 image of it goes through LDS once per chunk for the read-out, which is
-//    split by tokens.  Small batches scan every sequence as concurrent segments (two passes of
-//    this kernel around lin_prefill_prefix_kernel).
+//    of EIGHT wavefronts per (batch, head, 64-channel block): four updaters keep the running
+//    state in MFMA accumulators for the length of the sequence, split by feature slots, and
+//    publish a bf16 image of it in LDS once per chunk; four readers, split by tokens, compute
+//    the outputs from the chunk's rows and the image.  Small batches scan every sequence as
+//    concurrent segments (two passes of this kernel around lin_prefill_prefix_kernel).
 //
 //      within a chunk   A = tril(1 + s + s^2/2), s = q.k/4, from a K=16 MFMA on the raw
 //                       16-dim q, k (never expanding the features), then O^T += V^T A^T
@@ -21,8 +21,8 @@
 //        element, with the weights folded into a pre-scaled copy of k;
 //      - psi(q)^T (lane <-> token, registers <-> slots) is a product of two registers with
 //        compile-time indices, because each lane group keeps q rotated by 4*group.
-//    The normaliser is carried as a 65th value channel of ones, so numerator and
-//    denominator come out of the same MFMAs.  The in-chunk weights feed their product with V
+//    The normaliser is a quadratic form in the raw q over the first and second moments of k
+//    (see below), not a 65th value channel.  The in-chunk weights feed their product with V
 //    straight from the accumulator registers (accumulator layout == B/A operand layout for a
 //    product contracted over the accumulator's row index); V needs a transpose, done by the
 //    transposing LDS read.  At the end the 160-slot state is expanded to the (dv, 273) decode

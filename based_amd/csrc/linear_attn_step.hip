@@ -10,6 +10,9 @@
 // per workgroup into LDS, in four copies shifted by 0..3 floats so that each lane's four
 // consecutive features are one aligned 128-bit LDS read; the copies run 3 entries past 273
 // and wrap, which is exactly where a float4 straddles into the next state row.
+// The state is touched once per step and is far larger than any cache when every layer has its
+// own: all 18 loads of a wavefront are non-temporal and leave at the top of the kernel, before
+// the tables are built, and the stores are non-temporal too.
 #include "common.hpp"
 
 namespace based {
