@@ -147,7 +147,9 @@ constexpr int kLoadsPerUpdater = 3;   // of the 12 wave-wide direct loads of a c
 //   kModeDelta  tokens [t_begin, t_end) only, state update only (no outputs), state starting at
 //               zero and dumped to the workspace at the end (the segment's contribution);
 //   kModeFrom   tokens [t_begin, t_end) in full, state starting from the workspace entry (the
-//               exclusive prefix over the earlier segments).
+//               exclusive prefix over the earlier segments, made by lin_prefill_prefix_kernel);
+//   kModeFromSum  the same, but the workspace still holds the segments' own contributions and
+//               the workgroup adds up the earlier ones itself (few segments: saves a launch).
 //
 // The normaliser z_i = sum_{j<=i} (1 + s_ij + s_ij^2/2), s_ij = q_i.k_j/4, is NOT carried as a
 // 65th value channel.  Over the earlier chunks it is the quadratic form
@@ -155,7 +157,7 @@ constexpr int kLoadsPerUpdater = 3;   // of the 12 wave-wide direct loads of a c
 // which costs one MFMA on the raw q (K2 as a hi + lo pair of bf16 operands) and four
 // multiply-adds per lane; inside the chunk it is the row sum of the in-chunk weights.  K2 is one
 // 16x16 accumulator tile (two MFMAs per chunk on the k^T operand that psi(k) is generated from).
-constexpr int kModeFull = 0, kModeDelta = 1, kModeFrom = 2;
+constexpr int kModeFull = 0, kModeDelta = 1, kModeFrom = 2, kModeFromSum = 3;
 // One chain's state as it goes through the workspace of the segmented scan: the accumulator image
 // of S (slot tile, channel tile, lane, 4), then the accumulators of K2 and of K1 (lane, 4 each).
 constexpr int kSegStateFloats = BASED_PREFILL_SEGMENT_STATE_BYTES / 4;
@@ -508,6 +510,21 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
     if constexpr (kNorm) {
       K2 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK2 + lane * 4);
       K1 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK1 + lane * 4);
+    }
+  }
+  if constexpr (MODE == kModeFromSum) {
+    // same order of additions as lin_prefill_prefix_kernel: ((0 + d_0) + d_1) + ...
+    const float* src = ws_mine - (long)seg * kSegStateFloats;
+    for (int sp = 0; sp < seg; ++sp, src += kSegStateFloats) {
+#pragma unroll
+      for (int i = 0; i < kOwn; ++i)
+#pragma unroll
+        for (int et = 0; et < kCTiles; ++et)
+          S[i][et] += *reinterpret_cast<const f32x4*>(src + ((own_tile(w, i) * kCTiles + et) * 64 + lane) * 4);
+      if constexpr (kNorm) {
+        K2 += *reinterpret_cast<const f32x4*>(src + kWsK2 + lane * 4);
+        K1 += *reinterpret_cast<const f32x4*>(src + kWsK1 + lane * 4);
+      }
     }
   }
 
@@ -998,6 +1015,7 @@ extern "C" BASED_API int based_linear_attn_prefill(
 // Workgroup slots of one full wave of the MFMA prefill kernel on MI355X (256 CUs x 2 resident
 // workgroups); segment counts are chosen to fill about one such wave.
 static constexpr int64_t kPrefillSlots = 512;
+static constexpr int64_t kFoldSegments = 4;   // up to this many segments the second pass sums the earlier ones itself
 
 extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, int64_t L, int64_t dv,
                                                         int io_dtype, int64_t* n_seg,
@@ -1069,11 +1087,17 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
   int rc = check_launch(who);
   if (rc) return rc;
-  hipLaunchKernelGGL(lin_prefill_prefix_kernel, dim3((unsigned)chains, (kSegStateFloats / 4 + 255) / 256), dim3(256), 0, s,
-                     ws, (int)n_seg);
-  rc = check_launch(who);
-  if (rc) return rc;
-  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)n_seg),
+  // With few segments every workgroup of the second pass adds up the contributions before its
+  // own (at most kFoldSegments - 1 reads of 42 KB, mostly from L2); with many, a prefix pass over
+  // the workspace is cheaper than every workgroup reading half of its chain's entries.
+  const bool fold = n_seg <= kFoldSegments;
+  if (!fold) {
+    hipLaunchKernelGGL(lin_prefill_prefix_kernel, dim3((unsigned)chains, (kSegStateFloats / 4 + 255) / 256), dim3(256), 0,
+                       s, ws, (int)n_seg);
+    rc = check_launch(who);
+    if (rc) return rc;
+  }
+  hipLaunchKernelGGL(fold ? lin_prefill_mfma_kernel<kModeFromSum> : lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)n_seg),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
