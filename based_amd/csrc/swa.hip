@@ -75,7 +75,8 @@ struct SwaRows {
   f32x4 cs[2], sn[2];         // rotary factors (ROPE only)
 };
 
-constexpr int swa_head_lds_bytes(int nb) { return (2 * nb + 1) * kQTile * kRowBytes; }
+// per head: the K and V rings, and with paired heads 64 query rows (see QLDS in the kernel)
+constexpr int swa_head_lds_bytes(int nb, int g) { return (2 * nb + (g > 1 ? 1 : 0)) * kQTile * kRowBytes; }
 
 // ROPE: q and k are rotated on their way into LDS (non-interleaved rotary over the whole head,
 // cos/sin tables of 32 frequencies per position), as flash-attn's rotary layer does before the
@@ -84,7 +85,7 @@ constexpr int swa_head_lds_bytes(int nb) { return (2 * nb + 1) * kQTile * kRowBy
 // to a KV cache, the job of _update_kv_cache (slide_attention.py:255-281).
 // G > 1 needs q_sh == k_sh == v_sh == o_sh == c_sh == 64 and H % G == 0 (checked by the launcher).
 template <bool ROPE, int NB, int G>
-__global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4))) void swa_prefill_kernel(
+__global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 || ROPE ? 3 : 4)) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
@@ -96,7 +97,17 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
   // the next tile's rows.
   constexpr int NT = 4 * (NB - 1) + 1;   // key tiles of 16 a wavefront sees
   constexpr int NS = (NT + 1) / 2;       // key slabs of 32 in the second product (last one half empty)
-  constexpr int kHeadBytes = swa_head_lds_bytes(NB);
+  // Where the queries and the finished output tile pass through:
+  //   paired heads (QLDS): queries are fetched with the K rows (256-byte pieces) into 64 LDS rows
+  //     of their own; a wavefront's 16 of them, free once its operand is in registers, later stage
+  //     its output tile.
+  //   one head: every lane fetches its own operand from global memory one tile ahead (and rotates
+  //     it in registers: the channel pairs c, c + 32 of the rotation are the same lane's two operand
+  //     halves); the output tile is staged in the wavefront's 16 rows of the oldest K block, which
+  //     only this wavefront rewrites.  No LDS beyond the rings: 48 KB for the three-block ring,
+  //     three workgroups per compute unit.
+  constexpr bool QLDS = G > 1;
+  constexpr int kHeadBytes = swa_head_lds_bytes(NB, G);
   constexpr int kOffV = NB * kQTile * kRowBytes;
   constexpr int kOffQ = 2 * kOffV;
   extern __shared__ __align__(16) unsigned char swa_lds[];
@@ -149,11 +160,12 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
     for (int i = 0; i < 2; ++i) {
       const int key = key0 + piece_row(i);
       r.kp[i] = r.vp[i] = z4;  // rows outside the sequence are zeros (their weights are exactly 0)
-      r.qp[i] = z4;
+      if constexpr (QLDS) r.qp[i] = z4;
       if (key >= 0 && key < L) {
         r.kp[i] = *reinterpret_cast<const u32x4*>(k_mv + (long)key * k_sl + 8 * piece_idx(i));
         r.vp[i] = *reinterpret_cast<const u32x4*>(v_mv + (long)key * v_sl + 8 * piece_idx(i));
-        if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q_mv + (long)key * q_sl + 8 * piece_idx(i));
+        if constexpr (QLDS)
+          if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q_mv + (long)key * q_sl + 8 * piece_idx(i));
       }
     }
     if constexpr (ROPE) {
@@ -175,7 +187,8 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
   auto store_rows = [&](int blk, int key0, SwaRows& r, bool own_rows) {
     if constexpr (ROPE) {
       rope_rotate8(r.kp[0], r.kp[1], r.cs, r.sn);
-      if (own_rows) rope_rotate8(r.qp[0], r.qp[1], r.cs, r.sn);
+      if constexpr (QLDS)
+        if (own_rows) rope_rotate8(r.qp[0], r.qp[1], r.cs, r.sn);
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -184,7 +197,8 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
       const int pc = piece_idx(i);
       *reinterpret_cast<u32x4*>(mv_lds + row * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.kp[i];
       *reinterpret_cast<u32x4*>(mv_lds + kOffV + row * kRowBytes + ((pc ^ swz_v(lrow)) << 4)) = r.vp[i];
-      if (own_rows) *reinterpret_cast<u32x4*>(mv_lds + kOffQ + lrow * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.qp[i];
+      if constexpr (QLDS)
+        if (own_rows) *reinterpret_cast<u32x4*>(mv_lds + kOffQ + lrow * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.qp[i];
       const int key = key0 + lrow;
       if (own_rows && kc_mv != nullptr && key < L) {
         *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
@@ -192,20 +206,47 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
       }
     }
   };
+  // one head per workgroup: the Q operand of this lane's query (channels 32 ds + 8 grp ..+7),
+  // rotated in place when ROPE
+  const __bf16* const q_my = q + b * q_sb + (head0 + hsel) * q_sh;
+  auto load_q = [&](int q0, bf16x8 (&bq)[2]) {
+    const int n = q0 + 16 * wq + col;
+    u32x4 x[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
+    f32x4 cs[2], sn[2];
+    if (n < L) {
+#pragma unroll
+      for (int ds = 0; ds < 2; ++ds) x[ds] = *reinterpret_cast<const u32x4*>(q_my + (long)n * q_sl + 32 * ds + 8 * grp);
+      if constexpr (ROPE) {
+        const f32x4* c4 = reinterpret_cast<const f32x4*>(rope_cos + (long)n * (kHeadDim / 2) + 8 * grp);
+        const f32x4* s4 = reinterpret_cast<const f32x4*>(rope_sin + (long)n * (kHeadDim / 2) + 8 * grp);
+        cs[0] = c4[0];
+        cs[1] = c4[1];
+        sn[0] = s4[0];
+        sn[1] = s4[1];
+        rope_rotate8(x[0], x[1], cs, sn);
+      }
+    }
+    bq[0] = __builtin_bit_cast(bf16x8, x[0]);
+    bq[1] = __builtin_bit_cast(bf16x8, x[1]);
+  };
+
   int q0 = tile_begin * kQTile;
   SwaRows pre;
+  bf16x8 bq[2], bq_next[2];
   {
     // first tile: own rows in block 0, the keys 64 a to the left in block NB - a (one round trip)
     SwaRows left[NB - 1];
 #pragma unroll
     for (int a = 1; a < NB; ++a) load_rows(q0 - a * kQTile, left[a - 1], false);
     load_rows(q0, pre, true);
+    if constexpr (!QLDS) load_q(q0, bq);
 #pragma unroll
     for (int a = 1; a < NB; ++a) store_rows(NB - a, q0 - a * kQTile, left[a - 1], false);
     store_rows(0, q0, pre, true);
   }
   if (tile_begin + 1 < tile_end) {  // the next tile's rows travel while this one is computed
     load_rows(q0 + kQTile, pre, true);
+    if constexpr (!QLDS) load_q(q0 + kQTile, bq_next);
   }
 
   // lane-constant parts of the operand addresses (rows of a tile start at multiples of 16)
@@ -216,6 +257,8 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
   const int v_sw = swz_v(vt_row);
   const int v_half = (col & 3) >> 1;                   // piece 2 et + v_half
 
+  // key tiles i < i_win reach below the window of the wavefront's last query (see the softmax)
+  const int i_win = w_left >= 64 * (NB - 1) + 15 ? 0 : (64 * (NB - 1) + 30 - w_left) >> 4;
   int own = 0;  // ring block with keys [q0, q0+64); block own + 1 (mod NB) is the oldest
   for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile, own = own + 1 == NB ? 0 : own + 1) {
     const int oldest = own + 1 == NB ? 0 : own + 1;
@@ -228,11 +271,13 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
       return blk * kQTile + (x & (kQTile - 1));
     };
     __syncthreads();  // the staged rows are visible
-    unsigned char* const q_rows = my + kOffQ + 16 * wq * kRowBytes;  // this wavefront's 16 query rows
-    bf16x8 bq[2];
+    // 16 rows of LDS that are this wavefront's own at the time it stages its output tile
+    unsigned char* const q_rows = QLDS ? my + kOffQ + 16 * wq * kRowBytes : my + (oldest * kQTile + 16 * wq) * kRowBytes;
+    if constexpr (QLDS) {
 #pragma unroll
-    for (int ds = 0; ds < 2; ++ds)
-      bq[ds] = *reinterpret_cast<const bf16x8*>(q_rows + k_lane + (((4 * ds + grp) ^ k_sw) << 4));
+      for (int ds = 0; ds < 2; ++ds)
+        bq[ds] = *reinterpret_cast<const bf16x8*>(q_rows + k_lane + (((4 * ds + grp) ^ k_sw) << 4));
+    }
 
     // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
     // wavefront w sees staged keys 16 w .. 16 w + 16 NT - 1 (tile i = keys 16 w + 16 i ..)
@@ -249,25 +294,34 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
     }
 
     // ---- masked softmax over keys; lane holds keys 16 i + 4 grp + r of query n ----
+    // Only three kinds of key tile contain a masked (key, query) pair, and which they are is the
+    // same for the whole wavefront: the diagonal tile (causality), the tiles that reach below
+    // n0 + 15 - w_left (the far edge of the window), and tiles before the start of the sequence.
+    // All other tiles skip the mask arithmetic.  The scale is applied inside the exponent.
     float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < NT; ++i)
+    for (int i = 0; i < NT; ++i) {
+      const int klo = n0 - 64 * (NB - 1) + 16 * i;  // first key of the tile
+      if (i == NT - 1 || i < i_win || klo < 0) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = n0 - 64 * (NB - 1) + 16 * i + 4 * grp + r;
-        const bool keep = key >= 0 && key <= n && key >= n - w_left;
-        const float sc = keep ? st[i][r] * scale_log2e : -INFINITY;
-        st[i][r] = sc;
-        mx = fmaxf(mx, sc);
+        for (int r = 0; r < 4; ++r) {
+          const int key = klo + 4 * grp + r;
+          const bool keep = key >= 0 && key <= n && key >= n - w_left;
+          st[i][r] = keep ? st[i][r] : -INFINITY;
+        }
       }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, st[i][r]);
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mxs = mx * scale_log2e;
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < NT; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(st[i][r] - mx);  // exp2(-inf) = 0 for masked keys
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i][r], scale_log2e, -mxs));  // exp2(-inf) = 0 for masked keys
         st[i][r] = p;
         sum += p;
       }
@@ -313,6 +367,7 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
     // needed again, and rewritten only after the barrier below) so that every lane stores 16
     // bytes of a full 128-byte row ----
     const float inv = 1.0f / sum;
+    if constexpr (!QLDS) __syncthreads();  // every wavefront is done with the oldest block, whose rows stage the tile
 #pragma unroll
     for (int et = 0; et < 4; ++et) {
       const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
@@ -331,10 +386,19 @@ __global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 ? 3 : (ROPE ? 3 : 4)
 
     // ---- the oldest block takes the next tile's rows ----
     if (tile + 1 < tile_end) {
-      __syncthreads();  // every wavefront is done with the oldest block
+      if constexpr (QLDS) {
+        __syncthreads();  // every wavefront is done with the oldest block
+      } else {
+        // the staged tile has been read back (same wavefront, same rows: program order suffices)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        bq[0] = bq_next[0];
+        bq[1] = bq_next[1];
+      }
       store_rows(oldest, q0 + kQTile, pre, true);
       if (tile + 2 < tile_end) {
         load_rows(q0 + 2 * kQTile, pre, true);
+        if constexpr (!QLDS) load_q(q0 + 2 * kQTile, bq_next);
         // Measured: letting these loads overlap the next tile's compute is SLOWER.  With every
         // compute unit full of workgroups, one more tile in flight per workgroup only lengthens
         // the HBM queues; waiting here keeps the request stream of a workgroup in bursts of one
@@ -548,12 +612,6 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   if (B == 0 || L == 0) return BASED_OK;
   const int64_t n_tiles = (L + kQTile - 1) / kQTile;
   BASED_REQUIRE(B * H * n_tiles < (1ll << 31), BASED_ERR_SHAPE, "swa_prefill: grid too large");
-  // Consecutive query tiles of one (batch, head) are walked by one workgroup (the keys to the left
-  // of a tile are the previous tile's own keys, already staged); runs are as long as still
-  // leaves about four workgroups for each of the 256 compute units.
-  int64_t run_tiles = B * H * n_tiles / 1024;
-  run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
-  const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
   // Two heads per workgroup when they are neighbours in every tensor (the packed qkv layout) and
   // the ring is the two-block one; the three-block ring keeps one head per workgroup (LDS).
   const bool rope = rope_cos != nullptr;
@@ -561,6 +619,15 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   const bool pair = nb == 2 && H % 2 == 0 && q_sh == 64 && k_sh == 64 && v_sh == 64 && o_sh == 64 &&
                     (!kcache_out || c_sh == 64);
   const int g = pair ? 2 : 1;
+  // Consecutive query tiles of one (batch, head) are walked by one workgroup (the keys to the left
+  // of a tile are the previous tile's own keys, already staged).  Runs are as long as still gives
+  // every resident slot of the GPU one run: 256 compute units x the wavefront quartets that fit
+  // one (4 by registers; 3 for the three-block ring, by LDS, and for the single-head rotary variant).
+  const int64_t slots = 256 * ((nb == 3 || (g == 1 && rope)) ? 3 : 4);
+  int64_t want_runs = slots / (B * H);
+  want_runs = want_runs < 1 ? 1 : (want_runs > n_tiles ? n_tiles : want_runs);
+  const int64_t run_tiles = (n_tiles + want_runs - 1) / want_runs;
+  const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
   dim3 grid((unsigned)(B * (H / g) * runs_per_seq)), block(256 * g);
   using Kern = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int, int, int, int, long, long, long, long,
                         long, long, long, long, long, long, long, long, int, float, const float*, const float*, __bf16*,
@@ -569,7 +636,7 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   if (nb == 3) kern = rope ? swa_prefill_kernel<true, 3, 1> : swa_prefill_kernel<false, 3, 1>;
   else if (g == 2) kern = rope ? swa_prefill_kernel<true, 2, 2> : swa_prefill_kernel<false, 2, 2>;
   else kern = rope ? swa_prefill_kernel<true, 2, 1> : swa_prefill_kernel<false, 2, 1>;
-  const size_t lds = (size_t)g * swa_head_lds_bytes(nb);
+  const size_t lds = (size_t)g * swa_head_lds_bytes(nb, g);
   if (lds > 64 * 1024) {
     int dev = 0;
     BASED_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, BASED_ERR_LAUNCH,
