@@ -12,8 +12,9 @@
 //                   product contracted over keys, so P never leaves registers.  V^T (lane
 //                   <-> channel, registers <-> keys) is the one operand that needs a
 //                   transpose: V rows are staged as they come and read with the transposing
-//                   LDS load.  Outputs go out from registers: two lane groups trade channel
-//                   tiles with a row swap, after which every lane stores 2 x 16 contiguous bytes.
+//                   LDS load.  The 16 x 64 output tile of a wavefront is staged in 16 LDS rows
+//                   that are its own at that moment, so that every lane stores 16 bytes of a
+//                   full 128-byte row.
 // Whole-window softmax in one pass: 80 (144) keys fit in registers, so no online rescaling.
 // A workgroup holds G such wavefront quartets, one per head of G heads that are neighbours in
 // memory (G = 2 when the head stride is 64 elements): their rows of one token are one contiguous

@@ -178,6 +178,27 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     ms = max(ms_cold, ms_warm)
     byts = B * L * H * 4 * 64 * 2
     gbs = byts / (ms * 1e-3) / 1e9
+    # the released checkpoints' window layer: 128 keys to the left, rotary over the whole head, KV cache filled
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, 64, 2, dtype=torch.float32) / 64))
+    ang = torch.outer(torch.arange(L).float(), inv_freq)
+    rope = (ang.cos().contiguous().to(dev), ang.sin().contiguous().to(dev))
+    caches = [torch.empty(B, L, 2, H, 64, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+
+    def make_rel(sets, full):
+        def pf():
+            i = it[0] % sets
+            it[0] += 1
+            x = qkvs[i]
+            if full:
+                ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=128, rope=rope, kv_cache=caches[i], out=outs[i])
+            else:
+                ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=128, out=outs[i])
+        return pf
+
+    ms_w128_cold, _ = _events_ms(torch, make_rel(n_sets, False), steps, warmup)
+    ms_w128_warm, _ = _events_ms(torch, make_rel(1, False), steps, warmup)
+    ms_rel_cold, _ = _events_ms(torch, make_rel(n_sets, True), steps, warmup)
+    del caches
     cache = torch.zeros(B, L + decode_steps, 2, H, 64, dtype=torch.bfloat16, device=dev)
     cache[:, :L] = qkv[:, :, 1:]
     qn = torch.randn(B, 1, 3, H, 64, generator=g).bfloat16().to(dev)
@@ -195,6 +216,10 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
         "B": B, "L": L, "window": 64,
         "cold": {"ms": round(ms_cold, 5), "GBps": round(byts / (ms_cold * 1e-3) / 1e9, 1), "input_sets": n_sets},
         "warm": {"ms": round(ms_warm, 5), "GBps": round(byts / (ms_warm * 1e-3) / 1e9, 1), "input_sets": 1},
+        "window_128": {"cold_ms": round(ms_w128_cold, 5), "warm_ms": round(ms_w128_warm, 5),
+                       "cold_GBps": round(byts / (ms_w128_cold * 1e-3) / 1e9, 1),
+                       "with_rotary_and_cache_fill_cold_ms": round(ms_rel_cold, 5),
+                       "note": "same inputs, 128 keys to the left (the released checkpoints' window_size 256)"},
         "roofline": {"kernel": "swa_prefill_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["swa_prefill_kernel"], "algorithmic_bytes_per_launch": byts,
