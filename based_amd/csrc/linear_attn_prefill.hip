@@ -1027,8 +1027,15 @@ extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, in
   if (io_dtype != BASED_BF16 || (dv != 64 && dv != 128) || B <= 0 || H <= 0 || L <= 0) return BASED_OK;
   const int64_t chains = B * H * (dv / 64);
   const int64_t chunks = (L + kChunk - 1) / kChunk;
-  if (chains * 3 >= kPrefillSlots * 2 || chunks < 2) return BASED_OK;  // enough chains already
-  int64_t want = (kPrefillSlots + chains - 1) / chains;
+  // Measured on MI355X at L = 4096 (best segment count per batch size): 16 chains -> 16, 32 -> 8,
+  // 48..128 -> 4, and from 192 chains on the single pass wins (one workgroup alone on a compute
+  // unit is only 12 % slower per chunk than two sharing it, so filling the second slot does not
+  // pay for the second pass over k and v).  Hence: about one workgroup per compute unit, at least
+  // four segments (up to four need no prefix launch), and for long sequences segments of at most
+  // 32 chunks while that still fits the resident slots.
+  if (chains > kPrefillSlots / 4 || chunks < 2) return BASED_OK;
+  int64_t want = chains <= 16 ? 16 : (chains <= 32 ? 8 : 4);
+  while (want * 32 < chunks && chains * want * 2 <= kPrefillSlots) want *= 2;
   if (want > chunks) want = chunks;
   int64_t seg_chunks = (chunks + want - 1) / want;
   // a segment costs about three chunks' worth of fixed work (loading its prefix, dumping or

@@ -175,6 +175,12 @@ def test_split_plan(dev):
     assert n.value == 1 and w.value == 0                     # plenty of chains: single pass
     assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
     assert 2 <= n.value <= 64 and w.value == 16 * n.value * 43008
+    assert lib.based_linear_attn_prefill_plan(8, 16, 4096, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 4                                      # few enough segments for the pass without a prefix launch
+    assert lib.based_linear_attn_prefill_plan(12, 16, 4096, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 1                                      # 192 chains: the single pass is faster
+    assert lib.based_linear_attn_prefill_plan(1, 16, 32768, 128, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 16 and w.value == 32 * 16 * 43008      # long sequence: segments of 32 chunks
     assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 64, 1, ctypes.byref(n), ctypes.byref(w)) == 0
     assert n.value == 1                                      # fp32 path is never split
     assert lib.based_linear_attn_prefill_plan(1, 16, 64, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
