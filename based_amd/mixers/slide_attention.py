@@ -5,8 +5,9 @@ constructor arguments, parameter names (Wqkv / out_proj), forward and
 allocate_inference_cache signatures and the reference's linear (B, max_seqlen, 2, H, D) KV
 cache.  `window_size=W` means query i attends keys [i - W//2, i] (flash-attn's
 `window_size=(W//2, 0)` with causal=True, slide_attention.py:332-336).
-In scope: self-attention, num_heads_kv == num_heads, head_dim 64, no dropout / padding /
-varlen; other arguments raise NotImplementedError.  Non-half inputs are computed in bf16
+In scope: self-attention, num_heads_kv == num_heads, head_dim 64, window_size up to 256 (128 keys
+to the left, what the released checkpoints use), no dropout / padding / varlen; other arguments
+raise NotImplementedError.  Non-half inputs are computed in bf16
 (the reference casts to bf16 for prefill, slide_attention.py:76-78).
 """
 from __future__ import annotations

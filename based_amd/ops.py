@@ -129,7 +129,7 @@ def _rope_tables(rope, device, need_rows):
 def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=None, kv_cache=None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Sliding-window causal attention.  q, k, v: (B, L, H, 64) bf16 (any strides with the
-    last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i].
+    last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i], 0 <= w_left <= 128.
     rope: None or (cos, sin) fp32 (n_pos >= L, 32) tables; q and k are then rotated in the kernel
     (non-interleaved rotary over the whole head, positions 0..L-1).
     kv_cache: None or a (B, max_seqlen >= L, 2, H, 64) bf16 cache whose rows 0..L-1 receive the
