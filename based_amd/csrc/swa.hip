@@ -563,6 +563,185 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Any head dimension (a multiple of 8, up to 128), fp32 arithmetic: one wavefront per query.
+// Not a performance path: it serves the head sizes the MFMA kernels are not built for (the
+// reference's own test models have 16-dim heads) and is simple enough to be read as a second
+// statement of the same attention.  Lanes run over the keys of the window for the scores and
+// over the channels for the output.
+// ------------------------------------------------------------------------------------------
+constexpr int kAnyMaxDim = 128;
+constexpr int kAnyMaxKeys = 192;   // keys a query can see, rounded up to whole wavefront passes (129 -> 3 x 64)
+
+__global__ __launch_bounds__(256) void swa_prefill_anydim_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
+    __bf16* __restrict__ o, int H, int L, int D, long n_rows, long q_sb, long q_sl, long q_sh, long k_sb, long k_sl,
+    long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh, int w_left, float scale_log2e,
+    __bf16* __restrict__ kc_out, __bf16* __restrict__ vc_out, long c_sb, long c_st, long c_sh) {
+  const int lane = threadIdx.x & 63;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, h, n) flattened, n fastest
+  if (row >= n_rows) return;
+  const int n = (int)(row % L);
+  const int h = (int)((row / L) % H);
+  const long b = row / ((long)L * H);
+  const __bf16* qr = q + b * q_sb + (long)n * q_sl + h * q_sh;
+  const __bf16* kb = k + b * k_sb + h * k_sh;
+  const __bf16* vb = v + b * v_sb + h * v_sh;
+  const int lo = n - w_left > 0 ? n - w_left : 0;
+  const int nkeys = n - lo + 1;  // 1 .. w_left + 1
+  // scores: lane j of pass p takes key lo + 64 p + j
+  float sc[kAnyMaxKeys / 64];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int p = 0; p < kAnyMaxKeys / 64; ++p) {
+    const int j = 64 * p + lane;
+    float dot = -INFINITY;
+    if (j < nkeys) {
+      const __bf16* kr = kb + (long)(lo + j) * k_sl;
+      dot = 0.f;
+      for (int c = 0; c < D; c += 8) {
+        const bf16x8 kk = *reinterpret_cast<const bf16x8*>(kr + c);
+        const bf16x8 qq = *reinterpret_cast<const bf16x8*>(qr + c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dot = __builtin_fmaf(to_f32(kk[i]), to_f32(qq[i]), dot);
+      }
+      dot *= scale_log2e;
+    }
+    sc[p] = dot;
+    mx = fmaxf(mx, dot);
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+  float psum = 0.f;
+#pragma unroll
+  for (int p = 0; p < kAnyMaxKeys / 64; ++p) {
+    sc[p] = __builtin_amdgcn_exp2f(sc[p] - mx);  // exp2(-inf) = 0 for the lanes without a key
+    psum += sc[p];
+  }
+  const float denom = wave_sum(psum);
+  // output: lane c (and c + 64) accumulates its channel over the keys
+  float acc[kAnyMaxDim / 64] = {0.f, 0.f};
+#pragma unroll
+  for (int p = 0; p < kAnyMaxKeys / 64; ++p) {
+    const int cnt = nkeys - 64 * p < 64 ? nkeys - 64 * p : 64;
+    for (int j = 0; j < cnt; ++j) {
+      const float w = __shfl(sc[p], j, 64);
+      const __bf16* vr = vb + (long)(lo + 64 * p + j) * v_sl;
+#pragma unroll
+      for (int u = 0; u < kAnyMaxDim / 64; ++u)
+        if (lane + 64 * u < D) acc[u] = __builtin_fmaf(w, to_f32(vr[lane + 64 * u]), acc[u]);
+    }
+  }
+  __bf16* orow = o + b * o_sb + (long)n * o_sl + h * o_sh;
+#pragma unroll
+  for (int u = 0; u < kAnyMaxDim / 64; ++u)
+    if (lane + 64 * u < D) orow[lane + 64 * u] = (__bf16)(acc[u] / denom);
+  if (kc_out != nullptr) {  // this token's k and v rows join the cache
+    __bf16* kc = kc_out + b * c_sb + (long)n * c_st + h * c_sh;
+    __bf16* vc = vc_out + b * c_sb + (long)n * c_st + h * c_sh;
+#pragma unroll
+    for (int u = 0; u < kAnyMaxDim / 64; ++u)
+      if (lane + 64 * u < D) {
+        kc[lane + 64 * u] = kb[(long)n * k_sl + lane + 64 * u];
+        vc[lane + 64 * u] = vb[(long)n * v_sl + lane + 64 * u];
+      }
+  }
+}
+
+// Decode step for any head dimension: one wavefront per (b, h); cache rows lo .. pos - 1 plus the new
+// token, whose k and v are used from registers and written to cache row pos.
+__global__ __launch_bounds__(64) void swa_step_anydim_kernel(
+    const __bf16* __restrict__ q, const __bf16* __restrict__ k_new, const __bf16* __restrict__ v_new,
+    __bf16* __restrict__ kcache, __bf16* __restrict__ vcache, __bf16* __restrict__ o,
+    const int32_t* __restrict__ cache_seqlens, int pos_host, int H, int D, int max_seqlen, long q_sb, long q_sh,
+    long kn_sb, long kn_sh, long vn_sb, long vn_sh, long o_sb, long o_sh, long c_sb, long c_st, long c_sh, int w_left,
+    float scale_log2e) {
+  const int lane = threadIdx.x;
+  const int b = blockIdx.x / H, h = blockIdx.x % H;
+  int pos = cache_seqlens ? cache_seqlens[b] : pos_host;
+  pos = __builtin_amdgcn_readfirstlane(pos);
+  __bf16* orow = o + b * o_sb + h * o_sh;
+  if (pos < 0 || pos >= max_seqlen) {  // see swa_step_kernel: NaN marks what the host cannot be told
+#pragma unroll
+    for (int u = 0; u < kAnyMaxDim / 64; ++u)
+      if (lane + 64 * u < D) orow[lane + 64 * u] = (__bf16)__builtin_nanf("");
+    return;
+  }
+  const __bf16* qr = q + b * q_sb + h * q_sh;
+  const __bf16* knr = k_new + b * kn_sb + h * kn_sh;
+  const __bf16* vnr = v_new + b * vn_sb + h * vn_sh;
+  __bf16* kc = kcache + b * c_sb + h * c_sh;
+  __bf16* vc = vcache + b * c_sb + h * c_sh;
+  const int lo = pos - w_left > 0 ? pos - w_left : 0;
+  const int ncached = pos - lo;  // 0 .. 128
+  float sc[2];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int j = 64 * p + lane;
+    float dot = -INFINITY;
+    if (j < ncached) {
+      const __bf16* kr = kc + (long)(lo + j) * c_st;
+      dot = 0.f;
+      for (int c = 0; c < D; c += 8) {
+        const bf16x8 kk = *reinterpret_cast<const bf16x8*>(kr + c);
+        const bf16x8 qq = *reinterpret_cast<const bf16x8*>(qr + c);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dot = __builtin_fmaf(to_f32(kk[i]), to_f32(qq[i]), dot);
+      }
+      dot *= scale_log2e;
+    }
+    sc[p] = dot;
+    mx = fmaxf(mx, dot);
+  }
+  // the new token: lanes over channels
+  float part = 0.f, vn[kAnyMaxDim / 64];
+  __bf16 kn[kAnyMaxDim / 64];
+#pragma unroll
+  for (int u = 0; u < kAnyMaxDim / 64; ++u) {
+    vn[u] = 0.f;
+    kn[u] = (__bf16)0.f;
+    if (lane + 64 * u < D) {
+      kn[u] = knr[lane + 64 * u];
+      vn[u] = to_f32(vnr[lane + 64 * u]);
+      part = __builtin_fmaf(to_f32(qr[lane + 64 * u]), to_f32(kn[u]), part);
+    }
+  }
+  const float self = wave_sum(part) * scale_log2e;
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+  mx = fmaxf(mx, self);
+  float psum = 0.f;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    sc[p] = __builtin_amdgcn_exp2f(sc[p] - mx);
+    psum += sc[p];
+  }
+  const float pself = __builtin_amdgcn_exp2f(self - mx);
+  const float denom = wave_sum(psum) + pself;
+  float acc[kAnyMaxDim / 64];
+#pragma unroll
+  for (int u = 0; u < kAnyMaxDim / 64; ++u) acc[u] = pself * vn[u];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int cnt = ncached - 64 * p < 64 ? ncached - 64 * p : 64;
+    for (int j = 0; j < cnt; ++j) {
+      const float w = __shfl(sc[p], j, 64);
+      const __bf16* vr = vc + (long)(lo + 64 * p + j) * c_st;
+#pragma unroll
+      for (int u = 0; u < kAnyMaxDim / 64; ++u)
+        if (lane + 64 * u < D) acc[u] = __builtin_fmaf(w, to_f32(vr[lane + 64 * u]), acc[u]);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < kAnyMaxDim / 64; ++u)
+    if (lane + 64 * u < D) {
+      orow[lane + 64 * u] = (__bf16)(acc[u] / denom);
+      kc[(long)pos * c_st + lane + 64 * u] = kn[u];
+      vc[(long)pos * c_st + lane + 64 * u] = (__bf16)vn[u];
+    }
+}
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 constexpr int kMaxDevices = 64;
@@ -701,4 +880,74 @@ extern "C" BASED_API int based_swa_step(const void* q, const void* k_new, const 
                      o_sb, o_sh, c_sb, c_st, c_sh, w_left, scale * 1.4426950408889634f, rope_cos, rope_sin,
                      (int)rope_len);
   return check_launch("swa_step");
+}
+
+extern "C" BASED_API int based_swa_prefill_anydim(const void* q, const void* k, const void* v, void* o,
+                                                  int64_t B, int64_t H, int64_t L, int64_t D,
+                                                  int64_t q_sb, int64_t q_sl, int64_t q_sh,
+                                                  int64_t k_sb, int64_t k_sl, int64_t k_sh,
+                                                  int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                                                  int64_t o_sb, int64_t o_sl, int64_t o_sh,
+                                                  int w_left, float scale,
+                                                  void* kcache_out, void* vcache_out,
+                                                  int64_t c_sb, int64_t c_st, int64_t c_sh, int64_t max_seqlen,
+                                                  int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(q && k && v && o, BASED_ERR_ARG, "swa_prefill_anydim: null pointer argument");
+  BASED_REQUIRE((kcache_out == nullptr) == (vcache_out == nullptr), BASED_ERR_ARG,
+                "swa_prefill_anydim: cache outputs must be given together");
+  if (kcache_out)
+    BASED_REQUIRE(L <= max_seqlen, BASED_ERR_SHAPE, "swa_prefill_anydim: %ld tokens do not fit a cache of %ld rows",
+                  (long)L, (long)max_seqlen);
+  BASED_REQUIRE(B >= 0 && H > 0 && L >= 0, BASED_ERR_ARG, "swa_prefill_anydim: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_prefill_anydim: only bf16 is supported");
+  BASED_REQUIRE(D >= 8 && D <= kAnyMaxDim && D % 8 == 0, BASED_ERR_SHAPE,
+                "swa_prefill_anydim: head dim %ld unsupported (multiples of 8 up to %d)", (long)D, kAnyMaxDim);
+  BASED_REQUIRE(w_left >= 0 && w_left <= 128, BASED_ERR_SHAPE, "swa_prefill_anydim: left window %d unsupported (0..128)",
+                w_left);
+  const int64_t strides[] = {q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh};
+  for (int64_t st : strides)
+    BASED_REQUIRE(st % 8 == 0, BASED_ERR_ALIGN, "swa_prefill_anydim: q, k, v strides must be multiples of 8 elements");
+  BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v), BASED_ERR_ALIGN,
+                "swa_prefill_anydim: q, k, v must be 16-byte aligned");
+  if (B == 0 || L == 0) return BASED_OK;
+  const int64_t n_rows = B * H * L;
+  BASED_REQUIRE((n_rows + 3) / 4 < (1ll << 31) && L < (1ll << 31), BASED_ERR_SHAPE, "swa_prefill_anydim: grid too large");
+  hipLaunchKernelGGL(swa_prefill_anydim_kernel, dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)o,
+                     (int)H, (int)L, (int)D, (long)n_rows, q_sb, q_sl, q_sh, k_sb, k_sl, k_sh, v_sb, v_sl, v_sh, o_sb, o_sl,
+                     o_sh, w_left, scale * 1.4426950408889634f, (__bf16*)kcache_out, (__bf16*)vcache_out, c_sb, c_st,
+                     c_sh);
+  return check_launch("swa_prefill_anydim");
+}
+
+extern "C" BASED_API int based_swa_step_anydim(const void* q, const void* k_new, const void* v_new,
+                                               void* kcache, void* vcache, void* o,
+                                               const int32_t* cache_seqlens, int64_t pos_host,
+                                               int64_t B, int64_t H, int64_t D, int64_t max_seqlen,
+                                               int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
+                                               int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
+                                               int64_t c_sb, int64_t c_st, int64_t c_sh,
+                                               int w_left, float scale, int io_dtype, void* stream) {
+  using namespace based;
+  BASED_REQUIRE(q && k_new && v_new && kcache && vcache && o, BASED_ERR_ARG, "swa_step_anydim: null pointer argument");
+  BASED_REQUIRE(B >= 0 && H > 0 && max_seqlen > 0, BASED_ERR_ARG, "swa_step_anydim: bad sizes");
+  BASED_REQUIRE(io_dtype == BASED_BF16, BASED_ERR_DTYPE, "swa_step_anydim: only bf16 is supported");
+  BASED_REQUIRE(D >= 8 && D <= kAnyMaxDim && D % 8 == 0, BASED_ERR_SHAPE,
+                "swa_step_anydim: head dim %ld unsupported (multiples of 8 up to %d)", (long)D, kAnyMaxDim);
+  BASED_REQUIRE(w_left >= 0 && w_left <= 128, BASED_ERR_SHAPE, "swa_step_anydim: left window %d unsupported (0..128)",
+                w_left);
+  BASED_REQUIRE(max_seqlen < (1ll << 31) && B * H < (1ll << 31), BASED_ERR_SHAPE, "swa_step_anydim: sizes too large");
+  if (!cache_seqlens)
+    BASED_REQUIRE(pos_host >= 0 && pos_host < max_seqlen, BASED_ERR_ARG,
+                  "swa_step_anydim: position %ld outside the cache (max_seqlen %ld)", (long)pos_host, (long)max_seqlen);
+  BASED_REQUIRE(c_sb % 8 == 0 && c_st % 8 == 0 && c_sh % 8 == 0 && q_sb % 8 == 0 && q_sh % 8 == 0, BASED_ERR_ALIGN,
+                "swa_step_anydim: cache and q strides must be multiples of 8 elements");
+  BASED_REQUIRE(aligned16(kcache) && aligned16(q), BASED_ERR_ALIGN, "swa_step_anydim: kcache and q must be 16-byte aligned");
+  if (B == 0) return BASED_OK;
+  hipLaunchKernelGGL(swa_step_anydim_kernel, dim3((unsigned)(B * H)), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     (const __bf16*)q, (const __bf16*)k_new, (const __bf16*)v_new, (__bf16*)kcache, (__bf16*)vcache,
+                     (__bf16*)o, cache_seqlens, (int)pos_host, (int)H, (int)D, (int)max_seqlen, q_sb, q_sh, kn_sb, kn_sh,
+                     vn_sb, vn_sh, o_sb, o_sh, c_sb, c_st, c_sh, w_left, scale * 1.4426950408889634f);
+  return check_launch("swa_step_anydim");
 }

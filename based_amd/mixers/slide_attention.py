@@ -5,8 +5,9 @@ constructor arguments, parameter names (Wqkv / out_proj), forward and
 allocate_inference_cache signatures and the reference's linear (B, max_seqlen, 2, H, D) KV
 cache.  `window_size=W` means query i attends keys [i - W//2, i] (flash-attn's
 `window_size=(W//2, 0)` with causal=True, slide_attention.py:332-336).
-In scope: self-attention, num_heads_kv == num_heads, head_dim 64, window_size up to 256 (128 keys
-to the left, what the released checkpoints use), no dropout / padding / varlen; other arguments
+In scope: self-attention, num_heads_kv == num_heads, head_dim 64 (MFMA kernels; other multiples
+of 8 up to 128 run a plain kernel), window_size up to 256 (128 keys to the left, what the released
+checkpoints use), no dropout / padding / varlen; other arguments
 raise NotImplementedError.  Non-half inputs are computed in bf16
 (the reference casts to bf16 for prefill, slide_attention.py:76-78).
 """
@@ -123,8 +124,8 @@ class SlidingAttention(nn.Module):
         self.num_heads_kv = num_heads
         assert self.embed_dim % num_heads == 0, "embed_dim must be divisible by num_heads"
         self.head_dim = self.embed_dim // num_heads
-        if self.head_dim != 64:
-            raise NotImplementedError("the HIP kernels are built for head_dim 64")
+        if self.head_dim % 8 != 0 or self.head_dim > 128:
+            raise NotImplementedError("the HIP kernels take head dims that are multiples of 8 up to 128 (64: MFMA path)")
         self.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(self.head_dim)
         if self.rotary_emb_dim > 0:
             self.rotary_emb = RotaryEmbedding(self.rotary_emb_dim, base=rotary_emb_base,
@@ -166,7 +167,7 @@ class SlidingAttention(nn.Module):
         # the kernels; other rotary shapes are applied here with torch ops at host-known positions.
         rope = None
         if self.rotary_emb_dim > 0:
-            if self.rotary_emb_dim == self.head_dim and not self.rotary_emb.interleaved:
+            if self.head_dim == 64 and self.rotary_emb_dim == 64 and not self.rotary_emb.interleaved:
                 n_pos = seqlen if inference_params is None else max(inference_params.max_seqlen, offset + seqlen)
                 rope = self.rotary_emb.tables(n_pos, qkv.device)
             else:

@@ -128,16 +128,20 @@ def _rope_tables(rope, device, need_rows):
 
 def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=None, kv_cache=None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Sliding-window causal attention.  q, k, v: (B, L, H, 64) bf16 (any strides with the
+    """Sliding-window causal attention.  q, k, v: (B, L, H, D) bf16 (any strides with the
     last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i], 0 <= w_left <= 128.
+    D = 64 runs the MFMA kernel; other head dims (multiples of 8 up to 128) a plain one-wavefront-per-
+    query kernel without in-kernel rotary.
     rope: None or (cos, sin) fp32 (n_pos >= L, 32) tables; q and k are then rotated in the kernel
     (non-interleaved rotary over the whole head, positions 0..L-1).
     kv_cache: None or a (B, max_seqlen >= L, 2, H, 64) bf16 cache whose rows 0..L-1 receive the
     (rotated) k and v.  out: None or a (B, L, H, 64) tensor (last dim contiguous) to write into."""
     _require_cuda(q, k, v)
     B, L, H, D = q.shape
-    if D != 64 or k.shape != q.shape or v.shape != q.shape:
-        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)} (head dim 64)")
+    if k.shape != q.shape or v.shape != q.shape:
+        raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+    if D != 64 and rope is not None:
+        raise ValueError("in-kernel rotary needs head dim 64")
     for t in (q, k, v):
         if t.stride(-1) != 1:
             raise ValueError("innermost dimension must be contiguous")
@@ -160,19 +164,27 @@ def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=N
         if tuple(o.shape) != (B, L, H, D) or o.dtype != q.dtype or o.device != q.device or o.stride(-1) != 1:
             raise ValueError(f"out must be a ({B}, {L}, {H}, {D}) {q.dtype} tensor on {q.device}")
     with _on_device(q.device):
-        _lib.check(_lib.lib().based_swa_prefill(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L,
-            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-            v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
-            int(w_left), scale, cos_ptr, sin_ptr, n_pos, kc_ptr, vc_ptr, *c_strides, max_seqlen,
-            _dtype_code(q), _stream_ptr(q)))
+        if D == 64:
+            _lib.check(_lib.lib().based_swa_prefill(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L,
+                q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+                int(w_left), scale, cos_ptr, sin_ptr, n_pos, kc_ptr, vc_ptr, *c_strides, max_seqlen,
+                _dtype_code(q), _stream_ptr(q)))
+        else:
+            _lib.check(_lib.lib().based_swa_prefill_anydim(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L, D,
+                q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+                int(w_left), scale, kc_ptr, vc_ptr, *c_strides, max_seqlen, _dtype_code(q), _stream_ptr(q)))
     return o
 
 
 def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None, rope=None,
              out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Decode step.  q, k_new, v_new: (B, 1, H, 64) bf16; kv_cache (B, max_seqlen, 2, H, 64)
-    bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.
+    """Decode step.  q, k_new, v_new: (B, 1, H, D) bf16; kv_cache (B, max_seqlen, 2, H, D)
+    bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.  D = 64, or
+    another multiple of 8 up to 128 (plain kernel, no in-kernel rotary).
     pos: int (same for the whole batch) or an int32 device tensor of B positions.
     rope: None or (cos, sin) tables as for swa_prefill: q and k_new are rotated at `pos` first.
     out: None or a (B, 1, H, 64) tensor (last dim contiguous) to write into."""
@@ -182,7 +194,7 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
     if key not in _CHECKED:
         _require_cuda(q, k_new, v_new, kv_cache)
         B, one, H, D = q.shape
-        if one != 1 or D != 64 or k_new.shape != q.shape or v_new.shape != q.shape:
+        if one != 1 or k_new.shape != q.shape or v_new.shape != q.shape:
             raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k_new.shape)} v{tuple(v_new.shape)}")
         if kv_cache.dim() != 5 or kv_cache.shape[0] < B or kv_cache.shape[2] != 2 or tuple(kv_cache.shape[3:]) != (H, D):
             raise ValueError(f"bad cache shape {tuple(kv_cache.shape)}")
@@ -194,7 +206,9 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
         _dtype_code(q)
         _CHECKED[key] = True
     B, _, H, D = q.shape
-    scale = 0.125 if scale is None else float(scale)  # 1 / sqrt(64)
+    scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
+    if D != 64 and rope is not None:
+        raise ValueError("in-kernel rotary needs head dim 64")
     if isinstance(pos, torch.Tensor):
         if pos.dtype != torch.int32 or not pos.is_cuda or pos.numel() < B or not pos.is_contiguous():
             raise ValueError("cache_seqlens must be a contiguous int32 device tensor with B entries")
@@ -213,13 +227,21 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
     kc_ptr = kv_cache.data_ptr()
     vc_ptr = kc_ptr + kv_cache.stride(2) * kv_cache.element_size()
     with _on_device(q.device):
-        _lib.check(_lib.lib().based_swa_step(
-            q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
-            seq_ptr, pos_host, B, H, kv_cache.shape[1],
-            q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
-            v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
-            c_sb, c_st, c_sh,
-            int(w_left), scale, cos_ptr, sin_ptr, n_pos, _dtype_code(q), _stream_ptr(q)))
+        if D == 64:
+            _lib.check(_lib.lib().based_swa_step(
+                q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
+                seq_ptr, pos_host, B, H, kv_cache.shape[1],
+                q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
+                v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
+                c_sb, c_st, c_sh,
+                int(w_left), scale, cos_ptr, sin_ptr, n_pos, _dtype_code(q), _stream_ptr(q)))
+        else:
+            _lib.check(_lib.lib().based_swa_step_anydim(
+                q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
+                seq_ptr, pos_host, B, H, D, kv_cache.shape[1],
+                q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
+                v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
+                c_sb, c_st, c_sh, int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
     return o
 
 

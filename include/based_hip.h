@@ -277,6 +277,33 @@ BASED_API int based_swiglu(const void* u, void* out, int64_t rows, int64_t F, in
                  int io_dtype, void* stream);
 
 /*
+ * The same sliding-window attention for head dimensions other than 64 (any multiple of 8 up to
+ * 128), bf16, fp32 arithmetic, one wavefront per query: not a performance path, it exists so
+ * that models with other head sizes (the reference's own test models have 16-dim heads,
+ * based/tests/test_generation.py:7-34,69-80) run through the same module.  Same reference lines
+ * and argument meaning as based_swa_prefill / based_swa_step, plus the head dimension D; no
+ * in-kernel rotary (the caller rotates q and k first).
+ */
+BASED_API int based_swa_prefill_anydim(const void* q, const void* k, const void* v, void* o,
+                             int64_t B, int64_t H, int64_t L, int64_t D,
+                             int64_t q_sb, int64_t q_sl, int64_t q_sh,
+                             int64_t k_sb, int64_t k_sl, int64_t k_sh,
+                             int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                             int64_t o_sb, int64_t o_sl, int64_t o_sh,
+                             int w_left, float scale,
+                             void* kcache_out, void* vcache_out,
+                             int64_t c_sb, int64_t c_st, int64_t c_sh, int64_t max_seqlen,
+                             int io_dtype, void* stream);
+BASED_API int based_swa_step_anydim(const void* q, const void* k_new, const void* v_new,
+                          void* kcache, void* vcache, void* o,
+                          const int32_t* cache_seqlens, int64_t pos_host,
+                          int64_t B, int64_t H, int64_t D, int64_t max_seqlen,
+                          int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
+                          int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
+                          int64_t c_sb, int64_t c_st, int64_t c_sh,
+                          int w_left, float scale, int io_dtype, void* stream);
+
+/*
  * Measurement probes.  No counterpart in the reference: they are streaming kernels with the
  * memory access patterns of the kernels above and no arithmetic, so that a benchmark can report,
  * next to the published HBM bandwidth, what this machine delivers for that pattern.

@@ -47,8 +47,9 @@ def test_sliding_attention_parameters_and_cache():
     assert SlidingAttention(embed_dim=1024, num_heads=16, window_size=256).window == (128, 0)   # the released configs
     with pytest.raises(NotImplementedError):
         SlidingAttention(embed_dim=1024, num_heads=16, window_size=258)
+    assert SlidingAttention(embed_dim=256, num_heads=16).head_dim == 16      # the reference's test models: plain kernel
     with pytest.raises(NotImplementedError):
-        SlidingAttention(embed_dim=512, num_heads=16)
+        SlidingAttention(embed_dim=192, num_heads=16)                         # head dim 12
 
 
 def test_cpu_tensors_fail_loudly():

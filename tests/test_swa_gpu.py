@@ -101,9 +101,12 @@ def test_decode_matches_prefill_oracle(dev, P, T, w):
 def test_rejects(dev):
     from based_amd import ops
 
+    x = torch.zeros(1, 4, 2, 12, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.swa_prefill(x, x, x)  # head dim 12 (not a multiple of 8)
     x = torch.zeros(1, 4, 2, 32, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
-        ops.swa_prefill(x, x, x)  # head dim 32
+        ops.swa_prefill(x, x, x, rope=_rope_tables(4, dev))  # in-kernel rotary is for head dim 64
     y = torch.zeros(1, 4, 2, 64, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         ops.swa_prefill(y, y, y, w_left=129)
@@ -177,3 +180,66 @@ def test_decode_with_rotary_matches_parallel(dev, P, T, w):
         assert rel_l2(o.float(), ref[:, t:t + 1].float()) < TOL
     assert rel_l2(cache[:, :, 0].float(), k_r.float()) < 3e-3
     assert torch.equal(cache[:, :, 1].cpu(), qkv[:, :, 2])
+
+
+def _qkv_d(B, L, H, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(B, L, 3, H, D, generator=g).bfloat16()
+
+
+@pytest.mark.parametrize("B,L,H,D,w", [(2, 200, 3, 16, 64), (1, 300, 2, 32, 128), (1, 70, 2, 128, 17), (1, 1, 1, 8, 64),
+                                       (2, 130, 4, 16, 0), (1, 257, 2, 96, 100)])
+def test_other_head_dims_prefill_and_cache(dev, B, L, H, D, w):
+    """Head dims other than 64 (the reference's test models have 16): the plain kernel against the oracle,
+    with and without the cache output."""
+    from based_amd import ops
+
+    print(f"swa any-dim prefill case B={B} L={L} H={H} D={D} w={w}", flush=True)
+    qkv = _qkv_d(B, L, H, D, seed=23)
+    ref = O.sliding_window_attn(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    cache = torch.full((B, L + 3, 2, H, D), 3.0, dtype=torch.bfloat16, device=dev)
+    out = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, kv_cache=cache)
+    assert out.shape == (B, L, H, D) and rel_l2(out.float(), ref.float()) < 5e-3
+    assert torch.equal(cache[:, :L].cpu(), qkv[:, :, 1:]) and bool((cache[:, L:] == 3.0).all())
+    assert torch.equal(out, ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w))
+
+
+@pytest.mark.parametrize("D,P,T,w", [(16, 0, 70, 64), (16, 100, 40, 128), (32, 60, 10, 65), (128, 10, 6, 7)])
+def test_other_head_dims_decode(dev, D, P, T, w):
+    from based_amd import ops
+
+    B, H = 2, 3
+    L = P + T
+    qkv = _qkv_d(B, L, H, D, seed=29)
+    ref = O.sliding_window_attn(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    cache = torch.zeros(B, L + 2, 2, H, D, dtype=torch.bfloat16, device=dev)
+    if P > 0:
+        ops.swa_prefill(qd[:, :P, 0], qd[:, :P, 1], qd[:, :P, 2], w_left=w, kv_cache=cache)
+    for t in range(P, L):
+        print(f"swa any-dim step case D={D} P={P} w={w} pos={t}", flush=True)
+        p = t if t % 2 == 0 else torch.full((B,), t, dtype=torch.int32, device=dev)
+        o = ops.swa_step(qd[:, t:t + 1, 0], qd[:, t:t + 1, 1], qd[:, t:t + 1, 2], cache, p, w_left=w)
+        assert rel_l2(o.float(), ref[:, t:t + 1].float()) < 5e-3
+    assert torch.equal(cache[:, :L].cpu(), qkv[:, :, 1:])
+    bad = ops.swa_step(qd[:, :1, 0], qd[:, :1, 1], qd[:, :1, 2], cache, torch.full((B,), L + 2, dtype=torch.int32, device=dev), w_left=w)
+    assert bool(torch.isnan(bad.float()).all())        # device-side position outside the cache
+
+
+def test_plain_kernel_agrees_with_mfma_kernel_at_head_dim_64(dev):
+    """The plain kernels are a second statement of the attention: at head dim 64 they can be called
+    through the C ABI next to the MFMA kernels."""
+    from based_amd import _lib, ops
+
+    B, L, H, w = 2, 333, 4, 128
+    qkv = _qkv(B, L, H, seed=31).to(dev)
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    fast = ops.swa_prefill(q, k, v, w_left=w)
+    slow = torch.empty_like(fast)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(_lib.lib().based_swa_prefill_anydim(
+        q.data_ptr(), k.data_ptr(), v.data_ptr(), slow.data_ptr(), B, H, L, 64, q.stride(0), q.stride(1), q.stride(2),
+        k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2), slow.stride(0), slow.stride(1),
+        slow.stride(2), w, 0.125, None, None, 0, 0, 0, 0, _lib.BASED_BF16, stream))
+    assert rel_l2(fast.float(), slow.float()) < 4e-3
