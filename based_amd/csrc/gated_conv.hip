@@ -3,6 +3,9 @@
 // with u = [u1 | u2] the (B, L, 2D) output of the block's input projection
 // (based/models/mixers/convolution.py:195-210: depthwise causal Conv1d, SiLU, gate), plus the
 // single-token form on a rolling (B, D, K) state (convolution.py:88-109).
+// `gated` = 0 gives the convolution on its own, y = conv(u) (+ bias), u of width D: the
+// ShortConvolution module used as a mixer by itself (convolution.py:47-87, the path without the
+// fused CUDA kernel, which applies no activation).
 //
 // Prefill: a thread owns 16 bytes of channels (8 bf16 / 4 fp32) and walks kTokens consecutive
 // tokens with the last K-1 inputs kept in registers, so every u element is read once (plus a
@@ -43,7 +46,7 @@ __device__ __forceinline__ void store_dyn(void* p, long i, int dtype, float x) {
 template <typename T, int K>
 __global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
     const T* __restrict__ u, const T* __restrict__ weight, const T* __restrict__ bias, T* __restrict__ y,
-    void* __restrict__ state, int L, int D, long u_sb, long u_sl, long y_sb, long y_sl, int state_dtype) {
+    void* __restrict__ state, int L, int D, long u_sb, long u_sl, long y_sb, long y_sl, int state_dtype, int gated) {
   constexpr int N = Vec16<T>::kN;
   typedef typename Vec16<T>::type vec_t;
   const int c0 = (blockIdx.x * 256 + threadIdx.x) * N;  // first channel of this thread
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
       x2[i] = vec_t{};
       if (t0 + i < ntok) {
         x1[i] = *reinterpret_cast<const vec_t*>(u1 + (long)(l0 + t0 + i) * u_sl);
-        x2[i] = *reinterpret_cast<const vec_t*>(u2 + (long)(l0 + t0 + i) * u_sl);
+        if (gated) x2[i] = *reinterpret_cast<const vec_t*>(u2 + (long)(l0 + t0 + i) * u_sl);
       }
     }
 #pragma unroll
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
           float acc = bs[c];
 #pragma unroll
           for (int j = 0; j < K; ++j) acc = __builtin_fmaf(w[c][j], win[j][c], acc);
-          out[c] = from_f32<T>(silu(acc) * to_f32(x2[i][c]));
+          out[c] = from_f32<T>(gated ? silu(acc) * to_f32(x2[i][c]) : acc);
 #pragma unroll
           for (int j = 0; j < K - 1; ++j) win[j][c] = win[j + 1][c];
         }
@@ -153,16 +156,16 @@ template <typename E, int COUNT> __device__ __forceinline__ void store_run(void*
 template <typename T, typename TS, int K>
 __global__ __launch_bounds__(256) void gated_conv_step_kernel(
     const T* __restrict__ u, TS* __restrict__ state, const T* __restrict__ weight, const T* __restrict__ bias,
-    T* __restrict__ y, int B, int D, long u_sb, long y_sb) {
+    T* __restrict__ y, int B, int D, long u_sb, long y_sb, int gated) {
   constexpr int N = 8;
   const long item = (long)blockIdx.x * 256 + threadIdx.x;
   const int per_row = D / N;
   if (item >= (long)B * per_row) return;
   const int b = (int)(item / per_row);
   const int c0 = (int)(item % per_row) * N;
-  float x1[N], x2[N], st[N * K], w[N * K], bs[N], out[N];
+  float x1[N], x2[N] = {}, st[N * K], w[N * K], bs[N], out[N];
   load_run<T, N>(u + b * u_sb, c0, x1);
-  load_run<T, N>(u + b * u_sb, D + c0, x2);
+  if (gated) load_run<T, N>(u + b * u_sb, D + c0, x2);
   load_run<TS, N * K>(state, ((long)b * D + c0) * K, st);
   load_run<T, N * K>(weight, (long)c0 * K, w);
 #pragma unroll
@@ -176,7 +179,7 @@ __global__ __launch_bounds__(256) void gated_conv_step_kernel(
     float acc = bs[c];
 #pragma unroll
     for (int j = 0; j < K; ++j) acc = __builtin_fmaf(w[c * K + j], st[c * K + j], acc);
-    out[c] = silu(acc) * x2[c];
+    out[c] = gated ? silu(acc) * x2[c] : acc;
   }
   store_run<TS, N * K>(state, ((long)b * D + c0) * K, st);
   store_run<T, N>(y + b * y_sb, c0, out);
@@ -210,14 +213,14 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 template <typename T>
 int launch_gated_conv_prefill(const void* u, const void* weight, const void* bias, void* y, void* state,
                               int64_t B, int64_t L, int64_t D, int K, int64_t u_sb, int64_t u_sl,
-                              int64_t y_sb, int64_t y_sl, int state_dtype, hipStream_t stream) {
+                              int64_t y_sb, int64_t y_sl, int state_dtype, int gated, hipStream_t stream) {
   constexpr int N = Vec16<T>::kN;
   dim3 grid((unsigned)((D / N + 255) / 256), (unsigned)((L + kConvTokens - 1) / kConvTokens), (unsigned)B), block(256);
 #define BASED_CONV_CASE(KK)                                                                               \
   case KK:                                                                                                \
     hipLaunchKernelGGL((gated_conv_prefill_kernel<T, KK>), grid, block, 0, stream, (const T*)u,            \
                        (const T*)weight, (const T*)bias, (T*)y, state, (int)L, (int)D, u_sb, u_sl, y_sb,   \
-                       y_sl, state_dtype);                                                                \
+                       y_sl, state_dtype, gated);                                                         \
     break;
   switch (K) {
     BASED_CONV_CASE(2)
@@ -230,13 +233,13 @@ int launch_gated_conv_prefill(const void* u, const void* weight, const void* bia
 
 template <typename T, typename TS>
 int launch_gated_conv_step(const void* u, void* state, const void* weight, const void* bias, void* y,
-                           int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb, hipStream_t stream) {
+                           int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb, int gated, hipStream_t stream) {
   const int64_t items = B * (D / 8);
   dim3 grid((unsigned)((items + 255) / 256)), block(256);
 #define BASED_CONV_CASE(KK)                                                                              \
   case KK:                                                                                               \
     hipLaunchKernelGGL((gated_conv_step_kernel<T, TS, KK>), grid, block, 0, stream, (const T*)u, (TS*)state, \
-                       (const T*)weight, (const T*)bias, (T*)y, (int)B, (int)D, u_sb, y_sb);              \
+                       (const T*)weight, (const T*)bias, (T*)y, (int)B, (int)D, u_sb, y_sb, gated);       \
     break;
   switch (K) {
     BASED_CONV_CASE(2)
@@ -249,52 +252,83 @@ int launch_gated_conv_step(const void* u, void* state, const void* weight, const
 
 }  // namespace based
 
+namespace based {
+static int conv_prefill_impl(const char* who, int gated, const void* u, const void* weight, const void* bias, void* y,
+                             void* state, int64_t B, int64_t L, int64_t D, int K, int64_t u_sb, int64_t u_sl,
+                             int64_t y_sb, int64_t y_sl, int io_dtype, int state_dtype, void* stream) {
+  BASED_REQUIRE(u && weight && y, BASED_ERR_ARG, "%s: null pointer argument", who);
+  BASED_REQUIRE(B >= 0 && L >= 0 && D > 0, BASED_ERR_ARG, "%s: bad sizes", who);
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "%s: bad io dtype", who);
+  BASED_REQUIRE(state == nullptr || state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE,
+                "%s: bad state dtype", who);
+  BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "%s: kernel size %d unsupported (2..4)", who, K);
+  const int n = io_dtype == BASED_BF16 ? 8 : 4;
+  BASED_REQUIRE(D % n == 0, BASED_ERR_SHAPE, "%s: channel count must be a multiple of %d", who, n);
+  BASED_REQUIRE(u_sb % n == 0 && u_sl % n == 0 && y_sb % n == 0 && y_sl % n == 0, BASED_ERR_ALIGN,
+                "%s: strides must be multiples of %d elements", who, n);
+  BASED_REQUIRE(aligned16(u) && aligned16(y), BASED_ERR_ALIGN, "%s: tensors must be 16-byte aligned", who);
+  BASED_REQUIRE(B < 65536 && (L + kConvTokens - 1) / kConvTokens < 65536, BASED_ERR_SHAPE,
+                "%s: grid too large", who);
+  if (B == 0 || L == 0) return BASED_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return io_dtype == BASED_BF16
+             ? launch_gated_conv_prefill<__bf16>(u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl, state_dtype, gated, s)
+             : launch_gated_conv_prefill<float>(u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl, state_dtype, gated, s);
+}
+}  // namespace based
+
+namespace based {
+static int conv_step_impl(const char* who, int gated, const void* u, void* state, const void* weight, const void* bias,
+                          void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb, int io_dtype,
+                          int state_dtype, void* stream) {
+  BASED_REQUIRE(u && state && weight && y, BASED_ERR_ARG, "%s: null pointer argument", who);
+  BASED_REQUIRE(B >= 0 && D > 0, BASED_ERR_ARG, "%s: bad sizes", who);
+  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "%s: bad io dtype", who);
+  BASED_REQUIRE(state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE, "%s: bad state dtype", who);
+  BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "%s: kernel size %d unsupported (2..4)", who, K);
+  BASED_REQUIRE(D % 8 == 0, BASED_ERR_SHAPE, "%s: channel count must be a multiple of 8", who);
+  BASED_REQUIRE(u_sb % 8 == 0 && y_sb % 8 == 0, BASED_ERR_ALIGN, "%s: strides must be multiples of 8 elements", who);
+  BASED_REQUIRE(aligned16(u) && aligned16(y) && aligned16(state) && aligned16(weight) && aligned16(bias),
+                BASED_ERR_ALIGN, "%s: tensors must be 16-byte aligned", who);
+  BASED_REQUIRE(B * (D / 8) < (1ll << 39), BASED_ERR_SHAPE, "%s: grid too large", who);
+  if (B == 0) return BASED_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (io_dtype == BASED_BF16)
+    return state_dtype == BASED_BF16 ? launch_gated_conv_step<__bf16, __bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, gated, s)
+                                     : launch_gated_conv_step<__bf16, float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, gated, s);
+  return state_dtype == BASED_BF16 ? launch_gated_conv_step<float, __bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, gated, s)
+                                   : launch_gated_conv_step<float, float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, gated, s);
+}
+}  // namespace based
+
 extern "C" BASED_API int based_gated_conv_prefill(const void* u, const void* weight, const void* bias, void* y,
                                                   void* state, int64_t B, int64_t L, int64_t D, int K,
                                                   int64_t u_sb, int64_t u_sl, int64_t y_sb, int64_t y_sl,
                                                   int io_dtype, int state_dtype, void* stream) {
-  using namespace based;
-  BASED_REQUIRE(u && weight && y, BASED_ERR_ARG, "gated_conv_prefill: null pointer argument");
-  BASED_REQUIRE(B >= 0 && L >= 0 && D > 0, BASED_ERR_ARG, "gated_conv_prefill: bad sizes");
-  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_prefill: bad io dtype");
-  BASED_REQUIRE(state == nullptr || state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE,
-                "gated_conv_prefill: bad state dtype");
-  BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "gated_conv_prefill: kernel size %d unsupported (2..4)", K);
-  const int n = io_dtype == BASED_BF16 ? 8 : 4;
-  BASED_REQUIRE(D % n == 0, BASED_ERR_SHAPE, "gated_conv_prefill: channel count must be a multiple of %d", n);
-  BASED_REQUIRE(u_sb % n == 0 && u_sl % n == 0 && y_sb % n == 0 && y_sl % n == 0, BASED_ERR_ALIGN,
-                "gated_conv_prefill: strides must be multiples of %d elements", n);
-  BASED_REQUIRE(aligned16(u) && aligned16(y), BASED_ERR_ALIGN, "gated_conv_prefill: tensors must be 16-byte aligned");
-  BASED_REQUIRE(B < 65536 && (L + kConvTokens - 1) / kConvTokens < 65536, BASED_ERR_SHAPE,
-                "gated_conv_prefill: grid too large");
-  if (B == 0 || L == 0) return BASED_OK;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  return io_dtype == BASED_BF16
-             ? launch_gated_conv_prefill<__bf16>(u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl, state_dtype, s)
-             : launch_gated_conv_prefill<float>(u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl, state_dtype, s);
+  return based::conv_prefill_impl("gated_conv_prefill", 1, u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl,
+                                  io_dtype, state_dtype, stream);
 }
 
 extern "C" BASED_API int based_gated_conv_step(const void* u, void* state, const void* weight, const void* bias,
                                                void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
                                                int io_dtype, int state_dtype, void* stream) {
-  using namespace based;
-  BASED_REQUIRE(u && state && weight && y, BASED_ERR_ARG, "gated_conv_step: null pointer argument");
-  BASED_REQUIRE(B >= 0 && D > 0, BASED_ERR_ARG, "gated_conv_step: bad sizes");
-  BASED_REQUIRE(io_dtype == BASED_BF16 || io_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_step: bad io dtype");
-  BASED_REQUIRE(state_dtype == BASED_BF16 || state_dtype == BASED_F32, BASED_ERR_DTYPE, "gated_conv_step: bad state dtype");
-  BASED_REQUIRE(K >= 2 && K <= kConvMaxK, BASED_ERR_SHAPE, "gated_conv_step: kernel size %d unsupported (2..4)", K);
-  BASED_REQUIRE(D % 8 == 0, BASED_ERR_SHAPE, "gated_conv_step: channel count must be a multiple of 8");
-  BASED_REQUIRE(u_sb % 8 == 0 && y_sb % 8 == 0, BASED_ERR_ALIGN, "gated_conv_step: strides must be multiples of 8 elements");
-  BASED_REQUIRE(aligned16(u) && aligned16(y) && aligned16(state) && aligned16(weight) && aligned16(bias),
-                BASED_ERR_ALIGN, "gated_conv_step: tensors must be 16-byte aligned");
-  BASED_REQUIRE(B * (D / 8) < (1ll << 39), BASED_ERR_SHAPE, "gated_conv_step: grid too large");
-  if (B == 0) return BASED_OK;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (io_dtype == BASED_BF16)
-    return state_dtype == BASED_BF16 ? launch_gated_conv_step<__bf16, __bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s)
-                                     : launch_gated_conv_step<__bf16, float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s);
-  return state_dtype == BASED_BF16 ? launch_gated_conv_step<float, __bf16>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s)
-                                   : launch_gated_conv_step<float, float>(u, state, weight, bias, y, B, D, K, u_sb, y_sb, s);
+  return based::conv_step_impl("gated_conv_step", 1, u, state, weight, bias, y, B, D, K, u_sb, y_sb, io_dtype,
+                               state_dtype, stream);
+}
+
+extern "C" BASED_API int based_short_conv_prefill(const void* u, const void* weight, const void* bias, void* y,
+                                                  void* state, int64_t B, int64_t L, int64_t D, int K,
+                                                  int64_t u_sb, int64_t u_sl, int64_t y_sb, int64_t y_sl,
+                                                  int io_dtype, int state_dtype, void* stream) {
+  return based::conv_prefill_impl("short_conv_prefill", 0, u, weight, bias, y, state, B, L, D, K, u_sb, u_sl, y_sb, y_sl,
+                                  io_dtype, state_dtype, stream);
+}
+
+extern "C" BASED_API int based_short_conv_step(const void* u, void* state, const void* weight, const void* bias,
+                                               void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
+                                               int io_dtype, int state_dtype, void* stream) {
+  return based::conv_step_impl("short_conv_step", 0, u, state, weight, bias, y, B, D, K, u_sb, y_sb, io_dtype,
+                               state_dtype, stream);
 }
 
 extern "C" BASED_API int based_swiglu(const void* u, void* out, int64_t rows, int64_t F, int64_t u_sr, int64_t o_sr,

@@ -1,7 +1,8 @@
-"""Gated short convolution mixer; mirrors the interface of based/models/mixers/convolution.py:16-218:
-depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a rolling (B, D, K) state for
-decoding.  Everything between the two projections is one kernel (`ops.gated_conv_prefill` /
-`ops.gated_conv_step`); there is no host-tensor path."""
+"""Short convolution mixers; mirror the interface of based/models/mixers/convolution.py:16-218:
+BaseConv = in_proj -> depthwise causal conv (kernel 3) -> SiLU -> gate -> out_proj, with a rolling
+(B, D, K) state for decoding; everything between the two projections is one kernel
+(`ops.gated_conv_prefill` / `ops.gated_conv_step`).  ShortConvolution on its own is the same
+kernel without activation and gate.  There is no host-tensor path."""
 from __future__ import annotations
 
 import torch
@@ -19,10 +20,20 @@ class ShortConvolution(nn.Module):
                               padding=kernel_size - 1, bias=conv_bias, device=device, dtype=dtype)
 
     def forward(self, x: torch.Tensor, inference_params=None, **kwargs):
-        # Holds the nn.Conv1d parameters (state-dict names) and the rolling state of BaseConv, which
-        # runs conv + SiLU + gate as one kernel; the un-gated convolution as a mixer of its own is
-        # not part of the released Based stacks and has no kernel here.
-        raise NotImplementedError("ShortConvolution on its own is outside this build; use BaseConv")
+        """x (b, l, d) -> (b, l, d): the depthwise causal convolution alone (no activation), with the
+        rolling state of ShortConvolution.forward / step (convolution.py:47-109).  Inside BaseConv
+        this method is not used: conv, SiLU and gate are one kernel there."""
+        from .. import ops
+
+        weight, bias = self.conv.weight, self.conv.bias
+        if inference_params is None:
+            return ops.gated_conv_prefill(x, weight, bias, gated=False)
+        if inference_params.seqlen_offset > 0:
+            state = self._get_state(inference_params)
+            return ops.gated_conv_step(x, state[: x.shape[0]], weight, bias, gated=False)
+        self._init_state(inference_params)
+        state = self._get_state(inference_params)
+        return ops.gated_conv_prefill(x, weight, bias, state=state[: x.shape[0]], gated=False)
 
     def allocate_inference_cache(self, batch_size: int, max_seqlen: int, dtype=None, **kwargs):
         return torch.zeros(batch_size, self.d_model, self.kernel_size, device=self.conv.weight.device,

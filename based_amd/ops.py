@@ -296,15 +296,16 @@ def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False,
     return y, kv_state, k_state
 
 
-def gated_conv_prefill(u, weight, bias=None, state=None) -> torch.Tensor:
+def gated_conv_prefill(u, weight, bias=None, state=None, gated: bool = True) -> torch.Tensor:
     """y = silu(causal depthwise conv(u[..., :D]) + bias) * u[..., D:].  u: (B, L, 2D) with a
     contiguous last dimension; weight: the (D, 1, K) nn.Conv1d weight; bias (D) or None; state
-    None or (B, D, K) contiguous, overwritten with the last K inputs.  Returns y (B, L, D)."""
+    None or (B, D, K) contiguous, overwritten with the last K inputs.  Returns y (B, L, D).
+    gated=False: the convolution alone, y = conv(u) + bias with u (B, L, D)."""
     _require_cuda(u, weight)
-    if u.dim() != 3 or u.shape[-1] % 2 != 0:
+    if u.dim() != 3 or (gated and u.shape[-1] % 2 != 0):
         raise ValueError(f"u must be (B, L, 2D), got {tuple(u.shape)}")
     B, L, D2 = u.shape
-    D = D2 // 2
+    D = D2 // 2 if gated else D2
     if weight.dim() != 3 or weight.shape[0] != D or weight.shape[1] != 1:
         raise ValueError(f"weight must be ({D}, 1, K), got {tuple(weight.shape)}")
     K = weight.shape[2]
@@ -325,17 +326,19 @@ def gated_conv_prefill(u, weight, bias=None, state=None) -> torch.Tensor:
             raise ValueError(f"state must be a contiguous ({B}, {D}, {K}) tensor, got {tuple(state.shape)}")
         state_code = _dtype_code(state)
     y = torch.empty(B, L, D, dtype=u.dtype, device=u.device)
+    fn = _lib.lib().based_gated_conv_prefill if gated else _lib.lib().based_short_conv_prefill
     with _on_device(u.device):
-        _lib.check(_lib.lib().based_gated_conv_prefill(
+        _lib.check(fn(
             u.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None, y.data_ptr(),
             state.data_ptr() if state is not None else None, B, L, D, K,
             u.stride(0), u.stride(1), y.stride(0), y.stride(1), _dtype_code(u), state_code, _stream_ptr(u)))
     return y
 
 
-def gated_conv_step(u, state, weight, bias=None) -> torch.Tensor:
+def gated_conv_step(u, state, weight, bias=None, gated: bool = True) -> torch.Tensor:
     """Single-token gated short convolution.  u: (B, 1, 2D) or (B, 2D); state (B, D, K)
-    contiguous, rolled and updated in place.  Returns y with u's leading shape and D channels."""
+    contiguous, rolled and updated in place.  Returns y with u's leading shape and D channels.
+    gated=False: the convolution alone on u (B, 1, D) or (B, D)."""
     _require_cuda(u, state, weight)
     squeeze = u.dim() == 3
     if squeeze:
@@ -345,7 +348,7 @@ def gated_conv_step(u, state, weight, bias=None) -> torch.Tensor:
     else:
         u2d = u
     B, D2 = u2d.shape
-    D = D2 // 2
+    D = D2 // 2 if gated else D2
     K = weight.shape[-1]
     if tuple(weight.shape) != (D, 1, K) or tuple(state.shape) != (B, D, K) or not state.is_contiguous():
         raise ValueError(f"bad shapes u{tuple(u.shape)} weight{tuple(weight.shape)} state{tuple(state.shape)}")
@@ -358,8 +361,9 @@ def gated_conv_step(u, state, weight, bias=None) -> torch.Tensor:
         _require_cuda(u, bias)
         bias = bias.contiguous()
     y = torch.empty(B, D, dtype=u.dtype, device=u.device)
+    fn = _lib.lib().based_gated_conv_step if gated else _lib.lib().based_short_conv_step
     with _on_device(u.device):
-        _lib.check(_lib.lib().based_gated_conv_step(
+        _lib.check(fn(
             u2d.data_ptr(), state.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
             y.data_ptr(), B, D, K, u2d.stride(0), y.stride(0), _dtype_code(u), _dtype_code(state), _stream_ptr(u)))
     return y.unsqueeze(1) if squeeze else y

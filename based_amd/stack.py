@@ -23,7 +23,7 @@ import torch.nn.functional as F
 from . import ops
 
 from .generation import GenerationMixin
-from .mixers.convolution import BaseConv
+from .mixers.convolution import BaseConv, ShortConvolution
 from .mixers.linear_attention import LinearAttention, TaylorExp
 from .mixers.slide_attention import SlidingAttention
 
@@ -33,10 +33,12 @@ _TARGETS = {
     "based.models.mixers.linear_attention.TaylorExp": TaylorExp,
     "based.models.mixers.slide_attention.SlidingAttention": SlidingAttention,
     "based.models.mixers.convolution.BaseConv": BaseConv,
+    "based.models.mixers.convolution.ShortConvolution": ShortConvolution,
     "based_amd.mixers.linear_attention.LinearAttention": LinearAttention,
     "based_amd.mixers.linear_attention.TaylorExp": TaylorExp,
     "based_amd.mixers.slide_attention.SlidingAttention": SlidingAttention,
     "based_amd.mixers.convolution.BaseConv": BaseConv,
+    "based_amd.mixers.convolution.ShortConvolution": ShortConvolution,
 }
 
 

@@ -249,6 +249,21 @@ BASED_API int based_gated_conv_step(const void* u, void* state, const void* weig
                           int io_dtype, int state_dtype, void* stream);
 
 /*
+ * The short convolution on its own, y = conv(u) (+ bias), no activation, no gate: the
+ * ShortConvolution module used as a mixer by itself (based/models/mixers/convolution.py:47-109,
+ * the path without the fused CUDA kernel; the reference's "conv" test model,
+ * based/tests/test_generation.py:37-45).  Arguments as based_gated_conv_prefill / _step, except
+ * that u has D channels (rows u[b*u_sb + l*u_sl + c], c < D).
+ */
+BASED_API int based_short_conv_prefill(const void* u, const void* weight, const void* bias, void* y,
+                             void* state, int64_t B, int64_t L, int64_t D, int K,
+                             int64_t u_sb, int64_t u_sl, int64_t y_sb, int64_t y_sl,
+                             int io_dtype, int state_dtype, void* stream);
+BASED_API int based_short_conv_step(const void* u, void* state, const void* weight, const void* bias,
+                          void* y, int64_t B, int64_t D, int K, int64_t u_sb, int64_t y_sb,
+                          int io_dtype, int state_dtype, void* stream);
+
+/*
  * Residual add + RMSNorm of the prenorm block, one pass.  Replaces, in based/models/block.py,
  * `residual = dropped + residual; hidden = norm(residual.to(dtype=norm.weight.dtype));
  * residual = residual.to(torch.float32)` (:134-139 and :151-155, dropout-free) with the RMSNorm

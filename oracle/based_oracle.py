@@ -294,7 +294,8 @@ def mixer_kind(config, layer_idx: int) -> tuple:
     elif config.get("alt_mixer_layers") is not None and layer_idx in config["alt_mixer_layers"]:
         spec = config["alt_mixer"]
     target = spec["_target_"]
-    kind = "linear" if "linear_attention" in target else "slide" if "slide" in target else "conv"
+    kind = ("linear" if "linear_attention" in target else "slide" if "slide" in target
+            else "short_conv" if target.endswith("ShortConvolution") else "conv")
     return kind, spec
 
 
@@ -325,6 +326,10 @@ def stack_forward(input_ids, sd: dict, config: dict, dtype=torch.float32):
             u = F.linear(hidden, g(m + "in_proj.weight"), g(m + "in_proj.bias"))
             y = gated_short_conv(u, g(m + "conv.conv.weight")[:, 0], g(m + "conv.conv.bias"))
             hidden = F.linear(y, g(m + "out_proj.weight"), g(m + "out_proj.bias"))
+        elif kind == "short_conv":   # the convolution alone as the mixer (convolution.py:47-87)
+            hidden = short_conv(hidden.float(), g(m + "conv.weight")[:, 0].float()).to(dtype)
+            if g(m + "conv.bias") is not None:
+                hidden = (hidden.float() + g(m + "conv.bias").float()).to(dtype)
         elif kind == "linear":
             H = spec.get("num_heads", 16)
             fd = spec.get("feature_dim", 16)

@@ -102,3 +102,24 @@ def test_swiglu_matches_torch_statement(dev, shape, dtype):
     # against fp32 arithmetic as well (the bound of the build target)
     ref32 = y.float() * F.silu(gate.float())
     assert rel_l2(out.float(), ref32) < TOL[dtype]
+
+
+@pytest.mark.parametrize("K,dtype", [(3, torch.bfloat16), (4, torch.float32), (2, torch.bfloat16)])
+def test_convolution_alone_prefill_and_steps(dev, K, dtype):
+    """The ungated form (ShortConvolution as a mixer of its own): prefill, exact state, decode steps."""
+    from based_amd import ops
+
+    B, L, D, T = 2, 77, 64, 5
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(B, L + T, D, generator=g).to(dtype)
+    w = (torch.randn(D, 1, K, generator=g) * 0.5).to(dtype)
+    ref = O.short_conv(x.float(), w[:, 0].float())
+    tol = 5e-3 if dtype == torch.bfloat16 else 1e-5
+    xd, wd = x.to(dev), w.to(dev)
+    state = torch.zeros(B, D, K, dtype=dtype, device=dev)
+    y = ops.gated_conv_prefill(xd[:, :L], wd, None, state=state, gated=False)
+    assert y.shape == (B, L, D) and rel_l2(y.float(), ref[:, :L]) < tol
+    assert torch.equal(state.cpu(), x[:, L - K:L].transpose(1, 2))
+    for t in range(L, L + T):
+        yt = ops.gated_conv_step(xd[:, t:t + 1], state, wd, None, gated=False)
+        assert rel_l2(yt.float(), ref[:, t:t + 1]) < tol

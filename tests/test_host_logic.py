@@ -88,7 +88,7 @@ def test_cpu_modules_fail_loudly():
         RMSNorm(32)(x)
     with pytest.raises(ValueError):
         GatedMlp(32, hidden_features=64)(x)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError):
         ShortConvolution(32, kernel_size=3)(x)
     with pytest.raises(NotImplementedError):
         GPTLMHeadModel(based_360m_config(n_layer=1, vocab_size=64, rms_norm=False))

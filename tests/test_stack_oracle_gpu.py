@@ -112,6 +112,8 @@ BASE_CONFIG = {
     "scale_attn_by_inverse_layer_idx": False, "n_inner": 1408 * 2, "mlp_type": "alt",
 }
 REFERENCE_CONFIGS = {
+    "conv": {"mixer": {"_target_": "based.models.mixers.convolution.ShortConvolution", "kernel_size": 3, "use_cuda": False},
+             **BASE_CONFIG},
     "base_conv": {"mixer": {"_target_": "based.models.mixers.convolution.BaseConv", "kernel_size": 3, "l_max": 2048},
                   **BASE_CONFIG},
     "linear_attn": {"feature_dim": 16,
@@ -126,7 +128,7 @@ REFERENCE_CONFIGS = {
 }
 
 
-@pytest.mark.parametrize("config", ["base_conv", "linear_attn", "sliding"])
+@pytest.mark.parametrize("config", ["conv", "base_conv", "linear_attn", "sliding"])
 @pytest.mark.parametrize("prefill_size", [1, 128])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_reference_generation_configs_as_written(dev, config, prefill_size, dtype):
