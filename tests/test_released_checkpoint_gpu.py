@@ -119,6 +119,16 @@ def test_released_layout_checkpoint_loads_and_generates(dev, tmp_path):
     for i, sc in enumerate(out.scores):
         _assert_reference_bound(sc, O.stack_forward(seqs[:, : P + i], sd32, cfg)[:, -1], f"cached decode step {i}")
 
+    # the same request through the recorded decode graph (device-side positions feed the 129-row window
+    # step and its rotary): same tokens, logits equal to bf16 noise
+    print("released-layout checkpoint: graph decode", flush=True)
+    graphed = model.generate(input_ids=ids.to(dev), max_length=P + n_new, return_dict_in_generate=True,
+                             output_scores=True, top_k=1, cg=True)
+    assert torch.equal(graphed.sequences.cpu(), seqs)
+    for i, (a, b) in enumerate(zip(graphed.scores, out.scores)):
+        err = float((a.float() - b.float()).norm() / b.float().norm())
+        assert err < 1e-3, f"graph step {i}: rel-L2 {err:.2e} against eager"
+
 
 def test_released_360m_shape_builds_with_window_256(dev):
     """The full-width released configuration: constructs, runs a 300-token prefill and two decode
