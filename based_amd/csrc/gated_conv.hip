@@ -15,7 +15,7 @@
 
 namespace based {
 
-constexpr int kConvTokens = 16;   // tokens per thread in the prefill kernel
+constexpr int kConvTokens = 8;   // tokens per thread in the prefill kernel
 constexpr int kConvMaxK = 4;      // supported kernel sizes: 2..4
 
 template <typename T> struct Vec16;
