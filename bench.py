@@ -326,14 +326,16 @@ def bench_conv(torch, ops, steps, warmup, B=4, L=2048, D=2048, K=3, decode_B=128
     }
 
 
-def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128):
+def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128, released=False):
     """configs[3]: the 27-layer 360M-shaped stack (random weights, bf16): prefill of 2048 tokens,
-    then greedy decoding, eagerly and through the recorded decode graph."""
-    from based_amd.stack import GPTLMHeadModel, based_360m_config
+    then greedy decoding, eagerly and through the recorded decode graph.  released=True: the
+    released checkpoint's configuration instead (window_size 256, rotary, graph decoding only)."""
+    from based_amd.stack import GPTLMHeadModel, based_360m_config, based_360m_released_config
 
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
-    model = GPTLMHeadModel(based_360m_config(), device=dev, dtype=torch.bfloat16).eval()
+    cfg = based_360m_released_config() if released else based_360m_config()
+    model = GPTLMHeadModel(cfg, device=dev, dtype=torch.bfloat16).eval()
     ids = torch.randint(0, 50277, (B, prefill_len), dtype=torch.long, device=dev)
     out = {"B": B, "prefill_len": prefill_len, "new_tokens": new_tokens}
     with torch.inference_mode():
@@ -344,7 +346,7 @@ def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128):
         torch.cuda.synchronize()
         out["prefill_ms"] = (time.perf_counter() - t0) * 1e3
         out["prefill_tok_s"] = B * prefill_len / (out["prefill_ms"] * 1e-3)
-    for name, cg in (("eager", False), ("graph", True)):
+    for name, cg in ((("graph", True),) if released else (("eager", False), ("graph", True))):
         model.generate(input_ids=ids, max_length=prefill_len + new_tokens, cg=cg)  # warm-up / graph capture
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -500,6 +502,10 @@ def main():
     if args.only in (None, "stack"):
         st = bench_stack(torch)
         out["stack"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in st.items()}
+        rel = bench_stack(torch, released=True)
+        out["stack"]["released_config"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in rel.items()
+                                           if k in ("prefill_ms", "prefill_tok_s", "decode_graph_ms_per_token", "decode_graph_tok_s")}
+        out["stack"]["released_config"]["note"] = "window_size 256, rotary_emb_fraction 1, fla_parallel (based-360m.yaml)"
     if args.only == "stack":
         out.update({"value": round(out["stack"]["decode_graph_tok_s"], 1),
                     "ms_per_step": out["stack"]["decode_graph_ms_per_token"], "dtype": "bf16",
