@@ -80,6 +80,8 @@ SIGNATURES = {
         [_P, _P, _P, _P, _P] + [_I64] * 6 + [C.c_float, C.c_int, C.c_int, _P],
     ),
     "based_swiglu": (C.c_int, [_P, _P] + [_I64] * 4 + [C.c_int, _P]),
+    "based_decode_linear": (C.c_int, [_P, _I64, _P, _I64, _P, _I64, _P, _P, _I64, _I64, _I64, _I64, C.c_int,
+                                      _P, _I64, _P, _I64, _P, C.c_float, C.c_int, _P, C.c_int, _P, _P, C.c_int, _P]),
     "based_swa_step": (
         C.c_int,
         [_P, _P, _P, _P, _P, _P, _P, _I64] + [_I64] * 3 + [_I64] * 8 + [_I64] * 3

@@ -429,11 +429,13 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
         P[et][0] = pack_bf16(O[et][0] * inv, O[et][1] * inv);
         P[et][1] = pack_bf16(O[et][2] * inv, O[et][3] * inv);
       }
+      // The swap must not read a register in the two issue slots after a vector instruction wrote
+      // it; the compiler does not look into inline assembly, so each one carries the wait.
 #pragma unroll
       for (int e = 0; e < 2; ++e)
 #pragma unroll
         for (int d = 0; d < 2; ++d)
-          asm volatile("v_permlane16_swap_b32 %0, %1" : "+v"(P[e][d]), "+v"(P[e + 2][d]));
+          asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(P[e][d]), "+v"(P[e + 2][d]));
       {
         const int tau = 16 * nt + col;
         if (tau < ntok) {

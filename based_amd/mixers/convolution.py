@@ -75,6 +75,29 @@ class BaseConv(nn.Module):
     def forward(self, u, position_ids=None, inference_params=None, *args, **kwargs):
         return self.out_proj(self._gated_conv_hip(self.in_proj(u), inference_params))
 
+    def supports_decode_step(self) -> bool:
+        from .. import ops
+
+        return ops.decode_linear_weight_ok(self.in_proj.weight) and ops.decode_linear_weight_ok(self.out_proj.weight)
+
+    def decode_step(self, u, inference_params, **prologue):
+        """One token per sequence with the projections as `ops.decode_linear` launches: u (b, d_model)
+        bf16 -> (b, d_model).  `prologue` goes to in_proj (the block's residual add + norm,
+        possibly the embedding gather)."""
+        from .. import ops
+
+        state = self.conv._get_state(inference_params)
+        rows = prologue["row_index"].numel() if prologue.get("row_index") is not None else u.shape[0]
+        if self.in_proj.weight.shape[1] <= 2048 and self.conv.kernel_size <= 4:
+            # in_proj with the convolution step in its tail: one launch
+            y = ops.decode_linear(u, self.in_proj.weight, self.in_proj.bias, epilogue=ops.EPILOGUE_GATED_CONV_STEP,
+                                  conv_state=state[:rows], conv_weight=self.conv.conv.weight,
+                                  conv_bias=self.conv.conv.bias, **prologue)
+        else:
+            x = ops.decode_linear(u, self.in_proj.weight, self.in_proj.bias, **prologue)
+            y = ops.gated_conv_step(x, state[:rows], self.conv.conv.weight, self.conv.conv.bias)
+        return ops.decode_linear(y, self.out_proj.weight, self.out_proj.bias)
+
     def _gated_conv_hip(self, u, inference_params):
         """silu(conv(u1)) * u2 and the state handling of ShortConvolution.forward/step in one launch."""
         from .. import ops

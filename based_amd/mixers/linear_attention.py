@@ -127,6 +127,25 @@ class LinearAttention(nn.Module):
             inference_params.key_value_memory_dict[self.layer_idx] = (kv_state, k_state)
         return y
 
+    def decode_step(self, x: torch.Tensor, inference_params: InferenceParams, **prologue) -> torch.Tensor:
+        """One token per sequence with the projections as `ops.decode_linear` launches: x (b, d_model)
+        bf16 -> (b, d_model).  `prologue` goes to the first projection (the block's residual add +
+        norm, possibly the embedding gather, fused in front of it); with a `row_index` in it, x is
+        the table the rows are gathered from."""
+        qkv = ops.decode_linear(x, self._stacked_qkv_weight(), **prologue)
+        b = qkv.shape[0]
+        nq = self.feature_dim * self.num_heads
+        q = qkv[:, :nq].view(b, self.num_heads, 1, self.feature_dim)
+        k = qkv[:, nq:2 * nq].view(b, self.num_heads, 1, self.feature_dim)
+        v = qkv[:, 2 * nq:].view(b, self.num_heads, 1, self.head_dim)
+        kv_state, k_state = self._get_inference_cache(inference_params)
+        y = ops.linear_attn_step(q, k, v, kv_state[:b], k_state[:b], eps=self.eps)
+        return ops.decode_linear(y.view(b, self.num_heads * self.head_dim), self.out_proj.weight, self.out_proj.bias)
+
+    def supports_decode_step(self) -> bool:
+        return all(ops.decode_linear_weight_ok(w) for w in
+                   (self.proj_q.weight, self.proj_k.weight, self.proj_v.weight, self.out_proj.weight))
+
     def _stacked_qkv_weight(self) -> torch.Tensor:
         """[proj_q; proj_k; proj_v] weights as one matrix, rebuilt whenever one of them has been
         written to or replaced (tensor version counters and storage addresses are the key)."""

@@ -149,6 +149,32 @@ class SlidingAttention(nn.Module):
                                             self.num_heads_kv, self.head_dim, dtype=torch.bfloat16, device=like.device)
         return d[self.layer_idx]
 
+    def supports_decode_step(self) -> bool:
+        in_kernel_rotary = self.head_dim == 64 and self.rotary_emb_dim == 64 and not self.rotary_emb.interleaved \
+            if self.rotary_emb_dim > 0 else True
+        return (in_kernel_rotary and ops.decode_linear_weight_ok(self.Wqkv.weight)
+                and ops.decode_linear_weight_ok(self.out_proj.weight))
+
+    def decode_step(self, x, inference_params, **prologue):
+        """One token per sequence with the projections as `ops.decode_linear` launches: x (b, hidden)
+        bf16 -> (b, hidden).  `prologue` goes to the first projection (the block's residual add +
+        norm, possibly the embedding gather)."""
+        qkv = ops.decode_linear(x, self.Wqkv.weight, self.Wqkv.bias, **prologue)
+        b = qkv.shape[0]
+        qkv = qkv.view(b, 1, 3, self.num_heads, self.head_dim)
+        offset = inference_params.seqlen_offset
+        rope = None
+        if self.rotary_emb_dim > 0:
+            rope = self.rotary_emb.tables(max(inference_params.max_seqlen, offset + 1), qkv.device)
+        cache = self._cache(inference_params, qkv)
+        b0 = inference_params.batch_size_offset
+        pos = offset
+        if inference_params.lengths_per_sample is not None:
+            pos = inference_params.lengths_per_sample[b0:b0 + b]
+        context = ops.swa_step(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], cache[b0:b0 + b], pos,
+                               w_left=self.window[0], scale=self.softmax_scale, rope=rope)
+        return ops.decode_linear(context.view(b, self.embed_dim), self.out_proj.weight, self.out_proj.bias)
+
     def forward(self, x, x_kv=None, key_padding_mask=None, cu_seqlens=None, max_seqlen=None,
                 mixer_subset=None, inference_params=None, **kwargs):
         """x (batch, seqlen, hidden) -> (batch, seqlen, hidden)."""

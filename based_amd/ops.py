@@ -431,3 +431,118 @@ def swiglu(u) -> torch.Tensor:
         _lib.check(_lib.lib().based_swiglu(u2.data_ptr(), out.data_ptr(), u2.shape[0], F, u2.stride(0), out.stride(0),
                                            _dtype_code(u), _stream_ptr(u)))
     return out.view(*u.shape[:-1], F)
+
+
+DECODE_LINEAR_MAX_ROWS = 32  # BASED_DECODE_LINEAR_MAX_ROWS of include/based_hip.h
+PROLOGUE_NONE, PROLOGUE_ADD_RMS_NORM, PROLOGUE_SWIGLU = 0, 1, 2
+EPILOGUE_NONE, EPILOGUE_SWIGLU, EPILOGUE_GATED_CONV_STEP = 0, 1, 2
+
+
+def decode_linear_weight_ok(weight: torch.Tensor) -> bool:
+    """Whether `decode_linear` takes projections through this weight: bf16 (N, K) on the GPU with
+    contiguous rows, K a multiple of 8 up to 4096."""
+    return (weight.is_cuda and weight.dtype == torch.bfloat16 and weight.dim() == 2 and weight.stride(1) == 1
+            and weight.stride(0) % 8 == 0 and weight.shape[1] % 8 == 0 and weight.shape[1] <= 4096)
+
+
+def decode_linear(x, weight, bias=None, *, prologue: int = PROLOGUE_NONE, residual_in=None, residual_out=None,
+                  norm_weight=None, eps: float = 1e-5, row_index=None, epilogue: int = EPILOGUE_NONE,
+                  conv_state=None, conv_weight=None, conv_bias=None, out: Optional[torch.Tensor] = None
+                  ) -> torch.Tensor:
+    """y = epi(pro(x) @ weight.T (+ bias)) for the few rows of a single-token step, one launch.
+
+    x: (M, K) bf16 rows (M <= 32; any leading shape is flattened), or for PROLOGUE_SWIGLU (M, 2K):
+    value | gate.  weight: (N, K) bf16; bias None or (N).  PROLOGUE_ADD_RMS_NORM first forms
+    r = x + residual_in (fp32, residual_in may be None), writes r to residual_out (fp32, may be
+    None, never residual_in itself) and projects rms_norm(r) * norm_weight.  row_index: None, or an
+    int64 device vector of M row numbers into x (the embedding table).
+    EPILOGUE_SWIGLU: weight is (2F, K), y[:, f] = p[:, f] * silu(p[:, F + f]).
+    EPILOGUE_GATED_CONV_STEP: weight is (2F, K); the gated short-convolution step on p with
+    conv_state (M, F, k) rolled in place, conv_weight the (F, 1, k) or (F, k) Conv1d weight,
+    conv_bias None or (F).  Returns y (M, N) or (M, F), written into `out` when given."""
+    N, K = weight.shape
+    x2 = x if x.dim() == 2 else x.reshape(-1, x.shape[-1])
+    M = x2.shape[0] if row_index is None else row_index.numel()
+    n_out = N if epilogue == EPILOGUE_NONE else N // 2
+    key = ("decode_linear", x2.shape, x2.stride(), x2.dtype, x2.device, weight.shape, weight.stride(), weight.dtype,
+           weight.device, prologue, epilogue,
+           None if bias is None else (bias.shape, bias.dtype, bias.device, bias.stride()),
+           None if residual_in is None else (residual_in.shape, residual_in.stride(), residual_in.dtype, residual_in.device),
+           None if residual_out is None else (residual_out.shape, residual_out.stride(), residual_out.dtype, residual_out.device),
+           None if norm_weight is None else (norm_weight.shape, norm_weight.dtype, norm_weight.device, norm_weight.stride()),
+           None if row_index is None else (row_index.shape, row_index.dtype, row_index.device, row_index.stride()),
+           None if conv_state is None else (conv_state.shape, conv_state.stride(), conv_state.dtype, conv_state.device),
+           None if conv_weight is None else (conv_weight.shape, conv_weight.stride(), conv_weight.dtype, conv_weight.device),
+           None if conv_bias is None else (conv_bias.shape, conv_bias.stride(), conv_bias.dtype, conv_bias.device))
+    if key not in _CHECKED:
+        _require_cuda(x2, weight)
+        if x2.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            raise ValueError("decode_linear takes bfloat16 activations and weights")
+        if weight.dim() != 2 or weight.stride(1) != 1 or x2.stride(1) != 1:
+            raise ValueError("weight must be (N, K) and rows of x and weight contiguous")
+        if x2.shape[1] != (2 * K if prologue == PROLOGUE_SWIGLU else K):
+            raise ValueError(f"x {tuple(x.shape)} does not match weight {tuple(weight.shape)} (prologue {prologue})")
+        if M > DECODE_LINEAR_MAX_ROWS:
+            raise ValueError(f"decode_linear takes at most {DECODE_LINEAR_MAX_ROWS} rows, got {M}")
+        if bias is not None:
+            _require_cuda(x2, bias)
+            if tuple(bias.shape) != (N,) or bias.dtype != torch.bfloat16 or not bias.is_contiguous():
+                raise ValueError(f"bias must be a contiguous bfloat16 ({N},)")
+        if prologue == PROLOGUE_ADD_RMS_NORM:
+            if norm_weight is None:
+                raise ValueError("the norm prologue needs norm_weight")
+            _require_cuda(x2, norm_weight)
+            if tuple(norm_weight.shape) != (K,) or norm_weight.dtype != torch.bfloat16 or not norm_weight.is_contiguous():
+                raise ValueError(f"norm_weight must be a contiguous bfloat16 ({K},)")
+            for r in (residual_in, residual_out):
+                if r is not None:
+                    _require_cuda(x2, r)
+                    if r.dtype != torch.float32 or r.dim() != 2 or tuple(r.shape) != (M, K) or r.stride(1) != 1:
+                        raise ValueError(f"residuals must be float32 ({M}, {K}) with contiguous rows")
+        elif residual_in is not None or residual_out is not None or norm_weight is not None:
+            raise ValueError("residual and norm arguments belong to PROLOGUE_ADD_RMS_NORM")
+        if row_index is not None:
+            _require_cuda(x2, row_index)
+            if row_index.dtype != torch.int64 or row_index.dim() != 1 or not row_index.is_contiguous():
+                raise ValueError("row_index must be a contiguous int64 device vector")
+        if epilogue != EPILOGUE_NONE and N % 2 != 0:
+            raise ValueError("a paired epilogue needs an even number of weight rows")
+        if epilogue == EPILOGUE_GATED_CONV_STEP:
+            if conv_state is None or conv_weight is None:
+                raise ValueError("the convolution epilogue needs conv_state and conv_weight")
+            _require_cuda(x2, conv_state, conv_weight)
+            k = conv_weight.shape[-1]
+            if (conv_weight.numel() != n_out * k or conv_weight.shape[0] != n_out or not conv_weight.is_contiguous()
+                    or conv_weight.dtype != torch.bfloat16):
+                raise ValueError(f"conv_weight must be a contiguous bfloat16 ({n_out}, 1, k), got {tuple(conv_weight.shape)}")
+            if tuple(conv_state.shape) != (M, n_out, k) or not conv_state.is_contiguous():
+                raise ValueError(f"conv_state must be a contiguous ({M}, {n_out}, {k}) tensor, got {tuple(conv_state.shape)}")
+            _dtype_code(conv_state)
+            if conv_bias is not None:
+                _require_cuda(x2, conv_bias)
+                if tuple(conv_bias.shape) != (n_out,) or conv_bias.dtype != torch.bfloat16 or not conv_bias.is_contiguous():
+                    raise ValueError(f"conv_bias must be a contiguous bfloat16 ({n_out},)")
+        elif conv_state is not None or conv_weight is not None or conv_bias is not None:
+            raise ValueError("convolution arguments belong to EPILOGUE_GATED_CONV_STEP")
+        _CHECKED[key] = True
+    if out is None:
+        y = torch.empty(M, n_out, dtype=torch.bfloat16, device=x2.device)
+    else:
+        y = out
+        if tuple(y.shape) != (M, n_out) or y.dtype != torch.bfloat16 or y.device != x2.device or y.stride(1) != 1:
+            raise ValueError(f"out must be a ({M}, {n_out}) bfloat16 tensor on {x2.device} with contiguous rows")
+    conv = epilogue == EPILOGUE_GATED_CONV_STEP
+    with _on_device(x2.device):
+        _lib.check(_lib.lib().based_decode_linear(
+            x2.data_ptr(), x2.stride(0), None if row_index is None else row_index.data_ptr(),
+            x2.shape[0] if row_index is not None else 0,
+            weight.data_ptr(), weight.stride(0), None if bias is None else bias.data_ptr(),
+            y.data_ptr(), y.stride(0), M, N, K, prologue,
+            None if residual_in is None else residual_in.data_ptr(), 0 if residual_in is None else residual_in.stride(0),
+            None if residual_out is None else residual_out.data_ptr(), 0 if residual_out is None else residual_out.stride(0),
+            None if norm_weight is None else norm_weight.data_ptr(), float(eps), epilogue,
+            conv_state.data_ptr() if conv else None, _dtype_code(conv_state) if conv else 0,
+            conv_weight.data_ptr() if conv else None,
+            conv_bias.data_ptr() if conv and conv_bias is not None else None,
+            conv_weight.shape[-1] if conv else 0, _stream_ptr(x2)))
+    return y

@@ -239,6 +239,41 @@ class Block(nn.Module):
         (block.py:134-139), one kernel."""
         return ops.add_rms_norm(hidden_states, residual, norm.weight, norm.eps, self.residual_in_fp32)
 
+    def supports_decode_step(self) -> bool:
+        mlp = self.mlp
+        return (getattr(self.mixer, "supports_decode_step", lambda: False)()
+                and mlp.mlp_type == "base" and mlp.activation == "swiglu"
+                and ops.decode_linear_weight_ok(mlp.fc1.weight) and ops.decode_linear_weight_ok(mlp.fc2.weight)
+                and self.norm1.weight.dtype == torch.bfloat16 and self.residual_in_fp32)
+
+    def decode_step(self, hidden_states, residual, spare, inference_params, row_index=None):
+        """The block for one token per sequence in four to five launches: both norms run inside the
+        projection that consumes them (`ops.decode_linear`), the SwiGLU gate in the tail of fc1.
+        hidden_states (b, dim) bf16 (or the embedding table with `row_index`), residual fp32
+        (b, dim) or None; `spare` is a second fp32 (b, dim) buffer: the two take turns as the
+        input and the output of the residual stream.  Returns (hidden, residual, spare)."""
+        if residual is None:
+            residual_in, mid, last = None, spare[0], spare[1]
+        else:
+            residual_in, mid, last = residual, spare, residual
+        norm = dict(prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=residual_in, residual_out=mid,
+                    norm_weight=self.norm1.weight, eps=self.norm1.eps)
+        if row_index is not None:
+            norm["row_index"] = row_index
+        hidden_states = self.mixer.decode_step(hidden_states, inference_params, **norm)
+        norm = dict(prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=mid, residual_out=last,
+                    norm_weight=self.norm2.weight, eps=self.norm2.eps)
+        fc1, fc2 = self.mlp.fc1, self.mlp.fc2
+        if fc1.weight.shape[1] <= 2048:
+            # the gate in the tail of fc1
+            gated = ops.decode_linear(hidden_states, fc1.weight, fc1.bias, epilogue=ops.EPILOGUE_SWIGLU, **norm)
+            hidden_states = ops.decode_linear(gated, fc2.weight, fc2.bias)
+        else:
+            # wider models: the gate in front of fc2
+            gate_in = ops.decode_linear(hidden_states, fc1.weight, fc1.bias, **norm)
+            hidden_states = ops.decode_linear(gate_in, fc2.weight, fc2.bias, prologue=ops.PROLOGUE_SWIGLU)
+        return hidden_states, last, mid
+
     def forward(self, hidden_states, residual=None, mixer_kwargs=None, position_ids=None, decay=None):
         hidden_states, residual = self._add_norm(self.norm1, hidden_states, residual)
         mixer_kwargs = mixer_kwargs or {}
@@ -292,7 +327,49 @@ class GPTModel(nn.Module):
         return {i: layer.allocate_inference_cache(batch_size, max_seqlen, dtype=dtype, **kwargs)
                 for i, layer in enumerate(self.layers)}
 
+    # Single-token steps of a bf16 model run through `decode_layers`: every projection is an
+    # `ops.decode_linear` launch with the element-wise work in front of it folded in.  Set to False
+    # to send them through the general path (torch GEMMs + stand-alone norm and gate kernels).
+    fused_decode = True
+
+    def decode_layers_ok(self, input_ids, inference_params) -> bool:
+        if not (self.fused_decode and inference_params is not None and inference_params.seqlen_offset > 0
+                and input_ids.shape[1] == 1 and input_ids.shape[0] <= ops.DECODE_LINEAR_MAX_ROWS
+                and input_ids.is_cuda and not torch.is_grad_enabled()
+                and self.config.max_position_embeddings == 0):
+            return False
+        # the answer depends on dtypes and devices of the parameters only: worked out once per
+        # (dtype, device) of the embedding table
+        table = self.embeddings.word_embeddings.weight
+        cached = self.__dict__.get("_decode_layers_supported")
+        if cached is None or cached[0] != (table.dtype, table.device):
+            ok = (ops.decode_linear_weight_ok(table) and self.ln_f.weight.dtype == torch.bfloat16
+                  and all(layer.supports_decode_step() for layer in self.layers))
+            cached = ((table.dtype, table.device), ok)
+            self.__dict__["_decode_layers_supported"] = cached
+        return cached[1]
+
+    def decode_layers(self, input_ids, inference_params):
+        """All blocks for one token per sequence.  Returns (hidden (b, dim) bf16, residual (b, dim)
+        fp32): the inputs of the closing add + norm, which the caller folds into what follows."""
+        b = input_ids.shape[0]
+        table = self.embeddings.word_embeddings.weight
+        key = (b, table.device)
+        buffers = self.__dict__.setdefault("_decode_residuals", {}).get(key)
+        if buffers is None:
+            buffers = tuple(torch.empty(b, table.shape[1], dtype=torch.float32, device=table.device) for _ in range(2))
+            self._decode_residuals[key] = buffers
+        ids = input_ids.reshape(-1).contiguous()  # a column of a wider id tensor is a strided view
+        hidden_states, residual, spare = self.layers[0].decode_step(table, None, buffers, inference_params, row_index=ids)
+        for layer in self.layers[1:]:
+            hidden_states, residual, spare = layer.decode_step(hidden_states, residual, spare, inference_params)
+        return hidden_states, residual
+
     def forward(self, input_ids, position_ids=None, inference_params=None, stream=None):
+        if self.decode_layers_ok(input_ids, inference_params):
+            hidden_states, residual = self.decode_layers(input_ids, inference_params)
+            return ops.add_rms_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.eps,
+                                    want_residual=False)[0].unsqueeze(1)
         hidden_states = self.embeddings.word_embeddings(input_ids)
         if self.config.max_position_embeddings > 0:
             if position_ids is None:
@@ -376,9 +453,18 @@ class GPTLMHeadModel(nn.Module, GenerationMixin):
 
     def forward(self, input_ids, position_ids=None, inference_params=None, num_last_tokens=0, stream=None, **kwargs):
         assert input_ids.ndim == 2, f"Expected `input_ids` to have shape [b, slen], but got shape {input_ids.shape}"
+        CausalLMOutput = namedtuple("CausalLMOutput", ["logits"])
+        if (self.transformer.decode_layers_ok(input_ids, inference_params)
+                and ops.decode_linear_weight_ok(self.lm_head.weight)):
+            # closing add + norm inside the LM head's projection
+            hidden_states, residual = self.transformer.decode_layers(input_ids, inference_params)
+            ln_f = self.transformer.ln_f
+            logits = ops.decode_linear(hidden_states, self.lm_head.weight, self.lm_head.bias,
+                                       prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=residual,
+                                       norm_weight=ln_f.weight, eps=ln_f.eps)
+            return CausalLMOutput(logits=logits.unsqueeze(1))
         hidden_states = self.transformer(input_ids, position_ids=position_ids, inference_params=inference_params,
                                          stream=stream)
         if num_last_tokens > 0:
             hidden_states = hidden_states[:, -num_last_tokens:]
-        CausalLMOutput = namedtuple("CausalLMOutput", ["logits"])
         return CausalLMOutput(logits=self.lm_head(hidden_states))

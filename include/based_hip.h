@@ -292,6 +292,60 @@ BASED_API int based_swiglu(const void* u, void* out, int64_t rows, int64_t F, in
                  int io_dtype, void* stream);
 
 /*
+ * A projection of a single-token step, with the element-wise operation in front of it:
+ *
+ *     y[m, n] = sum_k pro(x)[m, k] * weight[n, k]  (+ bias[n])       m < M <= 32, bf16, fp32 sums
+ *
+ * Stands in for the `nn.Linear` calls of a decoding step, where the batch is the only row
+ * dimension: proj_q / proj_k / proj_v and out_proj (based/models/mixers/linear_attention.py:
+ * 105-108,126-128,251-252), Wqkv and out_proj (slide_attention.py:332-336,541,599), in_proj and
+ * out_proj of BaseConv (convolution.py:195-210), fc1 and fc2 (based/models/mlp.py:141-157) and
+ * the LM head (gpt.py:794-827); and, through `prologue`, for what the reference runs between them:
+ *
+ *   BASED_PROLOGUE_NONE          pro(x) = x, (M, K)
+ *   BASED_PROLOGUE_ADD_RMS_NORM  r = x + residual_in (r = x if residual_in is NULL), fp32;
+ *                                pro(x) = rms_norm(bf16(r)) * norm_weight, rounded to bf16;
+ *                                residual_out (if not NULL, and never residual_in itself) <- r.
+ *                                The arithmetic of based_add_rms_norm (block.py:134-139,151-155;
+ *                                based/ops/triton/layer_norm.py:117-118).
+ *   BASED_PROLOGUE_SWIGLU        x is (M, 2K); pro(x)[m, k] = x[m, k] * silu(x[m, K + k]), the
+ *                                arithmetic of based_swiglu (mlp.py:147-151).
+ *
+ * and, through `epilogue`, for what consumes the output of a projection in (value, gate) pairs;
+ * weight then has N = 2F rows, value rows first, and y is (M, F):
+ *
+ *   BASED_EPILOGUE_NONE             y = the projection
+ *   BASED_EPILOGUE_SWIGLU           y[m, f] = p[m, f] * silu(p[m, F + f]) with p the projection
+ *                                   rounded to bf16: fc1 and the gate (mlp.py:147-151)
+ *   BASED_EPILOGUE_GATED_CONV_STEP  one step of BaseConv's gated short convolution on p: the
+ *                                   arithmetic of based_gated_conv_step (convolution.py:78-109,
+ *                                   195-210); conv_state (M, F, conv_k) of conv_state_dtype is
+ *                                   rolled and updated in place, conv_weight (F, conv_k) and
+ *                                   conv_bias (F, or NULL) are bf16, conv_k 2 to 4.
+ *   Paired epilogues take K up to 2048 and not the SwiGLU prologue.
+ *
+ *   x            : rows at x[m * x_row_stride]; with x_row_index (M int64 values on the device)
+ *                  row m is x[x_row_index[m] * x_row_stride] instead: the embedding lookup of the
+ *                  first block (gpt.py:622-631).  An index outside [0, x_index_rows) gives that
+ *                  row of y NaN; nothing is read out of bounds.
+ *   weight       : (N, K) rows at weight[n * w_row_stride]; bias NULL or (N) contiguous
+ *   y            : (M, N) or (M, F), rows at y[m * y_row_stride]
+ *   residual_in / residual_out : fp32 (M, K), rows at the given strides (norm prologue only)
+ * K multiple of 8, at most 4096; row strides of x and weight multiples of 8 elements, of the
+ * residuals multiples of 4; x, weight, norm_weight and the residuals 16-byte aligned.
+ */
+enum { BASED_PROLOGUE_NONE = 0, BASED_PROLOGUE_ADD_RMS_NORM = 1, BASED_PROLOGUE_SWIGLU = 2 };
+enum { BASED_EPILOGUE_NONE = 0, BASED_EPILOGUE_SWIGLU = 1, BASED_EPILOGUE_GATED_CONV_STEP = 2 };
+#define BASED_DECODE_LINEAR_MAX_ROWS 32
+BASED_API int based_decode_linear(const void* x, int64_t x_row_stride, const int64_t* x_row_index,
+                        int64_t x_index_rows, const void* weight, int64_t w_row_stride,
+                        const void* bias, void* y, int64_t y_row_stride, int64_t M, int64_t N,
+                        int64_t K, int prologue, const float* residual_in, int64_t ri_row_stride,
+                        float* residual_out, int64_t ro_row_stride, const void* norm_weight,
+                        float eps, int epilogue, void* conv_state, int conv_state_dtype,
+                        const void* conv_weight, const void* conv_bias, int conv_k, void* stream);
+
+/*
  * The same sliding-window attention for head dimensions other than 64 (any multiple of 8 up to
  * 128), bf16, fp32 arithmetic, one wavefront per query: not a performance path, it exists so
  * that models with other head sizes (the reference's own test models have 16-dim heads,
