@@ -63,8 +63,10 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 // is pointed at these instead of being skipped or having its result replaced: a load under a
 // branch, or one whose result feeds a select, is waited for on the spot, and the memory round
 // trips of a wavefront then run one after the other instead of together.
-__device__ __attribute__((aligned(64))) const uint32_t kZeroPage[16] = {};
-__device__ __attribute__((aligned(16))) const uint32_t kNanPage[4] = {0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u};
+// (Not declared const: constant data lives in another address space, and a pointer that may be
+// either turns every load through it into a flat one, which is waited for like a branch.)
+__device__ __attribute__((aligned(64))) uint32_t kZeroPage[16] = {};
+__device__ __attribute__((aligned(16))) uint32_t kNanPage[4] = {0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u};
 
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
@@ -82,11 +84,12 @@ template <int N> __device__ __forceinline__ void reduce_tree(const float (&v)[N]
 #pragma unroll
   for (int i = 0; i < N / 2; ++i) {
     // Lanes 32..63 of a trade places with lanes 0..31 of b.  Inline assembly: the compiler's
-    // builtin returns the same register for both results here.  The swap must not read a register
-    // in the two issue slots after a vector instruction wrote it, and the compiler cannot see
-    // into the assembly, hence the s_nop.
+    // builtin returns the same register for both results here.  A vector instruction must not
+    // read the result of a dot-product instruction in the three issue slots after it (two after
+    // other vector instructions); the compiler cannot see into the assembly and the sums come
+    // straight from v_dot2, hence the s_nop.
     float a = v[2 * i], b = v[2 * i + 1];
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    asm volatile("s_nop 3\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
     half[i] = a + b;
   }
 #pragma unroll
@@ -292,12 +295,8 @@ __global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_
   const int w16 = lane >> 4, j16 = lane & 15;
   const int own_idx = 4 * j16 + 2 * (w16 & 1) + (w16 >> 1);
   const int own_r = own_idx / MT, own_m = own_idx % MT;
-  for (;;) {
-    const int g_next = g + g_step;
-    const bool more = g_next < a.n_groups;
-    u32x4 wnext[R][C];
-    if (more) load_rows(g_next, wnext);
-
+  // one row group: products, sums across the lanes, tail, store
+  auto finish_group = [&](const u32x4 (&wcur)[R][C], int g) {
     // what the tail needs from memory is asked for before the products, not after the sums
     const int out_col = EPI == kEpiNone ? g * R + own_r : g * RH + own_r;
     const bool owner = j16 < kOwners && own_m < a.M && out_col < (EPI == kEpiNone ? a.N : F);
@@ -375,12 +374,29 @@ __global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_
         a.y[(long)own_m * a.y_sr + out_col] = from_f32<__bf16>(out);
       }
     }
-    if (!more) break;
-    g = g_next;
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int c = 0; c < C; ++c) wcur[r][c] = wnext[r][c];
+  };
+
+  if (g_step >= a.n_groups) {  // one round (all but the LM head)
+    finish_group(wcur, g);
+    return;
+  }
+  // Several rounds: the rows of the next group are requested before the current one is worked
+  // on, into a second set of registers (the two sets take turns, nothing is copied), and always
+  // (past the end: the current group again), so that the number of loads in flight is the same on
+  // every path and the wait before the products can leave exactly those outstanding.
+  u32x4 wother[R][C];
+  for (;;) {
+    const int g1 = g + g_step;
+    const bool more1 = g1 < a.n_groups;
+    load_rows(more1 ? g1 : g, wother);
+    finish_group(wcur, g);
+    if (!more1) break;
+    const int g2 = g1 + g_step;
+    const bool more2 = g2 < a.n_groups;
+    load_rows(more2 ? g2 : g1, wcur);
+    finish_group(wother, g1);
+    if (!more2) break;
+    g = g2;
   }
 }
 

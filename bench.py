@@ -359,6 +359,95 @@ def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128, released=False):
     return out
 
 
+def bench_projections(torch, M=4):
+    """The projections of one decoding step of the 27-layer configuration (`based_decode_linear`, M rows =
+    the decoding batch), each timed as a recorded graph of launches over enough independent
+    weight matrices to exceed the last-level cache, next to `torch.nn.functional.linear` on the
+    same matrices.  The LM head (103 MB of weights per launch) carries an HBM roofline."""
+    import torch.nn.functional as F
+
+    from based_amd import ops
+
+    with torch.inference_mode():  # as the decoding loop runs (and as graphs recorded after it must)
+        return _bench_projections(torch, F, ops, M)
+
+
+def _bench_projections(torch, F, ops, M):
+    dev = torch.device("cuda:0")
+    D, F1, V = 1024, 2048, 50280
+
+    def timed_graph(fn, n_sets):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(n_sets):
+                fn(i)
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for i in range(n_sets):
+                    fn(i)
+        torch.cuda.current_stream().wait_stream(side)
+        ms, _ = _events_ms(torch, graph.replay, 10, 2)
+        return ms * 1e3 / n_sets
+
+    def weights(n, k, n_sets):
+        return [torch.randn(n, k, device=dev).mul_(0.05).to(torch.bfloat16) for _ in range(n_sets)]
+
+    x = torch.randn(M, D, device=dev).to(torch.bfloat16)
+    xg = torch.randn(M, F1, device=dev).to(torch.bfloat16)
+    res = torch.randn(M, D, device=dev)
+    res_out = torch.empty_like(res)
+    nw = torch.ones(D, device=dev, dtype=torch.bfloat16)
+    norm = dict(prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=res, residual_out=res_out, norm_weight=nw, eps=1e-5)
+    out = {"M": M, "note": "us per launch inside a recorded graph, weights rotating over > 256 MB; torch = F.linear alone "
+                           "(without the norm / gate / convolution step the fused launch contains)"}
+    cases = [
+        ("out_proj 1024x1024", D, D, lambda w, y: ops.decode_linear(x, w, out=y), x),
+        ("fc2 / conv out_proj 1024x2048", D, F1, lambda w, y: ops.decode_linear(xg, w, out=y), xg),
+        ("norm + qkv 1536x1024", 1536, D, lambda w, y: ops.decode_linear(x, w, out=y, **norm), x),
+        ("norm + fc1 4096x1024 + gate", 2 * F1, D,
+         lambda w, y: ops.decode_linear(x, w, out=y[:, :F1], epilogue=ops.EPILOGUE_SWIGLU, **norm), x),
+    ]
+    for name, n, k, fn, xin in cases:
+        n_sets = min(64, max(4, int(400e6 / (n * k * 2))))
+        ws = weights(n, k, n_sets)
+        y = torch.empty(M, n, dtype=torch.bfloat16, device=dev)
+        mine = timed_graph(lambda i: fn(ws[i], y), n_sets)
+        ref = timed_graph(lambda i: F.linear(xin, ws[i]), n_sets)
+        out[name] = {"us": round(mine, 2), "torch_linear_us": round(ref, 2), "weight_MB": round(n * k * 2 / 1e6, 1),
+                     "weight_sets": n_sets}
+        del ws
+    # in_proj of BaseConv with the convolution step in its tail
+    n_sets = 48
+    ws = weights(2 * F1, D, n_sets)
+    state = torch.zeros(M, F1, 3, device=dev, dtype=torch.bfloat16)
+    cw = torch.randn(F1, 1, 3, device=dev).to(torch.bfloat16)
+    cb = torch.zeros(F1, device=dev, dtype=torch.bfloat16)
+    y = torch.empty(M, F1, dtype=torch.bfloat16, device=dev)
+    mine = timed_graph(lambda i: ops.decode_linear(x, ws[i], out=y, epilogue=ops.EPILOGUE_GATED_CONV_STEP, conv_state=state,
+                                                   conv_weight=cw, conv_bias=cb, **norm), n_sets)
+    ref = timed_graph(lambda i: F.linear(x, ws[i]), n_sets)
+    out["norm + in_proj 4096x1024 + conv step"] = {"us": round(mine, 2), "torch_linear_us": round(ref, 2),
+                                                    "weight_MB": round(2 * F1 * D * 2 / 1e6, 1), "weight_sets": n_sets}
+    del ws
+    # LM head: closing norm + 50280 x 1024 projection, 103 MB of weights per launch
+    n_sets = 4
+    ws = weights(V, D, n_sets)
+    y = torch.empty(M, V, dtype=torch.bfloat16, device=dev)
+    mine = timed_graph(lambda i: ops.decode_linear(x, ws[i], out=y, prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=res,
+                                                   norm_weight=nw, eps=1e-5), n_sets)
+    ref = timed_graph(lambda i: F.linear(x, ws[i]), n_sets)
+    nbytes = V * D * 2 + M * D * 6 + M * V * 2
+    gbs = nbytes / (mine * 1e-6) / 1e9
+    out["norm + lm_head 50280x1024"] = {
+        "us": round(mine, 2), "torch_linear_us": round(ref, 2), "weight_MB": round(V * D * 2 / 1e6, 1), "weight_sets": n_sets,
+        "roofline": {"kernel": "decode_linear_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": nbytes}}
+    return out
+
+
 def cpu_baseline_decode(torch, B=128, H=16, dv=64, sample_steps=8):
     """The oracle's recurrent step on the host: `sample_steps` of the 256 steps at full batch."""
     from oracle import based_oracle as O
@@ -431,7 +520,7 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "copy", "machine"], default=None,
+    ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "projections", "copy", "machine"], default=None,
                     help="one workload only; 'copy' is a plain 256 MiB device copy (the library's copy probe) used to "
                          "calibrate the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run; 'machine' the memory "
                          "probes alone")
@@ -506,6 +595,13 @@ def main():
         out["stack"]["released_config"] = {k: (round(v, 3) if isinstance(v, float) else v) for k, v in rel.items()
                                            if k in ("prefill_ms", "prefill_tok_s", "decode_graph_ms_per_token", "decode_graph_tok_s")}
         out["stack"]["released_config"]["note"] = "window_size 256, rotary_emb_fraction 1, fla_parallel (based-360m.yaml)"
+    if args.only in (None, "stack", "projections"):
+        out["projections"] = bench_projections(torch)
+    if args.only == "projections":
+        lm = out["projections"]["norm + lm_head 50280x1024"]
+        out.update({"value": round(4 / (lm["us"] * 1e-6), 1), "ms_per_step": round(lm["us"] * 1e-3, 5), "dtype": "bf16",
+                    "config": {"workload": "closing norm + LM head projection of a decoding step, M=4, 50280 x 1024 bf16"},
+                    "roofline": lm["roofline"]})
     if args.only == "stack":
         out.update({"value": round(out["stack"]["decode_graph_tok_s"], 1),
                     "ms_per_step": out["stack"]["decode_graph_ms_per_token"], "dtype": "bf16",
