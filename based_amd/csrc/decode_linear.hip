@@ -1,5 +1,5 @@
 // Projections of a single-token step for gfx950: y[M, N] = pro(x)[M, K] . W[N, K]^T (+ bias) for
-// M <= 8 rows (the decoding batch), bf16 in and out, fp32 accumulation.
+// M <= 32 rows (the decoding batch, walked 8 at a time), bf16 in and out, fp32 accumulation.
 //
 // At these sizes a projection is a read of its weight matrix (2 .. 8 MB, 100 MB for the LM head)
 // and nothing else: a tiled GEMM leaves the machine idle and costs 6 - 17 us of launch + tail
@@ -144,8 +144,10 @@ __device__ __forceinline__ void lds_barrier() {
 // all its wavefronts through LDS.
 // Wavefronts per workgroup: a prologue is shared by as many wavefronts as there can be rows;
 // without one nothing is shared and single wavefronts spread over the most compute units.
+// One tile of at most MT activation rows (a.M of them, starting at row a.m0 of the call; the
+// pointers in `a` already point at the tile).
 template <int C, int MT, int PRO, int EPI>
-__global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_kernel(const DecodeLinearArgs a) {
+__device__ __forceinline__ void decode_linear_tile(const DecodeLinearArgs& a, bool first_tile) {
   constexpr int WV = PRO == kProNone ? 1 : MT;
   constexpr int R = 8 / C;
   constexpr int RH = R / 2;  // paired epilogues: RH value rows + RH gate rows per group
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_
   const int g_step = n_wg * WV;
   const bool have = g < a.n_groups;
   u32x4 wcur[R][C];
-  if (have) load_rows(g, wcur);  // in flight while the activations are prepared
+  load_rows(have ? g : 0, wcur);  // in flight while the activations are prepared
 
   // ---- activations: packed bf16 pieces of every row.  Without a prologue every wavefront fetches
   // them itself (measured faster than sharing them); a prologue is evaluated once per workgroup
@@ -216,6 +218,7 @@ __global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_
     }
   } else {
   __shared__ u32x4 xs[MT][C][64];
+  if (!first_tile) lds_barrier();  // every wavefront has taken the previous tile out of LDS
   if constexpr (PRO == kProNorm) {
     const int m = wave;
     if (m < a.M) {
@@ -400,6 +403,29 @@ __global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_
   }
 }
 
+// More than MT rows: the tiles are walked inside the launch (the weight rows of a wavefront come
+// from its own L1 / L2 from the second tile on).
+template <int C, int MT, int PRO, int EPI>
+__global__ __launch_bounds__(PRO == kProNone ? 64 : 64 * MT) void decode_linear_kernel(const DecodeLinearArgs a) {
+  if (a.M <= MT) {
+    decode_linear_tile<C, MT, PRO, EPI>(a, true);
+    return;
+  }
+  for (int m0 = 0; m0 < a.M; m0 += MT) {
+    DecodeLinearArgs t = a;
+    t.M = a.M - m0 < MT ? a.M - m0 : MT;
+    t.m0 = m0;
+    if (a.x_index != nullptr)
+      t.x_index = a.x_index + m0;
+    else
+      t.x = a.x + (long)m0 * a.x_sr;
+    t.y = a.y + (long)m0 * a.y_sr;
+    if (a.res_in != nullptr) t.res_in = a.res_in + (long)m0 * a.ri_sr;
+    if (a.res_out != nullptr) t.res_out = a.res_out + (long)m0 * a.ro_sr;
+    decode_linear_tile<C, MT, PRO, EPI>(t, m0 == 0);
+  }
+}
+
 constexpr int kDecodeLinearMaxWaves = 4096;  // row groups beyond this many are walked in a loop
 
 template <int C, int MT, int EPI>
@@ -522,23 +548,20 @@ extern "C" BASED_API int based_decode_linear(const void* x, int64_t x_row_stride
   a.conv_state_f32 = conv_state_dtype == BASED_F32;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)((K + 511) / 512);
-  const int tile = chunks > 4 ? 4 : 8;  // activation rows per launch
-  for (int64_t m0 = 0; m0 < M; m0 += tile) {
-    a.M = (int)(M - m0 < tile ? M - m0 : tile);
-    a.m0 = (int)m0;
-    a.x = static_cast<const __bf16*>(x) + (x_row_index ? 0 : m0 * x_row_stride);
-    a.x_index = x_row_index ? x_row_index + m0 : nullptr;
-    a.y = static_cast<__bf16*>(y) + m0 * y_row_stride;
-    a.res_in = residual_in ? residual_in + m0 * ri_row_stride : nullptr;
-    a.res_out = residual_out ? residual_out + m0 * ro_row_stride : nullptr;
-    if (chunks <= 1)
-      launch_decode_linear<1>(a, prologue, epilogue, s);
-    else if (chunks <= 2)
-      launch_decode_linear<2>(a, prologue, epilogue, s);
-    else if (chunks <= 4)
-      launch_decode_linear<4>(a, prologue, epilogue, s);
-    else
-      launch_decode_linear<8>(a, prologue, epilogue, s);
-  }
+  a.M = (int)M;
+  a.m0 = 0;
+  a.x = static_cast<const __bf16*>(x);
+  a.x_index = x_row_index;
+  a.y = static_cast<__bf16*>(y);
+  a.res_in = residual_in;
+  a.res_out = residual_out;
+  if (chunks <= 1)
+    launch_decode_linear<1>(a, prologue, epilogue, s);
+  else if (chunks <= 2)
+    launch_decode_linear<2>(a, prologue, epilogue, s);
+  else if (chunks <= 4)
+    launch_decode_linear<4>(a, prologue, epilogue, s);
+  else
+    launch_decode_linear<8>(a, prologue, epilogue, s);
   return check_launch("decode_linear");
 }
