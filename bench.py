@@ -43,6 +43,7 @@ MEASURED_TRAFFIC_BYTES = {
     "lin_step_kernel": 294355149,   # B=128, H=16, dv=64, rotating state sets: fetch 147,032,269 + write 147,322,880
     "lin_prefill_mfma_kernel": {96: 2208919860},  # B=96, L=4096, dv=64, states written; keyed by batch
     "swa_prefill_kernel": 283253146,   # B=8, H=16, L=4096: fetch 216,144,282 + write 67,108,864
+    "decode_linear_kernel_lm_head": 105068544,   # M=4, 50280 x 1024 + closing norm: fetch 104,456,397 + write 612,147
 }
 
 
@@ -443,7 +444,8 @@ def _bench_projections(torch, F, ops, M):
     out["norm + lm_head 50280x1024"] = {
         "us": round(mine, 2), "torch_linear_us": round(ref, 2), "weight_MB": round(V * D * 2 / 1e6, 1), "weight_sets": n_sets,
         "roofline": {"kernel": "decode_linear_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["decode_linear_kernel_lm_head"] if M == 4 else None,
                      "algorithmic_bytes_per_launch": nbytes}}
     return out
 
