@@ -38,7 +38,7 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
     long y_sb, long y_sh, float eps) {
   __shared__ float s_x[2][kFeat];                            // [0] = k, [1] = q
   __shared__ __align__(16) float s_tab[2][4][kTabLen];       // [0] = phi(k), [1] = phi(q)
-  __shared__ float s_v[256];
+  __shared__ float s_v[1024];  // one entry per thread (the first dv are read)
   __shared__ float s_den;
 
   const int tid = threadIdx.x;
@@ -52,41 +52,69 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
   // HBM round trip runs under the set-up below (feature tables, two barriers).  The state is
   // touched exactly once per step and the whole batch's state is far larger than any cache:
   // non-temporal loads and stores keep it from displacing anything.
+  // The small operands go first and nothing is loaded under a condition (a thread with nothing
+  // to fetch re-reads a valid element): the wait for q, k and v can then leave the eighteen state
+  // requests behind it in flight, and the feature tables are built under the HBM round trip
+  // instead of after it.
+  const int xi = tid & (2 * kFeat - 1);
+  const T* x_src = (xi >> 4) ? (q + b * q_sb + h * q_sh) : (k + b * k_sb + h * k_sh);
+  const float x_val = to_f32(x_src[xi & 15]);
+  const float v_val = to_f32(v[b * v_sb + h * v_sh + (tid < dv ? tid : 0)]);
+  // normaliser operands of wavefront 0 (every wavefront fetches them: no branch)
+  constexpr int kNormIters = (kExp + kWave - 1) / kWave;  // 5
+  float* ks = k_state + bh * kExp;
+  float ks_old[kNormIters];
+#pragma unroll
+  for (int i = 0; i < kNormIters; ++i) {
+    const int f = lane + kWave * i;
+    ks_old[i] = ks[f < kExp ? f : 0];
+  }
+
   f32x4* base = reinterpret_cast<f32x4*>(kv_state + (bh * dv + (long)kRowsPerWave * wave) * kExp);
   f32x4 d[kIters];
 #pragma unroll
   for (int t = 0; t < kIters; ++t) {
     const int j = t * kWave + lane;
-    if (t < kIters - 1 || j < kVec4PerWave) d[t] = __builtin_nontemporal_load(base + j);
+    d[t] = __builtin_nontemporal_load(base + (j < kVec4PerWave ? j : kVec4PerWave - 1));
   }
 
-  if (tid < 2 * kFeat) {
-    const int which = tid >> 4, i = tid & 15;
-    const T* src = which ? (q + b * q_sb + h * q_sh) : (k + b * k_sb + h * k_sh);
-    s_x[which][i] = to_f32(src[i]);
-  }
-  if (tid < dv) s_v[tid] = to_f32(v[b * v_sb + h * v_sh + tid]);
+  // (stored by every thread, duplicates included: a load whose only use sits under a condition is
+  // moved into that branch by the compiler, behind the state requests)
+  s_x[xi >> 4][xi & 15] = x_val;
+  s_v[tid] = v_val;
   __syncthreads();
 
-  for (int idx = tid; idx < 2 * 4 * kTabLen; idx += blockDim.x) {
-    const int which = idx / (4 * kTabLen);
-    const int rem = idx - which * (4 * kTabLen);
-    const int m = rem / kTabLen, i = rem - m * kTabLen;
-    const int e = i + m;
-    float val = 0.0f;
-    if (e < kExp + 3) val = phi_elem(s_x[which], e >= kExp ? e - kExp : e);
-    s_tab[which][m][i] = val;
+  // Entry i of copy m holds feature e = i + m (features 273..275 wrap to 0..2, beyond that
+  // zeros): a thread evaluates phi(k) and phi(q) once per e and files them in the four copies.
+  for (int e = tid; e < kTabLen + 3; e += blockDim.x) {
+    float val_k = 0.0f, val_q = 0.0f;
+    if (e < kExp + 3) {
+      const int f = e >= kExp ? e - kExp : e;
+      val_k = phi_elem(s_x[0], f);
+      val_q = phi_elem(s_x[1], f);
+    }
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int i = e - m;
+      if (i >= 0 && i < kTabLen) {
+        s_tab[0][m][i] = val_k;
+        s_tab[1][m][i] = val_q;
+      }
+    }
   }
   __syncthreads();
 
   // Normaliser: k_state += phi(k); den = phi(q) . k_state.  One wavefront owns it.
   if (wave == 0) {
-    float* ks = k_state + bh * kExp;
     float part = 0.0f;
-    for (int f = lane; f < kExp; f += kWave) {
-      const float nk = ks[f] + s_tab[0][0][f];
-      ks[f] = nk;
-      part += s_tab[1][0][f] * nk;
+#pragma unroll
+    for (int i = 0; i < kNormIters; ++i) {
+      const int f = lane + kWave * i;
+      if (f < kExp) {
+        const float nk = ks_old[i] + s_tab[0][0][f];
+        ks[f] = nk;
+        part += s_tab[1][0][f] * nk;
+      }
     }
     part = wave_sum(part);
     if (lane == 0) s_den = part;

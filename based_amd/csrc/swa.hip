@@ -468,11 +468,17 @@ __global__ __launch_bounds__(256) void swa_step_kernel(
     sn = rope_sin[(long)pos * (kHeadDim / 2) + (lane & 31)];
   }
   constexpr int kPerWave = kCached / 4;  // keys of this wavefront: j = wave, wave + 4, ...
+  // No load sits under a condition: a load in a branch is waited for at the end of the branch,
+  // and these sixteen would be sixteen memory round trips one after the other.  Rows past the
+  // window are fetched from row `lo` (inside the cache) and masked to zero as bits.
   float vv[kPerWave];
+  const uint16_t* vc16 = reinterpret_cast<const uint16_t*>(vc);
 #pragma unroll
   for (int u = 0; u < kPerWave; ++u) {
     const int j = 4 * u + wave;
-    vv[u] = j < ncached ? to_f32(vc[(long)(lo + j) * c_st + lane]) : 0.f;
+    const bool in_window = j < ncached;
+    const uint32_t raw = vc16[(long)(lo + (in_window ? j : 0)) * c_st + lane];
+    vv[u] = bf16_bits_to_f32(raw & (in_window ? 0xffffu : 0u));
   }
   float kn = to_f32(k_new[b * kn_sb + h * kn_sh + lane]);
   const float vn = to_f32(v_new[b * vn_sb + h * vn_sh + lane]);
