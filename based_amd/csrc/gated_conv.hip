@@ -57,12 +57,30 @@ __global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
   const T* u2 = u1 + D;
   T* yo = y + b * y_sb + c0;
 
+  // No load below sits under a condition, and no loaded value goes through a select: a load in
+  // a branch is waited for at the end of the branch, one memory round trip after the other.
+  // Rows that do not exist are fetched from a valid row and cleared (as bits) or never used.
+  typedef __attribute__((ext_vector_type(4))) uint32_t bits_t;
+  auto keep_if = [](vec_t x, bool keep) -> vec_t {
+    const uint32_t m = keep ? 0xffffffffu : 0u;
+    return __builtin_bit_cast(vec_t, __builtin_bit_cast(bits_t, x) & bits_t{m, m, m, m});
+  };
+
+  // filter taps: N * K consecutive elements; bias: N (an absent bias reads the taps and is cleared)
   float w[N][K], bs[N];
+  {
+    const vec_t* wp = reinterpret_cast<const vec_t*>(weight + (long)c0 * K);
+    vec_t wv[K];
 #pragma unroll
-  for (int c = 0; c < N; ++c) {
+    for (int j = 0; j < K; ++j) wv[j] = wp[j];
+    const vec_t bv = keep_if(*reinterpret_cast<const vec_t*>(bias != nullptr ? bias + c0 : weight + (long)c0 * K),
+                             bias != nullptr);
 #pragma unroll
-    for (int j = 0; j < K; ++j) w[c][j] = to_f32(weight[(long)(c0 + c) * K + j]);
-    bs[c] = bias != nullptr ? to_f32(bias[c0 + c]) : 0.0f;
+    for (int c = 0; c < N; ++c) {
+#pragma unroll
+      for (int j = 0; j < K; ++j) w[c][j] = to_f32(wv[(c * K + j) / N][(c * K + j) % N]);
+      bs[c] = to_f32(bv[c]);
+    }
   }
 
   // the K-1 inputs before the block (zeros before the sequence start)
@@ -70,25 +88,22 @@ __global__ __launch_bounds__(256) void gated_conv_prefill_kernel(
 #pragma unroll
   for (int j = 0; j < K - 1; ++j) {
     const int l = l0 - (K - 1) + j;
-    vec_t x = {};
-    if (l >= 0) x = *reinterpret_cast<const vec_t*>(u1 + (long)l * u_sl);
+    const vec_t x = keep_if(*reinterpret_cast<const vec_t*>(u1 + (long)(l >= 0 ? l : 0) * u_sl), l >= 0);
 #pragma unroll
     for (int c = 0; c < N; ++c) win[j][c] = to_f32(x[c]);
   }
 
   const int ntok = L - l0 < kConvTokens ? L - l0 : kConvTokens;
+  const T* gate_src = gated ? u2 : u1;  // without a gate the second operand is fetched and ignored
   constexpr int kBatch = 4;  // tokens whose loads are in flight together
 #pragma unroll
   for (int t0 = 0; t0 < kConvTokens; t0 += kBatch) {
     vec_t x1[kBatch], x2[kBatch];
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
-      x1[i] = vec_t{};
-      x2[i] = vec_t{};
-      if (t0 + i < ntok) {
-        x1[i] = *reinterpret_cast<const vec_t*>(u1 + (long)(l0 + t0 + i) * u_sl);
-        if (gated) x2[i] = *reinterpret_cast<const vec_t*>(u2 + (long)(l0 + t0 + i) * u_sl);
-      }
+      const long row = l0 + (t0 + i < ntok ? t0 + i : ntok - 1);  // past the end: the last token again, unused
+      x1[i] = *reinterpret_cast<const vec_t*>(u1 + row * u_sl);
+      x2[i] = *reinterpret_cast<const vec_t*>(gate_src + row * u_sl);
     }
 #pragma unroll
     for (int i = 0; i < kBatch; ++i) {
@@ -266,7 +281,8 @@ static int conv_prefill_impl(const char* who, int gated, const void* u, const vo
   BASED_REQUIRE(D % n == 0, BASED_ERR_SHAPE, "%s: channel count must be a multiple of %d", who, n);
   BASED_REQUIRE(u_sb % n == 0 && u_sl % n == 0 && y_sb % n == 0 && y_sl % n == 0, BASED_ERR_ALIGN,
                 "%s: strides must be multiples of %d elements", who, n);
-  BASED_REQUIRE(aligned16(u) && aligned16(y), BASED_ERR_ALIGN, "%s: tensors must be 16-byte aligned", who);
+  BASED_REQUIRE(aligned16(u) && aligned16(y) && aligned16(weight) && aligned16(bias), BASED_ERR_ALIGN,
+                "%s: tensors must be 16-byte aligned", who);
   BASED_REQUIRE(B < 65536 && (L + kConvTokens - 1) / kConvTokens < 65536, BASED_ERR_SHAPE,
                 "%s: grid too large", who);
   if (B == 0 || L == 0) return BASED_OK;
