@@ -10,6 +10,10 @@
 
 namespace based {
 
+// (not const: constant data lives in another address space, and a pointer that may be in either
+// makes the load a flat one, which is waited for on the spot)
+__device__ __attribute__((aligned(32))) uint32_t kNormZeroPage[8] = {};
+
 constexpr int kNormMaxChunks = 8;  // a lane holds up to 8 chunks of 8 elements: rows up to 4096 wide
 
 template <typename T> __device__ __forceinline__ void load8(const T* p, float (&v)[8]);
@@ -50,19 +54,26 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(
   if (res_in != nullptr) res_in += row * ri_sr;
   if (res_out != nullptr) res_out += row * ro_sr;
 
-  float v[NCH][8];
+  // Every load is issued unconditionally and up front (a load under a condition is waited for at
+  // the end of its branch, one round trip after the other): chunks past the row end re-read the
+  // start of the row (and are not used), an absent residual reads a page of zeros.
+  float v[NCH][8], w[NCH][8];
   float ss = 0.f;
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int e0 = (c * 64 + lane) * 8;
-    if (e0 < D) {
-      load8<TX>(x + e0, v[c]);
-      if (res_in != nullptr) {
-        float r[8];
-        load8<TR>(res_in + e0, r);
+    const int ec = e0 < D ? e0 : 0;
+    load8<TX>(x + ec, v[c]);
+    load8<TX>(weight + ec, w[c]);
+    float r[8];
+    load8<TR>(res_in != nullptr ? res_in + ec : reinterpret_cast<const TR*>(kNormZeroPage), r);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[c][i] += r[i];
-      }
+    for (int i = 0; i < 8; ++i) v[c][i] += r[i];
+  }
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int e0 = (c * 64 + lane) * 8;
+    if (e0 < D) {
       if (res_out != nullptr) store8<TR>(res_out + e0, v[c]);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -77,10 +88,9 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(
   for (int c = 0; c < NCH; ++c) {
     const int e0 = (c * 64 + lane) * 8;
     if (e0 < D) {
-      float w[8], o[8];
-      load8<TX>(weight + e0, w);
+      float o[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) o[i] = v[c][i] * rstd * w[i];
+      for (int i = 0; i < 8; ++i) o[i] = v[c][i] * rstd * w[c][i];
       store8<TX>(y + e0, o);
     }
   }
