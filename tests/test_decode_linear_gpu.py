@@ -49,6 +49,24 @@ def test_lm_head_shape_and_strided_operands(dev):
     assert torch.equal(out[:, :N], y) and bool((out[:, N:] == 7).all())
 
 
+@pytest.mark.parametrize("M,N,K,norm", [(12, 20000, 1024, True), (3, 9000, 2048, False), (9, 40000, 64, True),
+                                        (32, 50280, 1024, True)])
+def test_more_row_groups_than_wavefronts(dev, M, N, K, norm):
+    """Launches whose wavefronts walk several row groups (two register sets taking turns), also
+    with more activation rows than one tile holds."""
+    from based_amd import ops
+
+    print(f"decode_linear rounds M={M} N={N} K={K} norm={norm}", flush=True)
+    x, w, b = _rand((M, K), dev, 50), _rand((N, K), dev, 51, 0.05), _rand((N,), dev, 52)
+    if norm:
+        nw, res = _rand((K,), dev, 53), _rand((M, K), dev, 54).float()
+        normed, _ = ops.add_rms_norm(x, res, nw, 1e-5, residual_in_fp32=True)
+        y = ops.decode_linear(x, w, b, prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=res, norm_weight=nw, eps=1e-5)
+        _check_product(y, normed, w, b)
+    else:
+        _check_product(ops.decode_linear(x, w, b), x, w, b)
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (4, 1536, 1024), (8, 4096, 1024), (3, 100, 2048), (4, 64, 4096),
                                    (7, 64, 4096), (12, 256, 256)])
 @pytest.mark.parametrize("with_residual", [False, True])
