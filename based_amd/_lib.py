@@ -27,6 +27,11 @@ SIGNATURES = {
         C.c_int,
         [_P, _P, _P, _P, _P, _P] + [_I64] * 3 + [_I64] * 8 + [C.c_float, C.c_int, _P],
     ),
+    "based_linear_attn_step_deferred": (
+        C.c_int,
+        [_P, _P, _P, _P, _P, _P, _P, _P, _P] + [_I64] * 3 + [_I64] * 8 + [C.c_float, C.c_int, C.c_int, _P],
+    ),
+    "based_linear_attn_flush_deferred": (C.c_int, [_P, _P, _P, _P] + [_I64] * 3 + [_P]),
     "based_linear_attn_prefill": (
         C.c_int,
         [_P, _P, _P, _P, _P, _P] + [_I64] * 4 + [_I64] * 12 + [C.c_float, C.c_int, _P],

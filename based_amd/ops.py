@@ -112,6 +112,97 @@ def linear_attn_step(q, k, v, kv_state, k_state, eps: float = 1e-12, out: Option
     return y
 
 
+DEFERRED_MAX_STEPS = 8  # BASED_DEFERRED_MAX_STEPS
+
+
+def deferred_step_buffers(batch: int, heads: int, dv: int, device) -> tuple:
+    """The ring of `linear_attn_step_deferred` for (batch, heads) states: keys (B, H, 8, 16) and
+    values (B, H, 8, dv) in fp32, and the per-(batch, head) fill count (B, H) int32, all zero."""
+    return (torch.zeros(batch, heads, DEFERRED_MAX_STEPS, FEATURE_DIM, dtype=torch.float32, device=device),
+            torch.zeros(batch, heads, DEFERRED_MAX_STEPS, dv, dtype=torch.float32, device=device),
+            torch.zeros(batch, heads, dtype=torch.int32, device=device))
+
+
+def _check_deferred(kv_state, pending):
+    pend_k, pend_v, pend_n = pending
+    B, H, _, dv, _ = kv_state.shape
+    _require_cuda(kv_state, pend_k, pend_v, pend_n)
+    if (tuple(pend_k.shape) != (B, H, DEFERRED_MAX_STEPS, FEATURE_DIM) or tuple(pend_v.shape) != (B, H, DEFERRED_MAX_STEPS, dv)
+            or tuple(pend_n.shape) != (B, H)):
+        raise ValueError(f"bad ring shapes {tuple(pend_k.shape)} {tuple(pend_v.shape)} {tuple(pend_n.shape)} for a "
+                         f"state {tuple(kv_state.shape)}")
+    if pend_k.dtype != torch.float32 or pend_v.dtype != torch.float32 or pend_n.dtype != torch.int32:
+        raise ValueError("the ring is float32 keys and values and an int32 count")
+    if not (pend_k.is_contiguous() and pend_v.is_contiguous() and pend_n.is_contiguous()):
+        raise ValueError("the ring must be contiguous")
+
+
+def linear_attn_step_deferred(q, k, v, kv_state, k_state, pending, period: int, eps: float = 1e-12,
+                              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`linear_attn_step` with the write-back of kv_state deferred: the step reads kv_state, updates
+    k_state and parks the token's raw k and v in `pending` (from `deferred_step_buffers`); every
+    `period`-th step (1..8) applies the parked tokens and its own to kv_state in one pass.  The
+    output is the one of `linear_attn_step` up to fp32 summation order; kv_state is current only
+    after such a step or after `linear_attn_flush_deferred`.  Leading rows of larger states and
+    rings may be passed (views of the first B rows)."""
+    key = ("lin_step_deferred", q.shape, q.stride(), k.shape, k.stride(), v.shape, v.stride(), kv_state.shape,
+           kv_state.stride(), k_state.shape, k_state.stride(), q.dtype, k.dtype, v.dtype, kv_state.dtype, k_state.dtype,
+           q.device, k.device, v.device, kv_state.device, k_state.device,
+           tuple((t.shape, t.stride(), t.dtype, t.device) for t in pending), int(period))
+    if key not in _CHECKED:
+        _require_cuda(q, k, v, kv_state, k_state)
+        B, H, l, d = q.shape
+        assert l == 1, f"q.shape is {tuple(q.shape)} but should be ({B}, {H}, 1, {d})"
+        dv = v.shape[-1]
+        if d != FEATURE_DIM or k.shape != q.shape or v.shape[:3] != q.shape[:3]:
+            raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+        if kv_state.dtype != torch.float32 or k_state.dtype != torch.float32:
+            raise ValueError("decode states must be float32")
+        if tuple(kv_state.shape) != (B, H, 1, dv, EXPANDED_DIM) or tuple(k_state.shape) != (B, H, 1, 1, EXPANDED_DIM):
+            raise ValueError(f"bad state shapes {tuple(kv_state.shape)} {tuple(k_state.shape)}")
+        if not (kv_state.is_contiguous() and k_state.is_contiguous()):
+            raise ValueError("decode states must be contiguous")
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ValueError("q, k, v must share a dtype")
+        for t in (q, k, v):
+            if t.stride(-1) != 1:
+                raise ValueError("innermost dimension must be contiguous")
+        if not 1 <= int(period) <= DEFERRED_MAX_STEPS:
+            raise ValueError(f"period must be in [1, {DEFERRED_MAX_STEPS}], got {period}")
+        _check_deferred(kv_state, pending)
+        _dtype_code(q)
+        _CHECKED[key] = True
+    B, H, _, _ = q.shape
+    dv = v.shape[-1]
+    if out is None:
+        y = torch.empty(B, H, 1, dv, dtype=q.dtype, device=q.device)
+    else:
+        y = out
+        if tuple(y.shape) != (B, H, 1, dv) or y.dtype != q.dtype or y.device != q.device or y.stride(-1) != 1:
+            raise ValueError(f"out must be a ({B}, {H}, 1, {dv}) {q.dtype} tensor on {q.device}")
+    pend_k, pend_v, pend_n = pending
+    with _on_device(q.device):
+        _lib.check(_lib.lib().based_linear_attn_step_deferred(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), kv_state.data_ptr(), k_state.data_ptr(), pend_k.data_ptr(),
+            pend_v.data_ptr(), pend_n.data_ptr(), y.data_ptr(), B, H, dv,
+            q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1), y.stride(0), y.stride(1),
+            float(eps), int(period), _dtype_code(q), _stream_ptr(q)))
+    return y
+
+
+def linear_attn_flush_deferred(kv_state, pending) -> None:
+    """Applies the tokens parked by `linear_attn_step_deferred` to kv_state (B,H,1,dv,273) and
+    empties the ring."""
+    if kv_state.dtype != torch.float32 or kv_state.dim() != 5 or not kv_state.is_contiguous():
+        raise ValueError("kv_state must be a contiguous float32 (B, H, 1, dv, 273) tensor")
+    _check_deferred(kv_state, pending)
+    B, H, _, dv, _ = kv_state.shape
+    pend_k, pend_v, pend_n = pending
+    with _on_device(kv_state.device):
+        _lib.check(_lib.lib().based_linear_attn_flush_deferred(kv_state.data_ptr(), pend_k.data_ptr(), pend_v.data_ptr(),
+                                                               pend_n.data_ptr(), B, H, dv, _stream_ptr(kv_state)))
+
+
 def _rope_tables(rope, device, need_rows):
     """(cos, sin) fp32 (n_pos, 32) contiguous device tables -> (cos_ptr, sin_ptr, n_pos) or Nones."""
     if rope is None:

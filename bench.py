@@ -135,6 +135,53 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
     }
 
 
+def bench_decode_deferred(torch, ops, period=8, B=128, H=16, dv=64, n_sets=4, cycles=6):
+    """The decode step with the write-back of the state deferred (`ops.linear_attn_step_deferred`,
+    not the reference's semantics for kv_state between steps, same outputs): `cycles` x `period`
+    steps on each of `n_sets` state sets visited in turn (cold, as bench_decode), so that the
+    average contains the reading steps and the applying steps in their proportion.  Bytes: the
+    variant's own count, i.e. the state read on every step and written on every `period`-th."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(0)
+    states = [(torch.randn(B, H, 1, dv, D_EXP, generator=g).to(dev), (torch.rand(B, H, 1, 1, D_EXP, generator=g) + 1).to(dev))
+              for _ in range(n_sets)]
+    rings = [ops.deferred_step_buffers(B, H, dv, dev) for _ in range(n_sets)]
+    q = torch.randn(B, H, 1, 16, generator=g).bfloat16().to(dev)
+    k = torch.randn(B, H, 1, 16, generator=g).bfloat16().to(dev)
+    v = torch.randn(B, H, 1, dv, generator=g).bfloat16().to(dev)
+    y = torch.empty(B, H, 1, dv, dtype=torch.bfloat16, device=dev)
+    n_steps = cycles * period
+
+    def run():
+        for _ in range(n_steps):
+            for (kv_state, k_state), ring in zip(states, rings):
+                ops.linear_attn_step_deferred(q, k, v, kv_state, k_state, ring, period, out=y)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            run()
+    torch.cuda.current_stream().wait_stream(side)
+    ms, _ = _events_ms(torch, graph.replay, 10, 2)
+    ms /= n_steps * n_sets
+    assert torch.isfinite(y.float()).all() and all(bool((r[2] == 0).all()) for r in rings)
+    state_bytes = B * H * D_EXP * dv * 4
+    small = B * H * (2 * D_EXP * 4 + (2 * 16 + 2 * dv) * 2)
+    ring_bytes = B * H * (16 + dv) * 4 * (period - 1) / 2  # the ring as read by an average step
+    own_bytes = state_bytes * (1 + 1 / period) + small + ring_bytes
+    in_place_bytes = 2 * state_bytes + small
+    return {"period": period, "us_per_step": round(ms * 1e3, 2), "tok_s": round(B / (ms * 1e-3), 1),
+            "bytes_per_step": int(own_bytes), "GBps": round(own_bytes / (ms * 1e-3) / 1e9, 1),
+            "frac_of_hbm_peak": round(own_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "in_place_bytes_per_step": in_place_bytes,
+            "note": "opt-in (LinearAttention(deferred_state_steps=8)); average over reading and applying steps, "
+                    f"{n_sets} state sets in turn; the headline figure is the in-place step"}
+
+
 def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
     """Linear-attention prefill.  Launches that move less than the last-level cache holds are timed
     over several independent input sets visited in turn (cold) and on one set (warm); the figure
@@ -570,6 +617,8 @@ def main():
                     "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
                     "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5),
                     "decode_cold": d["cold"], "decode_warm": d["warm"]})
+        with torch.inference_mode():
+            out["decode_deferred"] = bench_decode_deferred(torch, ops)
     if args.only in (None, "prefill"):
         pre = [bench_prefill(torch, ops, 30, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]

@@ -69,6 +69,33 @@ BASED_API int based_linear_attn_step(const void* q, const void* k, const void* v
                            float eps, int io_dtype, void* stream);
 
 /*
+ * The same step with the write-back of the state deferred (no counterpart in the reference, whose
+ * recurrent_forward rewrites kv_state on every token, based/models/mixers/linear_attention.py:
+ * 230-252; y is the same up to fp32 summation order).  Writing the state is half of the step's
+ * memory traffic and the output does not need it: with S the state as last written and
+ * (k_j, v_j) the tokens since,
+ *   phi(q) . (S + sum_j phi(k_j) v_j^T) = phi(q) . S + sum_j (1 + s_j + s_j^2 / 2) v_j,  s_j = q . k_j / 4.
+ * A call reads kv_state, updates k_state, and keeps the raw k and v of the token in a ring per
+ * (batch, head); the call that finds period - 1 tokens there applies them and its own token to
+ * kv_state in one read-modify-write pass and empties the ring.  period = 1 is
+ * based_linear_attn_step.  Between those calls kv_state lacks the ring's tokens:
+ * based_linear_attn_flush_deferred applies them (for a reader of kv_state other than this call).
+ *
+ *   pend_k : (B, H, BASED_DEFERRED_MAX_STEPS, 16) fp32, contiguous
+ *   pend_v : (B, H, BASED_DEFERRED_MAX_STEPS, dv) fp32, contiguous
+ *   pend_n : (B, H) int32, tokens in the ring; zero it when the state is (re)initialised
+ *   period : 1 .. BASED_DEFERRED_MAX_STEPS; other arguments as based_linear_attn_step
+ */
+#define BASED_DEFERRED_MAX_STEPS 8
+BASED_API int based_linear_attn_step_deferred(
+    const void* q, const void* k, const void* v, float* kv_state, float* k_state, float* pend_k, float* pend_v,
+    int32_t* pend_n, void* y, int64_t B, int64_t H, int64_t dv, int64_t q_sb, int64_t q_sh, int64_t k_sb,
+    int64_t k_sh, int64_t v_sb, int64_t v_sh, int64_t y_sb, int64_t y_sh, float eps, int period, int io_dtype,
+    void* stream);
+BASED_API int based_linear_attn_flush_deferred(float* kv_state, const float* pend_k, const float* pend_v,
+                                               int32_t* pend_n, int64_t B, int64_t H, int64_t dv, void* stream);
+
+/*
  * Causal Taylor linear attention over a whole sequence (prefill), feature map,
  * normaliser and decode-state construction fused.
  * Replaces LinearAttention.parallel_forward up to (not including) out_proj, and the
