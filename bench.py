@@ -171,7 +171,7 @@ def bench_decode_deferred(torch, ops, period=8, B=128, H=16, dv=64, n_sets=4, cy
     assert torch.isfinite(y.float()).all() and all(bool((r[2] == 0).all()) for r in rings)
     state_bytes = B * H * D_EXP * dv * 4
     small = B * H * (2 * D_EXP * 4 + (2 * 16 + 2 * dv) * 2)
-    ring_bytes = B * H * (16 + dv) * 4 * (period - 1) / 2  # the ring as read by an average step
+    ring_bytes = B * H * (16 + dv) * 4 * (8 + 1)  # every step reads the whole ring (8 slots); most append one token
     own_bytes = state_bytes * (1 + 1 / period) + small + ring_bytes
     in_place_bytes = 2 * state_bytes + small
     return {"period": period, "us_per_step": round(ms * 1e3, 2), "tok_s": round(B / (ms * 1e-3), 1),
