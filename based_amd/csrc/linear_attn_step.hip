@@ -196,7 +196,8 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
 // (batch, head) in a small ring; every `period`-th step applies the whole ring and the current
 // token in one pass (read, `period` rank-one updates, write).  k_state is small and is updated
 // on every step.  The ring and its fill count live in device memory, per (batch, head), so that
-// a recorded graph replays correctly; all workgroups of a call are at the same count.
+// a recorded graph replays correctly (normally every workgroup of a call finds the same count, but
+// nothing depends on it: a (batch, head) is one workgroup's business from the count to the state).
 // ------------------------------------------------------------------------------------------
 constexpr int kPendMax = BASED_DEFERRED_MAX_STEPS;
 
