@@ -94,7 +94,6 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
     from based_amd import _lib
 
     lib = _lib.lib()
-    stream = torch.cuda.current_stream().cuda_stream
     args = [(qs[i].data_ptr(), ks[i].data_ptr(), vs[i].data_ptr()) for i in range(n_in)]
     st_ptrs = [(a.data_ptr(), b.data_ptr()) for a, b in states]
     it = [0]
@@ -106,13 +105,31 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
             it[0] += 1
             rc = lib.based_linear_attn_step(a[0], a[1], a[2], st[0], st[1], y.data_ptr(),
                                             B, H, dv, H * 16, 16, H * 16, 16, H * dv, dv, H * dv, dv,
-                                            1e-12, 0, stream)
+                                            1e-12, 0, torch.cuda.current_stream().cuda_stream)
             if rc:
                 _lib.check(rc)
         return step
 
-    ms_cold, wall = _events_ms(torch, make_step(n_sets), steps, warmup)
-    ms_warm, _ = _events_ms(torch, make_step(1), steps, warmup)
+    def in_graph(sets):
+        """The same `steps` launches recorded once and replayed, as the decoding loop issues them
+        (generation.py: capture_graph); one replay is timed."""
+        step = make_step(sets)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):
+                step()
+            side.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(steps):
+                    step()
+        torch.cuda.current_stream().wait_stream(side)
+        return _events_ms(torch, graph.replay, 1, 2)[0] / steps
+
+    eager_cold, wall = _events_ms(torch, make_step(n_sets), steps, warmup)
+    eager_warm, _ = _events_ms(torch, make_step(1), steps, warmup)
+    ms_cold, ms_warm = in_graph(n_sets), in_graph(1)
     bytes_per_launch = B * H * (2 * D_EXP * dv * 4 + 2 * D_EXP * 4 + (2 * 16 + 2 * dv) * 2)
     ms = max(ms_cold, ms_warm)
     gbs = bytes_per_launch / (ms * 1e-3) / 1e9
@@ -122,14 +139,17 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
         "ms": ms,
         "wall_ms": wall,
         "cold": {"ms": round(ms_cold, 5), "GBps": round(bytes_per_launch / (ms_cold * 1e-3) / 1e9, 1), "state_sets": n_sets,
-                 "working_set_MB": round(n_sets * (kv_state.numel() + k_state.numel()) * 4 / 1e6, 1)},
+                 "working_set_MB": round(n_sets * (kv_state.numel() + k_state.numel()) * 4 / 1e6, 1),
+                 "launched_one_by_one_ms": round(eager_cold, 5)},
         "warm": {"ms": round(ms_warm, 5), "GBps": round(bytes_per_launch / (ms_warm * 1e-3) / 1e9, 1), "state_sets": 1,
-                 "working_set_MB": round((kv_state.numel() + k_state.numel()) * 4 / 1e6, 1)},
+                 "working_set_MB": round((kv_state.numel() + k_state.numel()) * 4 / 1e6, 1),
+                 "launched_one_by_one_ms": round(eager_warm, 5)},
         "roofline": {"kernel": "lin_step_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else None,
                      "algorithmic_bytes_per_launch": bytes_per_launch,
-                     "timed": "the slower of cold (rotating state sets) and warm (one set)"},
+                     "timed": "the slower of cold (rotating state sets) and warm (one set); the steps are recorded in "
+                              "one graph and one replay is timed (launched one by one: see decode_cold / decode_warm)"},
         "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, "
                     f"bf16 q/k/v, {n_sets} independent state sets visited in turn",
     }
