@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the Based sequence-mixer hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|stack|copy|machine]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only decode|prefill|swa|conv|stack|projections|copy|machine]
 
 Headline workload (`value`): the recurrent decode step of Taylor linear attention at
 B=128, H=16, dv=64 — fp32 kv_state (128,16,1,64,273) + k_state, initialised from a seeded
@@ -16,7 +16,11 @@ L=4096 (tokens/s and fraction of bf16 MFMA peak) and the sliding-window attentio
 decode of the B=8, H=16, L=4096 configuration.
 
 `roofline.achieved` = algorithmic bytes (or FLOPs) per launch / average launch duration,
-timed with HIP events on the stream the kernels are launched on (torch's current stream).
+timed with HIP events on the stream the kernels are launched on.  The K decode steps are
+recorded once in a graph, as the decoding loop issues them, and one replay of it is the timed
+region (the kernel's own duration: what the kernel trace shows); the same K launches issued one
+by one from the host carry the gap between two launches as well and are reported beside it
+(`decode_cold.launched_one_by_one_ms`).
 `cpu_baseline` = the CPU oracle (a PyTorch restatement of the reference arithmetic) timed on
 this host's cores on a bounded sample of the same workload.
 """
