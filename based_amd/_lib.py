@@ -69,9 +69,6 @@ SIGNATURES = {
         C.c_int,
         [_P] * 6 + [_P, _I64] + [_I64] * 4 + [_I64] * 8 + [_I64] * 3 + [C.c_int, C.c_float, C.c_int, _P],
     ),
-    "based_probe_stream_qkv": (C.c_int, [_P, _P, _I64, _I64, _I64, C.c_int, _P]),
-    "based_probe_rmw": (C.c_int, [_P, _I64, _P]),
-    "based_probe_copy": (C.c_int, [_P, _P, _I64, _P]),
     "based_short_conv_prefill": (
         C.c_int,
         [_P, _P, _P, _P, _P] + [_I64] * 3 + [C.c_int] + [_I64] * 4 + [C.c_int, C.c_int, _P],

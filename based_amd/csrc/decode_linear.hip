@@ -472,6 +472,13 @@ template <int C> void launch_decode_linear(const DecodeLinearArgs& a, int prolog
   }
 }
 
+// whether the byte ranges [a, a + na) and [b, b + nb) intersect (an absent tensor intersects nothing)
+static bool ranges_overlap(const void* a, int64_t na, const void* b, int64_t nb) {
+  if (a == nullptr || b == nullptr || na <= 0 || nb <= 0) return false;
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + (uintptr_t)nb && b0 < a0 + (uintptr_t)na;
+}
+
 }  // namespace based
 
 extern "C" BASED_API int based_decode_linear(const void* x, int64_t x_row_stride, const int64_t* x_row_index,
@@ -500,8 +507,6 @@ extern "C" BASED_API int based_decode_linear(const void* x, int64_t x_row_stride
   uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight);
   if (prologue == kProNorm) {
     BASED_REQUIRE(norm_weight != nullptr, BASED_ERR_ARG, "decode_linear: the norm prologue needs its weight");
-    BASED_REQUIRE(residual_out == nullptr || residual_out != residual_in, BASED_ERR_ARG,
-                  "decode_linear: residual_out must not be residual_in (every workgroup re-reads the input)");
     BASED_REQUIRE(ri_row_stride % 4 == 0 && ro_row_stride % 4 == 0, BASED_ERR_ALIGN,
                   "decode_linear: residual row strides must be multiples of 4 elements");
     bits |= reinterpret_cast<uintptr_t>(residual_in) | reinterpret_cast<uintptr_t>(residual_out) |
@@ -529,6 +534,19 @@ extern "C" BASED_API int based_decode_linear(const void* x, int64_t x_row_stride
                 "decode_linear: a row index needs the number of rows it may address");
   BASED_REQUIRE((bits & 15) == 0, BASED_ERR_ALIGN, "decode_linear: tensors must be 16-byte aligned");
   if (M == 0) return BASED_OK;
+  {
+    // Every workgroup re-reads x and residual_in while workgroup 0 writes residual_out and the tails
+    // write y: an output that overlaps an input, even partly (a view shifted by some rows), would be
+    // a race between workgroups.  Compared as byte ranges.
+    const int64_t x_rows = x_row_index ? x_index_rows : M;
+    const int64_t x_bytes = ((x_rows - 1) * x_row_stride + (prologue == kProSwiglu ? 2 * K : K)) * 2;
+    const int64_t ri_bytes = ((M - 1) * ri_row_stride + K) * 4, ro_bytes = ((M - 1) * ro_row_stride + K) * 4;
+    const int64_t y_bytes = ((M - 1) * y_row_stride + (epilogue == kEpiNone ? N : N / 2)) * 2;
+    BASED_REQUIRE(!ranges_overlap(residual_out, ro_bytes, residual_in, ri_bytes) &&
+                      !ranges_overlap(residual_out, ro_bytes, x, x_bytes) && !ranges_overlap(y, y_bytes, x, x_bytes) &&
+                      !ranges_overlap(y, y_bytes, residual_in, ri_bytes) && !ranges_overlap(y, y_bytes, residual_out, ro_bytes),
+                  BASED_ERR_ARG, "decode_linear: an output (y, residual_out) overlaps an input or the other output");
+  }
 
   DecodeLinearArgs a;
   a.x_sr = x_row_stride;

@@ -256,6 +256,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
   const int grp = lane >> 4;
   const long bh = chain_of_block();
   const int eb = blockIdx.y;  // 64-channel block of the value dimension
+  const int live_ch = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // channels of this block that exist (a multiple of 16)
   const int b = (int)(bh / H), h = (int)(bh % H);
   y += b * y_sb + h * y_sh + 64 * eb;
   const int seg = blockIdx.z;
@@ -439,9 +440,11 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       {
         const int tau = 16 * nt + col;
         if (tau < ntok) {
+          // (in the last block of a head dim that is no multiple of 64 the channels past dv were
+          // computed from stand-in data and are dropped here)
           __bf16* dst = y + (long)(t0 + tau) * y_sl + out_ch;
-          *reinterpret_cast<u32x4*>(dst) = u32x4{P[0][0], P[0][1], P[2][0], P[2][1]};
-          *reinterpret_cast<u32x4*>(dst + 16) = u32x4{P[1][0], P[1][1], P[3][0], P[3][1]};
+          if (out_ch + 8 <= live_ch) *reinterpret_cast<u32x4*>(dst) = u32x4{P[0][0], P[0][1], P[2][0], P[2][1]};
+          if (out_ch + 24 <= live_ch) *reinterpret_cast<u32x4*>(dst + 16) = u32x4{P[1][0], P[1][1], P[3][0], P[3][1]};
         }
       }
     }
@@ -453,7 +456,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
     if (kv_state != nullptr && last_seg) {
       const float* blk = reinterpret_cast<const float*>(lds + kOffImg);
 #pragma unroll 1
-      for (int et = 0; et < kCTiles; ++et) {
+      for (int et = 0; 16 * et < live_ch; ++et) {
         __syncthreads();
         __syncthreads();
         f32x4* dst = reinterpret_cast<f32x4*>(kv_state + (bh * dv + 64 * eb + 16 * et) * kExp);
@@ -475,6 +478,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   const int grp = lane >> 4;
   const long bh = chain_of_block();
   const int eb = blockIdx.y;  // 64-channel block of the value dimension
+  const int live_ch = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // channels of this block that exist (a multiple of 16)
   const int b = (int)(bh / H), h = (int)(bh % H);
   q += b * q_sb + h * q_sh;
   k += b * k_sb + h * k_sh;
@@ -558,7 +562,11 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
         dst = slot + (id < 2 ? 0 : kDataK) + 1024 * (id & 1);
       } else {
         row = 8 * (id - 4) + (lane >> 3);
-        src = v + (long)(tc + row) * v_sl + 8 * ((lane & 7) ^ (2 * ((lane >> 3) & 3)));
+        // a piece past the head dim (last block of a dv that is no multiple of 64) is fetched from
+        // piece 0 instead: channels are independent, so what such channels compute touches no
+        // other, and they are never stored
+        const int piece = (lane & 7) ^ (2 * ((lane >> 3) & 3));
+        src = v + (long)(tc + row) * v_sl + (8 * piece < live_ch ? 8 * piece : 0);
         dst = slot + kDataV + 1024 * (id - 4);
       }
       if (ntok == kChunk || row < ntok) {
@@ -762,6 +770,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
     static_assert(16 * kExp * 4 <= kImgBytes, "expansion block must fit in a state image buffer");
     static_for<kCTiles>([&](auto ET) {
       constexpr int et = decltype(ET)::value;
+      if (16 * et >= live_ch) return;  // uniform over the workgroup (the readers count the same rounds)
       __syncthreads();  // the buffer is free (main loop done / previous block copied out)
       float* row = blk + col * kExp;
       static_for<kOwn>([&](auto II) {
@@ -969,6 +978,11 @@ __global__ __launch_bounds__(256) void lin_prefill_f32_kernel(
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
+// Head dims the MFMA kernel serves: whole 16-channel tiles.  A block of 64 channels per workgroup;
+// the last block of a head dim that is no multiple of 64 (112 = 64 + 48, the released 1B / 1.3B
+// models) runs with its missing tiles fed stand-in data and dropped at the stores.
+static bool prefill_mfma_takes(int64_t dv) { return dv >= 16 && dv <= 1024 && dv % 16 == 0; }
+
 }  // namespace based
 
 extern "C" BASED_API int based_linear_attn_prefill(
@@ -986,14 +1000,14 @@ extern "C" BASED_API int based_linear_attn_prefill(
   BASED_REQUIRE(B * H < (1ll << 31) && L < (1ll << 31), BASED_ERR_SHAPE, "linear_attn_prefill: sizes too large");
   if (B == 0) return BASED_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (io_dtype == BASED_BF16 && (dv == 64 || dv == 128)) {
+  if (io_dtype == BASED_BF16 && prefill_mfma_takes(dv)) {
     const int64_t strides[] = {q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl};
     for (int64_t st : strides)
       BASED_REQUIRE(st % 8 == 0, BASED_ERR_ALIGN,
                     "linear_attn_prefill: bf16 strides must be multiples of 8 elements (16 bytes)");
     BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
                   "linear_attn_prefill: tensors must be 16-byte aligned");
-    dim3 grid((unsigned)(B * H), (unsigned)(dv / 64)), block(kThreads);
+    dim3 grid((unsigned)(B * H), (unsigned)((dv + 63) / 64)), block(kThreads);
     hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFull>, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
                        q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, (float*)nullptr, 0, 1);
@@ -1026,8 +1040,8 @@ extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, in
   BASED_REQUIRE(n_seg && workspace_bytes, BASED_ERR_ARG, "linear_attn_prefill_plan: null output pointer");
   *n_seg = 1;
   *workspace_bytes = 0;
-  if (io_dtype != BASED_BF16 || (dv != 64 && dv != 128) || B <= 0 || H <= 0 || L <= 0) return BASED_OK;
-  const int64_t chains = B * H * (dv / 64);
+  if (io_dtype != BASED_BF16 || !based::prefill_mfma_takes(dv) || B <= 0 || H <= 0 || L <= 0) return BASED_OK;
+  const int64_t chains = B * H * ((dv + 63) / 64);
   const int64_t chunks = (L + kChunk - 1) / kChunk;
   // Measured on MI355X at L = 4096 (best segment count per batch size): 16 chains -> 16, 32 -> 8,
   // 48..128 -> 4, and from 192 chains on the single pass wins (one workgroup alone on a compute
@@ -1063,8 +1077,8 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   BASED_REQUIRE(q && k && v && y, BASED_ERR_ARG, "%s: null pointer argument", who);
   BASED_REQUIRE((kv_state == nullptr) == (k_state == nullptr), BASED_ERR_ARG,
                 "%s: kv_state and k_state must both be given or both be NULL", who);
-  BASED_REQUIRE(io_dtype == BASED_BF16 && (dv == 64 || dv == 128), BASED_ERR_SHAPE,
-                "%s: only the bf16 MFMA path (dv 64 or 128) can be split", who);
+  BASED_REQUIRE(io_dtype == BASED_BF16 && prefill_mfma_takes(dv), BASED_ERR_SHAPE,
+                "%s: only the bf16 MFMA path (head dims that are multiples of 16) can be split", who);
   BASED_REQUIRE(B > 0 && H > 0 && L > 0 && B * H < (1ll << 31) && L < (1ll << 31), BASED_ERR_ARG, "%s: bad sizes", who);
   const int64_t chunks = (L + kChunk - 1) / kChunk;
   BASED_REQUIRE(n_seg >= 2 && n_seg <= chunks && n_seg < 65536, BASED_ERR_ARG, "%s: %ld segments for %ld chunks", who,
@@ -1072,7 +1086,8 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   const int64_t seg_chunks = (chunks + n_seg - 1) / n_seg;
   BASED_REQUIRE((n_seg - 1) * seg_chunks < chunks, BASED_ERR_ARG,
                 "%s: segment count %ld leaves empty segments (use the plan)", who, (long)n_seg);
-  const int64_t chains = B * H * (dv / 64);
+  const int64_t eblocks = (dv + 63) / 64;
+  const int64_t chains = B * H * eblocks;
   const int64_t need = chains * n_seg * (int64_t)kSegStateFloats * 4;
   if (workspace_limit >= 0)
     BASED_REQUIRE(need <= workspace_limit, BASED_ERR_SHAPE,
@@ -1090,7 +1105,7 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   const int seg_tokens = (int)(seg_chunks * kChunk);
   dim3 block(kThreads);
   // pass 1: every segment but the last accumulates its own contribution to the state
-  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)(n_seg - 1)),
+  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)(B * H), (unsigned)eblocks, (unsigned)(n_seg - 1)),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
@@ -1106,7 +1121,7 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
     rc = check_launch(who);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(fold ? lin_prefill_mfma_kernel<kModeFromSum> : lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)(dv / 64), (unsigned)n_seg),
+  hipLaunchKernelGGL(fold ? lin_prefill_mfma_kernel<kModeFromSum> : lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)eblocks, (unsigned)n_seg),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
@@ -1114,10 +1129,10 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
 }
 
 // Scratch of based_linear_attn_prefill_split_static: one array per GPU, part of the code object,
-// alive until the process ends.  64 MiB hold 1310 (chain, segment) state images, more than any
-// segment count the plan entry point returns (it aims at 768 workgroup slots and never exceeds
-// 1150 images).  In host code the array's name is only a handle for hipGetSymbolAddress; the
-// device address is looked up once per device and kept in g_scratch_ptr.
+// alive until the process ends.  64 MiB hold 1560 (chain, segment) state images of 43,008 bytes,
+// more than any plan the plan entry point returns (it fills at most kPrefillSlots = 512 workgroup
+// slots, i.e. at most 512 images).  In host code the array's name is only a handle for
+// hipGetSymbolAddress; the device address is looked up once per device and kept in g_scratch_ptr.
 constexpr int64_t kStaticScratchBytes = BASED_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char g_split_scratch[kStaticScratchBytes];
 constexpr int kMaxDevices = 64;
@@ -1171,13 +1186,20 @@ extern "C" BASED_API int based_linear_attn_prefill_split_static(
   if (n_seg <= 1)  // the unsplit kernel has no scratch at all
     return based_linear_attn_prefill(q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh,
                                      k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, io_dtype, stream);
-  // size check first: an oversized request is refused without touching the device
-  if (io_dtype == BASED_BF16 && (dv == 64 || dv == 128) && B > 0 && H > 0)
-    BASED_REQUIRE(B * H * (dv / 64) * n_seg * (int64_t)kSegStateFloats * 4 <= kStaticScratchBytes, BASED_ERR_SHAPE,
+  // Size check first: an oversized request is refused without touching the device.  Every factor
+  // is bounded before the product is formed (B * H < 2^31, at most 2 channel blocks, n_seg < 2^16,
+  // 43,008 bytes per image: below 2^63).
+  BASED_REQUIRE(B > 0 && H > 0 && B < (1ll << 31) && H < (1ll << 31) && B * H < (1ll << 31) && n_seg < 65536 &&
+                    L > 0 && L < (1ll << 31),
+                BASED_ERR_ARG, "linear_attn_prefill_split_static: bad sizes");
+  if (io_dtype == BASED_BF16 && prefill_mfma_takes(dv)) {
+    const int64_t chains = B * H * ((dv + 63) / 64);
+    BASED_REQUIRE(chains * n_seg * (int64_t)kSegStateFloats * 4 <= kStaticScratchBytes, BASED_ERR_SHAPE,
                   "linear_attn_prefill_split_static: %ld chains x %ld segments need %ld bytes of scratch, the "
                   "static array holds %ld",
-                  (long)(B * H * (dv / 64)), (long)n_seg, (long)(B * H * (dv / 64) * n_seg * (int64_t)kSegStateFloats * 4),
+                  (long)chains, (long)n_seg, (long)(chains * n_seg * (int64_t)kSegStateFloats * 4),
                   (long)kStaticScratchBytes);
+  }
   void* scratch = static_scratch_for_current_device("linear_attn_prefill_split_static");
   if (scratch == nullptr) return BASED_ERR_LAUNCH;
   return launch_prefill_split("linear_attn_prefill_split_static", q, k, v, y, kv_state, k_state, B, H, L, dv, q_sb,

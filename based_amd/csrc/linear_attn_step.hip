@@ -211,6 +211,10 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_kernel(
 // ------------------------------------------------------------------------------------------
 constexpr int kPendMax = BASED_DEFERRED_MAX_STEPS;
 
+// Register budget: the kernel is left at what the allocator needs without spilling (192 vector
+// registers at dv <= 64: two workgroups per compute unit).  Forcing three (launch bounds of three
+// wavefronts per SIMD, 168 registers) makes the allocator spill 22 registers per lane to scratch
+// memory, and the step is then a third slower instead of a tenth faster.
 template <typename T, int kMaxThreads>
 __global__ __launch_bounds__(kMaxThreads) void lin_step_deferred_kernel(
     const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
@@ -235,10 +239,6 @@ __global__ __launch_bounds__(kMaxThreads) void lin_step_deferred_kernel(
 
   // small operands first, everything unconditional (see lin_step_kernel)
   int n = pend_n[bh];
-  // (No effect on a valid count, 0..7.  With this statement in this place hipcc's scheduler ends at
-  // 166 vector registers instead of 192: three resident workgroups per compute unit instead of two,
-  // 33.7 instead of 36.9 us per step at B=128.)
-  n &= ~(kPendMax << 5);
   const int xi = tid & (2 * kFeat - 1);
   const T* x_src = (xi >> 4) ? (q + b * q_sb + h * q_sh) : (k + b * k_sb + h * k_sh);
   const float x_val = to_f32(x_src[xi & 15]);

@@ -181,15 +181,31 @@ class LinearAttention(nn.Module):
                    (self.proj_q.weight, self.proj_k.weight, self.proj_v.weight, self.out_proj.weight))
 
     def _stacked_qkv_weight(self) -> torch.Tensor:
-        """[proj_q; proj_k; proj_v] weights as one matrix, rebuilt whenever one of them has been
-        written to or replaced (tensor version counters and storage addresses are the key)."""
+        """[proj_q; proj_k; proj_v] weights as one matrix for the single-token step.  The first call
+        moves the three weights into one tensor and turns each `weight.data` into a view of its
+        rows, so there is no second copy that could go stale: writes through `weight.data`,
+        optimizers and `load_state_dict` all land in the shared storage.  Only a weight whose
+        tensor is replaced (`.to()`, a new Parameter, `weight.data = other`) changes the key below
+        (storage address, version counter), and the stack is then rebuilt from the live weights."""
         ws = (self.proj_q.weight, self.proj_k.weight, self.proj_v.weight)
         key = tuple((w.data_ptr(), w._version) for w in ws)
         cached = getattr(self, "_qkv_cache", None)
         if cached is None or cached[0] != key:
-            cached = (key, torch.cat([w.detach() for w in ws], dim=0))
+            with torch.inference_mode(False), torch.no_grad():
+                stacked = torch.cat([w.detach() for w in ws], dim=0)
+                row = 0
+                for w in ws:
+                    w.data = stacked[row:row + w.shape[0]]
+                    row += w.shape[0]
+            cached = (tuple((w.data_ptr(), w._version) for w in ws), stacked)
             self._qkv_cache = cached
         return cached[1]
+
+    def invalidate_stacked_weights(self) -> None:
+        """Forgets the stacked projection matrix (it is rebuilt from proj_q / proj_k / proj_v at the
+        next single-token step).  Never needed for in-place writes; for callers that swap weight
+        tensors behind the module's back in ways the key above cannot see."""
+        self._qkv_cache = None
 
     def parallel_forward(self, x: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
         """q, k: (b, h, l, 16) raw; v: (b, h, l, head_dim).  Returns out_proj(y), plus the decode
@@ -228,7 +244,10 @@ class LinearAttention(nn.Module):
         """(kv_state (B,H,1,head_dim,273), k_state (B,H,1,1,273)).  The states are carried in
         fp32 whatever `dtype` asks for: the decode kernel accumulates in place in fp32.  With
         `deferred_state_steps` > 1 the ring of the deferred update follows: keys (B,H,8,16), values
-        (B,H,8,head_dim), fill count (B,H)."""
+        (B,H,8,head_dim), fill count (B,H).  Such a cache is a 5-tuple and its kv_state lacks the
+        tokens still parked in the ring: whoever reads, copies or reorders kv_state itself (beam
+        search, cache export) must call `flush_deferred_state` first; unpacking it as
+        `(kv_state, k_state)` is only valid for the default 2-tuple."""
         device = self.out_proj.weight.device
         kv_state = torch.zeros(batch_size, self.num_heads, 1, self.head_dim, self.expanded_size(),
                                dtype=torch.float32, device=device)

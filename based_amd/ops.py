@@ -369,7 +369,7 @@ def linear_attn_prefill(q, k, v, eps: float = 1e-12, return_state: bool = False,
                                                       ctypes.byref(ws_bytes)))
     if isinstance(split, int) and not isinstance(split, bool) and split > 1:
         n_seg = ctypes.c_int64(split)  # explicit segment count (tests)
-        ws_bytes = ctypes.c_int64(B * H * (dv // 64) * split * _lib.PREFILL_SEGMENT_STATE_BYTES)
+        ws_bytes = ctypes.c_int64(B * H * ((dv + 63) // 64) * split * _lib.PREFILL_SEGMENT_STATE_BYTES)
     args = (q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(),
             kv_state.data_ptr() if return_state else None, k_state.data_ptr() if return_state else None,
             B, H, L, dv,
@@ -458,6 +458,9 @@ def gated_conv_step(u, state, weight, bias=None, gated: bool = True) -> torch.Te
             u2d.data_ptr(), state.data_ptr(), weight.data_ptr(), bias.data_ptr() if bias is not None else None,
             y.data_ptr(), B, D, K, u2d.stride(0), y.stride(0), _dtype_code(u), _dtype_code(state), _stream_ptr(u)))
     return y.unsqueeze(1) if squeeze else y
+
+
+ADD_RMS_NORM_MAX_DIM = 4096  # widest row based_add_rms_norm takes
 
 
 def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool = True, want_residual: bool = True):

@@ -167,6 +167,22 @@ def create_mixer_cls(config, layer_idx=None, device=None, dtype=None):
     return partial(_instantiate, value, device=device, dtype=dtype, layer_idx=layer_idx)
 
 
+def _norm_kernel_takes(x, residual, weight) -> bool:
+    """Whether `ops.add_rms_norm` accepts these device tensors: rows of a multiple of 8 up to 4096
+    elements, bf16 or fp32 activations with a weight of the same dtype, a residual
+    stream in bf16 or fp32 (fp32 for fp32 activations)."""
+    D = x.shape[-1]
+    if not (x.is_cuda and weight.is_cuda):
+        raise ValueError("based_amd runs on HIP device tensors only (no CPU path)")
+    if not (x.dtype in (torch.bfloat16, torch.float32) and weight.dtype == x.dtype
+            and D % 8 == 0 and D <= ops.ADD_RMS_NORM_MAX_DIM and weight.is_contiguous()):
+        return False
+    if residual is None:
+        return True
+    return (residual.shape == x.shape and residual.dtype in (torch.bfloat16, torch.float32)
+            and not (x.dtype == torch.float32 and residual.dtype != torch.float32))
+
+
 class RMSNorm(nn.Module):
     """x * rsqrt(mean(x^2) + eps) * weight (based/ops/triton/layer_norm.py:117-118), no bias."""
 
@@ -176,7 +192,30 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(hidden_size, device=device, dtype=dtype))
 
     def forward(self, x):
-        return ops.add_rms_norm(x, None, self.weight, self.eps, want_residual=False)[0]
+        if _norm_kernel_takes(x, None, self.weight):
+            return ops.add_rms_norm(x, None, self.weight, self.eps, want_residual=False)[0]
+        # shapes, dtypes or devices the kernel is not built for: the closed form as the reference states it
+        rstd = 1 / torch.sqrt(x.square().mean(dim=-1, keepdim=True) + self.eps)
+        return (x * rstd * self.weight).to(x.dtype)
+
+
+def add_norm(norm, hidden_states, residual, residual_in_fp32: bool, want_residual: bool = True):
+    """residual + hidden, the norm of the sum, and the sum itself for the next block
+    (block.py:134-139; gpt.py:676-694 for the closing norm).  RMSNorm on tensors the kernel takes
+    is one launch; nn.LayerNorm (`rms_norm: False`, the reference's default) and everything the
+    kernel refuses run the reference's own torch statement."""
+    if isinstance(norm, RMSNorm) and _norm_kernel_takes(hidden_states, residual, norm.weight):
+        if residual is None:
+            return ops.add_rms_norm(hidden_states, None, norm.weight, norm.eps, residual_in_fp32, want_residual)
+        return ops.add_rms_norm(hidden_states, residual, norm.weight, norm.eps,
+                                residual.dtype == torch.float32, want_residual)
+    residual = (hidden_states + residual) if residual is not None else hidden_states
+    hidden_states = norm(residual.to(dtype=norm.weight.dtype))
+    if not want_residual:
+        return hidden_states, None
+    if residual_in_fp32:
+        residual = residual.to(torch.float32)
+    return hidden_states, residual
 
 
 _GATE_ACTIVATIONS = {"glu": torch.sigmoid, "swiglu": F.silu, "geglu": F.gelu}
@@ -236,14 +275,15 @@ class Block(nn.Module):
 
     def _add_norm(self, norm, hidden_states, residual):
         """residual + hidden, the norm of the sum, and the sum kept for the next block
-        (block.py:134-139), one kernel."""
-        return ops.add_rms_norm(hidden_states, residual, norm.weight, norm.eps, self.residual_in_fp32)
+        (block.py:134-139)."""
+        return add_norm(norm, hidden_states, residual, self.residual_in_fp32)
 
     def supports_decode_step(self) -> bool:
         mlp = self.mlp
         return (getattr(self.mixer, "supports_decode_step", lambda: False)()
                 and mlp.mlp_type == "base" and mlp.activation == "swiglu"
                 and ops.decode_linear_weight_ok(mlp.fc1.weight) and ops.decode_linear_weight_ok(mlp.fc2.weight)
+                and isinstance(self.norm1, RMSNorm) and isinstance(self.norm2, RMSNorm)
                 and self.norm1.weight.dtype == torch.bfloat16 and self.residual_in_fp32)
 
     def decode_step(self, hidden_states, residual, spare, inference_params, row_index=None):
@@ -308,9 +348,8 @@ class GPTModel(nn.Module):
         self.embeddings.word_embeddings = nn.Embedding(vocab, config.hidden_size, **fk)
         if config.max_position_embeddings > 0:
             self.embeddings.position_embeddings = nn.Embedding(config.max_position_embeddings, config.hidden_size, **fk)
-        if not config.rms_norm:
-            raise NotImplementedError("the block glue kernel implements RMSNorm (rms_norm: True in the released configs)")
-        norm_cls = partial(RMSNorm, eps=config.layer_norm_epsilon, **fk)
+        # rms_norm absent from a reference config means nn.LayerNorm (gpt.py:352,537)
+        norm_cls = partial(RMSNorm if config.rms_norm else nn.LayerNorm, eps=config.layer_norm_epsilon, **fk)
         mlp_cls = partial(GatedMlp, hidden_features=config.n_inner, activation=config.activation_function,
                           bias1=config.mlp_fc1_bias, bias2=config.mlp_fc2_bias, mlp_type=config.mlp_type,
                           ff_mult=config.ff_mult, **fk)
@@ -343,7 +382,8 @@ class GPTModel(nn.Module):
         table = self.embeddings.word_embeddings.weight
         cached = self.__dict__.get("_decode_layers_supported")
         if cached is None or cached[0] != (table.dtype, table.device):
-            ok = (ops.decode_linear_weight_ok(table) and self.ln_f.weight.dtype == torch.bfloat16
+            ok = (ops.decode_linear_weight_ok(table) and isinstance(self.ln_f, RMSNorm)
+                  and self.ln_f.weight.dtype == torch.bfloat16
                   and all(layer.supports_decode_step() for layer in self.layers))
             cached = ((table.dtype, table.device), ok)
             self.__dict__["_decode_layers_supported"] = cached
@@ -368,8 +408,7 @@ class GPTModel(nn.Module):
     def forward(self, input_ids, position_ids=None, inference_params=None, stream=None):
         if self.decode_layers_ok(input_ids, inference_params):
             hidden_states, residual = self.decode_layers(input_ids, inference_params)
-            return ops.add_rms_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.eps,
-                                    want_residual=False)[0].unsqueeze(1)
+            return add_norm(self.ln_f, hidden_states, residual, True, want_residual=False)[0].unsqueeze(1)
         hidden_states = self.embeddings.word_embeddings(input_ids)
         if self.config.max_position_embeddings > 0:
             if position_ids is None:
@@ -383,8 +422,7 @@ class GPTModel(nn.Module):
         for layer in self.layers:
             hidden_states, residual = layer(hidden_states, residual=residual, position_ids=position_ids,
                                             mixer_kwargs=mixer_kwargs)
-        return ops.add_rms_norm(hidden_states, residual, self.ln_f.weight, self.ln_f.eps,
-                                residual_in_fp32=residual.dtype == torch.float32, want_residual=False)[0]
+        return add_norm(self.ln_f, hidden_states, residual, self.residual_in_fp32, want_residual=False)[0]
 
 
 class GPTLMHeadModel(nn.Module, GenerationMixin):

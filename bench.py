@@ -51,6 +51,52 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+PROBE_SRC = os.path.join(ROOT, "bench_probes.hip")
+PROBE_LIB = os.path.join(ROOT, "libbench_probes.so")
+
+
+def build_probes() -> str:
+    """Compiles bench_probes.hip (streaming kernels with no arithmetic, used by `--only machine` and
+    `--only copy`) into libbench_probes.so beside this file; cross-compiles, no GPU needed.  The
+    probes are measurement tools of this benchmark, not part of the product library."""
+    import shutil
+    import subprocess
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", PROBE_SRC, "-o", PROBE_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {PROBE_SRC}:\n{r.stdout}\n{r.stderr}")
+    return PROBE_LIB
+
+
+_probes = None
+
+
+def probes():
+    """The loaded probe library (built beforehand by build_probes(); a GPU run never compiles)."""
+    global _probes
+    if _probes is None:
+        import ctypes as C
+
+        if not os.path.exists(PROBE_LIB):
+            raise RuntimeError(f"{PROBE_LIB} not found: build it with `python -c 'import bench; bench.build_probes()'`")
+        lib = C.CDLL(PROBE_LIB)
+        lib.bench_probe_stream_qkv.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_void_p]
+        lib.bench_probe_rmw.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
+        lib.bench_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+        for fn in (lib.bench_probe_stream_qkv, lib.bench_probe_rmw, lib.bench_probe_copy):
+            fn.restype = C.c_int
+        _probes = lib
+    return _probes
+
+
+def _probe_ok(rc):
+    if rc != 0:
+        raise RuntimeError(f"bench probe refused its arguments or failed to launch (code {rc})")
+
+
 def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0):
     """Average milliseconds per call of fn(), HIP events on the current stream.  warmup_ms > 0
     keeps launching (untimed) until that much wall time has passed: the board's power management
@@ -317,11 +363,9 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
 
 def bench_machine(torch, steps=20, warmup=4, n_sets=4):
     """What this machine's memory delivers for the access patterns of the HBM-bound kernels, measured
-    with the library's probe kernels (no arithmetic) over rotating buffers beyond the last-level
-    cache: the ceiling next to which the 8 TB/s figure should be read."""
-    from based_amd import _lib
-
-    lib = _lib.lib()
+    with the probe kernels of bench_probes.hip (no arithmetic) over rotating buffers beyond the
+    last-level cache: the ceiling next to which the 8 TB/s figure should be read."""
+    lib = probes()
     dev = torch.device("cuda:0")
     stream = torch.cuda.current_stream().cuda_stream
     out = {}
@@ -333,7 +377,7 @@ def bench_machine(torch, steps=20, warmup=4, n_sets=4):
     def rmw():
         b = bufs[it[0] % n_sets]
         it[0] += 1
-        _lib.check(lib.based_probe_rmw(b.data_ptr(), n, stream))
+        _probe_ok(lib.bench_probe_rmw(b.data_ptr(), n, stream))
 
     ms, _ = _events_ms(torch, rmw, steps, warmup)
     out["rmw_cold_GBps"] = round(2 * n / (ms * 1e-3) / 1e9, 1)
@@ -342,7 +386,7 @@ def bench_machine(torch, steps=20, warmup=4, n_sets=4):
     def cp():
         i = it[0] % n_sets
         it[0] += 1
-        _lib.check(lib.based_probe_copy(bufs[i].data_ptr(), srcs[i].data_ptr(), n, stream))
+        _probe_ok(lib.bench_probe_copy(bufs[i].data_ptr(), srcs[i].data_ptr(), n, stream))
 
     ms, _ = _events_ms(torch, cp, steps, warmup)
     out["copy_cold_GBps"] = round(2 * n / (ms * 1e-3) / 1e9, 1)
@@ -355,11 +399,11 @@ def bench_machine(torch, steps=20, warmup=4, n_sets=4):
         def st():
             i = it[0] % n_sets
             it[0] += 1
-            _lib.check(lib.based_probe_stream_qkv(xs[i].data_ptr(), os_[i].data_ptr(), B, H, L, g, stream))
+            _probe_ok(lib.bench_probe_stream_qkv(xs[i].data_ptr(), os_[i].data_ptr(), B, H, L, g, stream))
 
         ms, _ = _events_ms(torch, st, steps, warmup)
         out[f"stream_qkv_cold_GBps_{g}_heads"] = round(B * L * H * 512 / (ms * 1e-3) / 1e9, 1)
-    out["note"] = ("probe kernels of the library over %d rotating buffer sets; GB/s of bytes read + written" % n_sets)
+    out["note"] = ("probe kernels of bench_probes.hip over %d rotating buffer sets; GB/s of bytes read + written" % n_sets)
     return out
 
 
@@ -594,7 +638,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "projections", "copy", "machine"], default=None,
-                    help="one workload only; 'copy' is a plain 256 MiB device copy (the library's copy probe) used to "
+                    help="one workload only; 'copy' is a plain 256 MiB device copy (the copy probe of bench_probes.hip) used to "
                          "calibrate the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run; 'machine' the memory "
                          "probes alone")
     ap.add_argument("--prefill-batches", default="1,8,32,96",
@@ -613,13 +657,11 @@ def main():
     from based_amd import ops
 
     if args.only == "copy":
-        from based_amd import _lib
-
         n = 256 * 1024 * 1024
         src = torch.empty(n, dtype=torch.uint8, device="cuda:0").fill_(1)
         dst = torch.empty_like(src)
         stream = torch.cuda.current_stream().cuda_stream
-        ms, _ = _events_ms(torch, lambda: _lib.check(_lib.lib().based_probe_copy(dst.data_ptr(), src.data_ptr(), n, stream)),
+        ms, _ = _events_ms(torch, lambda: _probe_ok(probes().bench_probe_copy(dst.data_ptr(), src.data_ptr(), n, stream)),
                            args.steps, args.warmup)
         assert bool((dst == 1).all())
         print(json.dumps({"workload": "plain device copy (probe_rw_kernel)", "bytes_read": n, "bytes_written": n,

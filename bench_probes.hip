@@ -1,5 +1,6 @@
-// Measurement probes: plain streaming kernels with the memory access patterns of the hot kernels
-// and no arithmetic to speak of.  What they reach on a given machine is the ceiling the real
+// Measurement probes of bench.py (a library of their own, libbench_probes.so; not part of the
+// product library and not declared in its header): plain streaming kernels with the memory access
+// patterns of the hot kernels and no arithmetic to speak of.  What they reach on a given machine is the ceiling the real
 // kernels are measured against next to the published HBM figure (the benchmark reports both).
 //   stream_qkv : reads a packed (B, L, 3, H, 64) bf16 tensor and writes a (B, L, H, 64) one the way
 //                the window-attention prefill does: a workgroup walks a run of tokens of G
@@ -8,9 +9,18 @@
 //                state update of the recurrent decode step.
 //   copy       : plain 16-byte-per-lane copy of known size; the calibration kernel for the
 //                profiler's HBM byte counters.
-#include "common.hpp"
+//
+// Every entry point returns 0, or 1 for arguments it does not take.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace based {
+#define PROBE_API extern "C" __attribute__((visibility("default")))
+#define PROBE_REQUIRE(cond) \
+  do {                      \
+    if (!(cond)) return 1;  \
+  } while (0)
+
+namespace bench_probes {
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
@@ -69,46 +79,44 @@ __global__ __launch_bounds__(256) void probe_rw_kernel(u32x4* dst, const u32x4* 
 
 static bool probe_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-}  // namespace based
+}  // namespace bench_probes
 
-extern "C" BASED_API int based_probe_stream_qkv(const void* qkv, void* o, int64_t B, int64_t H, int64_t L,
+PROBE_API int bench_probe_stream_qkv(const void* qkv, void* o, int64_t B, int64_t H, int64_t L,
                                                 int heads_per_group, void* stream) {
-  using namespace based;
-  BASED_REQUIRE(qkv && o, BASED_ERR_ARG, "probe_stream_qkv: null pointer argument");
-  BASED_REQUIRE(B > 0 && H > 0 && L > 0 && B < 65536 && H < 65536 && L < (1ll << 30), BASED_ERR_ARG,
-                "probe_stream_qkv: bad sizes");
-  BASED_REQUIRE(heads_per_group == 1 || heads_per_group == 2 || heads_per_group == 4, BASED_ERR_SHAPE,
-                "probe_stream_qkv: heads per group must be 1, 2 or 4");
-  BASED_REQUIRE(H % heads_per_group == 0, BASED_ERR_SHAPE, "probe_stream_qkv: H must be a multiple of the group");
-  BASED_REQUIRE(probe_aligned16(qkv) && probe_aligned16(o), BASED_ERR_ALIGN, "probe_stream_qkv: 16-byte alignment");
+  using namespace bench_probes;
+  PROBE_REQUIRE(qkv && o);
+  PROBE_REQUIRE(B > 0 && H > 0 && L > 0 && B < 65536 && H < 65536 && L < (1ll << 30));
+  PROBE_REQUIRE(heads_per_group == 1 || heads_per_group == 2 || heads_per_group == 4);
+  PROBE_REQUIRE(H % heads_per_group == 0);
+  PROBE_REQUIRE(probe_aligned16(qkv) && probe_aligned16(o));
   // as the attention launcher: runs long enough to leave about 1024 x 256 threads in flight
   const int64_t n_tiles = (L + 63) / 64;
   int64_t run_tiles = B * H * n_tiles / 1024;
   run_tiles = run_tiles < 1 ? 1 : (run_tiles > n_tiles ? n_tiles : run_tiles);
   const int64_t runs = (n_tiles + run_tiles - 1) / run_tiles * heads_per_group;
   const int64_t grid = B * (H / heads_per_group) * runs;
-  BASED_REQUIRE(grid < (1ll << 31), BASED_ERR_SHAPE, "probe_stream_qkv: grid too large");
+  PROBE_REQUIRE(grid < (1ll << 31));
   auto kern = heads_per_group == 1 ? probe_stream_qkv_kernel<1>
                                    : (heads_per_group == 2 ? probe_stream_qkv_kernel<2> : probe_stream_qkv_kernel<4>);
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), 0, static_cast<hipStream_t>(stream),
                      (const u32x4*)qkv, (u32x4*)o, (int)B, (int)H, (int)L, (int)runs);
-  return check_launch("probe_stream_qkv");
+  return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
-extern "C" BASED_API int based_probe_rmw(void* buf, int64_t bytes, void* stream) {
-  using namespace based;
-  BASED_REQUIRE(buf && bytes > 0 && bytes % 16 == 0, BASED_ERR_ARG, "probe_rmw: need a buffer of a multiple of 16 bytes");
-  BASED_REQUIRE(probe_aligned16(buf), BASED_ERR_ALIGN, "probe_rmw: 16-byte alignment");
+PROBE_API int bench_probe_rmw(void* buf, int64_t bytes, void* stream) {
+  using namespace bench_probes;
+  PROBE_REQUIRE(buf && bytes > 0 && bytes % 16 == 0);
+  PROBE_REQUIRE(probe_aligned16(buf));
   hipLaunchKernelGGL(probe_rw_kernel<false>, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream),
                      (u32x4*)buf, (const u32x4*)buf, (size_t)(bytes / 16));
-  return check_launch("probe_rmw");
+  return hipGetLastError() == hipSuccess ? 0 : 2;
 }
 
-extern "C" BASED_API int based_probe_copy(void* dst, const void* src, int64_t bytes, void* stream) {
-  using namespace based;
-  BASED_REQUIRE(dst && src && bytes > 0 && bytes % 16 == 0, BASED_ERR_ARG, "probe_copy: need buffers of a multiple of 16 bytes");
-  BASED_REQUIRE(probe_aligned16(dst) && probe_aligned16(src), BASED_ERR_ALIGN, "probe_copy: 16-byte alignment");
+PROBE_API int bench_probe_copy(void* dst, const void* src, int64_t bytes, void* stream) {
+  using namespace bench_probes;
+  PROBE_REQUIRE(dst && src && bytes > 0 && bytes % 16 == 0);
+  PROBE_REQUIRE(probe_aligned16(dst) && probe_aligned16(src));
   hipLaunchKernelGGL(probe_rw_kernel<true>, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream),
                      (u32x4*)dst, (const u32x4*)src, (size_t)(bytes / 16));
-  return check_launch("probe_copy");
+  return hipGetLastError() == hipSuccess ? 0 : 2;
 }

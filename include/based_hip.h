@@ -399,24 +399,6 @@ BASED_API int based_swa_step_anydim(const void* q, const void* k_new, const void
                           int64_t c_sb, int64_t c_st, int64_t c_sh,
                           int w_left, float scale, int io_dtype, void* stream);
 
-/*
- * Measurement probes.  No counterpart in the reference: they are streaming kernels with the
- * memory access patterns of the kernels above and no arithmetic, so that a benchmark can report,
- * next to the published HBM bandwidth, what this machine delivers for that pattern.
- *
- * based_probe_stream_qkv: reads a packed (B, L, 3, H, 64) bf16 tensor and writes a (B, L, H, 64) one
- *   as based_swa_prefill does for heads_per_group (1, 2 or 4) neighbouring heads per workgroup;
- *   512 bytes move per (token, head), as in the attention itself.
- * based_probe_rmw: reads and rewrites `bytes` (a multiple of 16) in place, 16 bytes per lane,
- *   non-temporal, like the state update of based_linear_attn_step; 2 * bytes move.
- * based_probe_copy: dst <- src, `bytes` (a multiple of 16), same access; the kernel of known size
- *   against which a profiler's HBM byte counters are calibrated.
- */
-BASED_API int based_probe_stream_qkv(const void* qkv, void* o, int64_t B, int64_t H, int64_t L,
-                                     int heads_per_group, void* stream);
-BASED_API int based_probe_rmw(void* buf, int64_t bytes, void* stream);
-BASED_API int based_probe_copy(void* dst, const void* src, int64_t bytes, void* stream);
-
 #ifdef __cplusplus
 }
 #endif

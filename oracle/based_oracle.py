@@ -28,13 +28,16 @@ tests/test_oracle.py):
   rotary_embedding        position 0 == identity, norm preservation, relative-position
                           property of the rotated dot product, complex-number brute
                           force                                            -> pinned against
-                          the published RoPE formula (GPT-NeoX half-split layout); the
+                          the published RoPE formula (GPT-NeoX half-split layout, the
+                          GPT-J interleaved layout, rotation of a leading part of the head
+                          only: each as a complex multiplication of its own pairing); the
                           reference takes it from flash-attn's rotary layer (absent), so
                           agreement with THAT library is "parity unpinned".
   gated_short_conv(_step) F.conv1d(groups=D, padding=K-1)[..., :L] + F.silu, per-element
                           brute force, step == parallel                   -> pinned
   add_rms_norm            closed form on hand-made rows, the cast BEFORE the norm (a bf16
                           sum rounded first), the fp32 residual stream     -> pinned
+  add_layer_norm          F.layer_norm (library routine), hand-made rows   -> pinned
   gated_mlp               F.glu / explicit products for the four (activation, layout)
                           combinations                                      -> pinned
   stack_forward           composition of the functions above in the order of
@@ -246,19 +249,31 @@ def gated_short_conv_step(u, state, weight, bias=None):
     return (F.silu(c.float()) * u[..., D:].float()).to(u.dtype)
 
 
-def rotary_embedding(x, positions, base: float = 10000.0):
-    """Rotary position embedding over the whole last dimension, non-interleaved ("half-split")
-    layout, as the reference applies to q and k of the sliding-window mixer through flash-attn's
-    RotaryEmbedding (slide_attention.py:346-355,553-556; rotary_emb_interleaved=False):
-        out[..., i]       = x[..., i] cos(p w_i) - x[..., i + D/2] sin(p w_i)
-        out[..., i + D/2] = x[..., i] sin(p w_i) + x[..., i + D/2] cos(p w_i),   w_i = base^(-2i/D).
+def rotary_embedding(x, positions, base: float = 10000.0, rotary_dim: int = None, interleaved: bool = False):
+    """Rotary position embedding of the first `rotary_dim` channels (default: all of them) of the
+    last dimension, as the reference applies to q and k of the sliding-window mixer through
+    flash-attn's RotaryEmbedding (slide_attention.py:346-355,553-556); channels past rotary_dim
+    pass through.  With R = rotary_dim and w_i = base^(-2i/R), i < R/2:
+      non-interleaved ("half-split", rotary_emb_interleaved=False), pairs (i, i + R/2):
+        out[..., i]       = x[..., i] cos(p w_i) - x[..., i + R/2] sin(p w_i)
+        out[..., i + R/2] = x[..., i] sin(p w_i) + x[..., i + R/2] cos(p w_i)
+      interleaved (GPT-J style), pairs (2i, 2i + 1):
+        out[..., 2i]      = x[..., 2i] cos(p w_i) - x[..., 2i + 1] sin(p w_i)
+        out[..., 2i + 1]  = x[..., 2i] sin(p w_i) + x[..., 2i + 1] cos(p w_i).
     x: (B, L, H, D); positions: (L,) integer tensor.  fp32 arithmetic, cast back to x.dtype."""
     D = x.shape[-1]
-    inv_freq = 1.0 / (base ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
-    ang = torch.outer(positions.float(), inv_freq)            # (L, D/2)
+    R = D if rotary_dim is None else int(rotary_dim)
+    assert 0 < R <= D and R % 2 == 0
+    inv_freq = 1.0 / (base ** (torch.arange(0, R, 2, dtype=torch.float32) / R))
+    ang = torch.outer(positions.float(), inv_freq)            # (L, R/2)
     cos, sin = ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]
-    x1, x2 = x[..., : D // 2].float(), x[..., D // 2:].float()
-    return torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).to(x.dtype)
+    if interleaved:
+        x1, x2 = x[..., 0:R:2].float(), x[..., 1:R:2].float()
+        rot = torch.stack([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1).flatten(-2)
+    else:
+        x1, x2 = x[..., : R // 2].float(), x[..., R // 2: R].float()
+        rot = torch.cat([x1 * cos - x2 * sin, x1 * sin + x2 * cos], dim=-1)
+    return torch.cat([rot.to(x.dtype), x[..., R:]], dim=-1)
 
 
 def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool = True):
@@ -268,6 +283,20 @@ def add_rms_norm(x, residual, weight, eps: float = 1e-5, residual_in_fp32: bool 
     r = x if residual is None else x + residual
     y = rms_norm(r.to(x.dtype), weight, eps)
     return y, (r.float() if residual_in_fp32 else r)
+
+
+def add_layer_norm(x, residual, weight, bias, eps: float = 1e-5, residual_in_fp32: bool = True):
+    """The same glue with nn.LayerNorm, the norm of a reference config without `rms_norm`
+    (gpt.py:352,537; block.py:134-139): r = x + residual, y = (c - mean(c)) / sqrt(var(c) + eps) *
+    weight + bias with c = r cast to the norm's dtype and the biased variance.  Returns (y, r)."""
+    r = x if residual is None else x + residual
+    c = r.to(weight.dtype)
+    mu = c.mean(dim=-1, keepdim=True)
+    var = (c - mu).square().mean(dim=-1, keepdim=True)
+    y = (c - mu) / torch.sqrt(var + eps) * weight
+    if bias is not None:
+        y = y + bias
+    return y.to(weight.dtype), (r.float() if residual_in_fp32 else r)
 
 
 # ----------------------------------------------------------------------------------------------
@@ -301,8 +330,8 @@ def mixer_kind(config, layer_idx: int) -> tuple:
 
 def stack_forward(input_ids, sd: dict, config: dict, dtype=torch.float32):
     """Parallel forward of the Based stack: embeddings (+ learned positions) ->
-    [add + RMSNorm -> mixer -> add + RMSNorm -> gated MLP] x n_layer -> add + final RMSNorm ->
-    LM head (GPTModel.forward gpt.py:622-736, Block.forward block.py:134-163, dropout-free,
+    [add + norm -> mixer -> add + norm -> gated MLP] x n_layer -> add + final norm -> LM head;
+    norm = RMSNorm with `rms_norm`, nn.LayerNorm without (gpt.py:352,537) (GPTModel.forward gpt.py:622-736, Block.forward block.py:134-163, dropout-free,
     prenorm, residual stream in fp32 when residual_in_fp32).  `sd` is a state dict with the
     reference's parameter names; `config` a plain dict with the reference's keys.  Activations are
     kept in `dtype` between the operations exactly where the model would hold them in its own
@@ -313,13 +342,19 @@ def stack_forward(input_ids, sd: dict, config: dict, dtype=torch.float32):
     n_embd, n_head, eps = config["n_embd"], config["n_head"], config.get("layer_norm_epsilon", 1e-5)
     res_fp32 = config.get("residual_in_fp32", False)
     B, L = input_ids.shape
+
+    def norm(x, residual, name):
+        if config.get("rms_norm", False):
+            return add_rms_norm(x, residual, g(name + ".weight"), eps, res_fp32)
+        return add_layer_norm(x, residual, g(name + ".weight"), g(name + ".bias"), eps, res_fp32)
+
     hidden = F.embedding(input_ids, g("transformer.embeddings.word_embeddings.weight"))
     if config.get("max_position_embeddings", 0) > 0:
         hidden = hidden + g("transformer.embeddings.position_embeddings.weight")[:L]
     residual = None
     for i in range(config["n_layer"]):
         pre = f"transformer.layers.{i}."
-        hidden, residual = add_rms_norm(hidden, residual, g(pre + "norm1.weight"), eps, res_fp32)
+        hidden, residual = norm(hidden, residual, pre + "norm1")
         kind, spec = mixer_kind(config, i)
         m = pre + "mixer."
         if kind == "conv":
@@ -348,17 +383,17 @@ def stack_forward(input_ids, sd: dict, config: dict, dtype=torch.float32):
             q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
             rot = int(config.get("rotary_emb_fraction", 0.0) * hd)
             if rot > 0:
-                assert rot == hd, "only whole-head rotary is restated"
                 pos = torch.arange(L)
-                q = rotary_embedding(q, pos, config.get("rotary_emb_base", 10000.0))
-                k = rotary_embedding(k, pos, config.get("rotary_emb_base", 10000.0))
+                inter = config.get("rotary_emb_interleaved", False)
+                q = rotary_embedding(q, pos, config.get("rotary_emb_base", 10000.0), rot, inter)
+                k = rotary_embedding(k, pos, config.get("rotary_emb_base", 10000.0), rot, inter)
             scale = hd ** -0.5 if config.get("scale_attn_weights", True) else 1.0
             o = sliding_window_attn(q, k, v, w_left=spec.get("window_size", 128) // 2, scale=scale)
             hidden = F.linear(o.reshape(B, L, n_embd).to(dtype), g(m + "out_proj.weight"), g(m + "out_proj.bias"))
-        hidden, residual = add_rms_norm(hidden, residual, g(pre + "norm2.weight"), eps, res_fp32)
+        hidden, residual = norm(hidden, residual, pre + "norm2")
         p = pre + "mlp."
         hidden = gated_mlp(hidden, g(p + "fc1.weight"), g(p + "fc2.weight"), g(p + "fc3.weight"),
                            config.get("activation_function", "swiglu"), g(p + "fc1.bias"), g(p + "fc2.bias"),
                            g(p + "fc3.bias"))
-    hidden, _ = add_rms_norm(hidden, residual, g("transformer.ln_f.weight"), eps, res_fp32)
+    hidden, _ = norm(hidden, residual, "transformer.ln_f")
     return F.linear(hidden, g("lm_head.weight"))

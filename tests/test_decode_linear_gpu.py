@@ -205,3 +205,24 @@ def test_rejects(dev):
         ops.decode_linear(x, w, epilogue=ops.EPILOGUE_GATED_CONV_STEP)
     with pytest.raises(ValueError):
         ops.decode_linear(x, w, conv_weight=_rand((4, 1, 3), dev, 20))
+
+
+def test_overlapping_outputs_are_refused(dev):
+    """An output that shares bytes with an input (not only the identical pointer: a view shifted by
+    a row) would race between workgroups; the entry point compares byte ranges and refuses."""
+    from based_amd import ops
+
+    torch.manual_seed(11)
+    M, K, N = 4, 256, 256
+    w = torch.randn(N, K, device=dev, dtype=torch.bfloat16)
+    nw = torch.ones(K, device=dev, dtype=torch.bfloat16)
+    buf = torch.randn(M + 1, K, device=dev, dtype=torch.float32)
+    x = torch.randn(M, K, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):   # residual_out = residual_in shifted by one row
+        ops.decode_linear(x, w, prologue=ops.PROLOGUE_ADD_RMS_NORM, residual_in=buf[:M], residual_out=buf[1:],
+                          norm_weight=nw)
+    xb = torch.randn(M + 1, K, device=dev, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):   # y aliases rows of x
+        ops.decode_linear(xb[:M], w, out=xb[1:])
+    y = ops.decode_linear(xb[:M], w)  # the same call with a fresh output is fine
+    assert torch.isfinite(y.float()).all()

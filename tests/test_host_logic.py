@@ -90,8 +90,10 @@ def test_cpu_modules_fail_loudly():
         GatedMlp(32, hidden_features=64)(x)
     with pytest.raises(ValueError):
         ShortConvolution(32, kernel_size=3)(x)
-    with pytest.raises(NotImplementedError):
-        GPTLMHeadModel(based_360m_config(n_layer=1, vocab_size=64, rms_norm=False))
+    # a LayerNorm stack (rms_norm: False, the reference's default) builds; its norms are torch modules
+    ln_model = GPTLMHeadModel(based_360m_config(n_layer=1, vocab_size=64, rms_norm=False))
+    assert isinstance(ln_model.transformer.ln_f, torch.nn.LayerNorm)
+    assert "transformer.layers.0.norm1.bias" in ln_model.state_dict()
 
 
 def test_stack_routing_and_state_dict_names():

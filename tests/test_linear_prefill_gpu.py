@@ -50,6 +50,44 @@ def test_bf16_mfma_matches_oracle(dev, B, H, L, dv):
     _check(dev, q, k, v, torch.bfloat16)
 
 
+@pytest.mark.parametrize("B,H,L,dv", [(1, 2, 200, 112), (2, 3, 65, 112), (1, 2, 130, 16), (1, 2, 100, 48),
+                                      (1, 1, 77, 80), (1, 2, 64, 96), (1, 1, 150, 176), (1, 2, 1, 112)])
+def test_bf16_mfma_head_dims_that_are_no_multiple_of_64(dev, B, H, L, dv):
+    """Head dims in whole 16-channel tiles: the last 64-channel block of a workgroup grid runs with
+    fewer live tiles (112 = 64 + 48 is the released 1B / 1.3B shape: n_embd 1792 over 16 heads).
+    Outputs AND states against the oracle; the channels past dv must not leak into anything (the
+    output and state tensors are exactly dv wide, so an out-of-range store would corrupt a
+    neighbouring head, which the comparison would show)."""
+    print(f"prefill bf16 odd-dv case B={B} H={H} L={L} dv={dv}", flush=True)
+    q, k, v = _qkv(B, H, L, dv, torch.bfloat16, seed=23)
+    _check(dev, q, k, v, torch.bfloat16)
+
+
+def test_bf16_mfma_dv112_projection_layout_split_and_steps(dev):
+    """dv = 112 in the layout the module hands over ((B, L, H*112) projections viewed (B, H, L, 112)),
+    scanned in one pass and as segments, then decoded on: every step equals the parallel form."""
+    from based_amd import ops
+
+    B, H, L, T, dv = 2, 16, 700, 5, 112
+    g = torch.Generator().manual_seed(24)
+    qp = torch.randn(B, L + T, H * 16, generator=g).bfloat16()
+    kp = torch.randn(B, L + T, H * 16, generator=g).bfloat16()
+    vp = torch.randn(B, L + T, H * dv, generator=g).bfloat16()
+    view = lambda t, d: t.view(B, L + T, H, d).transpose(1, 2)
+    y_ref = O.linear_attn_cumsum(view(qp, 16).float(), view(kp, 16).float(), view(vp, dv).float())
+    qd, kd, vd = view(qp.to(dev), 16), view(kp.to(dev), 16), view(vp.to(dev), dv)
+    y1, kv1, ks1 = ops.linear_attn_prefill(qd[:, :, :L], kd[:, :, :L], vd[:, :, :L], return_state=True, split=False)
+    y2, kv2, ks2 = ops.linear_attn_prefill(qd[:, :, :L], kd[:, :, :L], vd[:, :, :L], return_state=True, split=3)
+    assert y1.transpose(1, 2).is_contiguous()
+    assert rel_l2(y1.float(), y_ref[:, :, :L]) < 1e-2 and rel_l2(y2.float(), y_ref[:, :, :L]) < 1e-2
+    kv_ref, ks_ref = O.linear_attn_prefill_state(view(kp, 16)[:, :, :L].float(), view(vp, dv)[:, :, :L].float())
+    for kv, ks in ((kv1, ks1), (kv2, ks2)):
+        assert rel_l2(kv, kv_ref) < 5e-3 and rel_l2(ks, ks_ref) < 5e-3
+    for t in range(L, L + T):
+        y = ops.linear_attn_step(qd[:, :, t:t + 1], kd[:, :, t:t + 1], vd[:, :, t:t + 1], kv1, ks1)
+        assert rel_l2(y.float(), y_ref[:, :, t:t + 1]) < 1e-2
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_golden_reference_causal_product(dev, dtype):
     """Both prefill kernels against the committed output of the reference's compiled CPU causal
@@ -82,7 +120,7 @@ def test_config1_fp32(dev):
 
 
 @pytest.mark.parametrize("B,H,L,dv,dtype", [(1, 2, 37, 64, torch.float32), (2, 1, 9, 32, torch.float32),
-                                            (1, 2, 70, 16, torch.bfloat16), (1, 1, 50, 192, torch.float32)])
+                                            (1, 2, 70, 24, torch.bfloat16), (1, 1, 50, 192, torch.float32)])
 def test_fp32_kernel_shapes(dev, B, H, L, dv, dtype):
     print(f"prefill f32-kernel case B={B} H={H} L={L} dv={dv} {dtype}", flush=True)
     q, k, v = _qkv(B, H, L, dv, dtype, seed=9)
@@ -201,3 +239,7 @@ def test_split_plan(dev):
     assert n.value == 1                                      # fp32 path is never split
     assert lib.based_linear_attn_prefill_plan(1, 16, 64, 64, 0, ctypes.byref(n), ctypes.byref(w)) == 0
     assert n.value == 1                                      # a single chunk cannot be split
+    assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 112, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value >= 2 and w.value == 32 * n.value * 43008  # dv 112: two channel blocks per (batch, head)
+    assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 72, 0, ctypes.byref(n), ctypes.byref(w)) == 0
+    assert n.value == 1 and w.value == 0                     # not whole 16-channel tiles: the fp32 kernel, never split

@@ -132,3 +132,45 @@ def test_graph_decode_equals_eager(dev):
             assert rel_l2(a.float(), b_.float()) < 1e-3, f"trial {trial} position {i}"
         assert torch.equal(graphed.sequences, eager.sequences)
     assert len(model._decoding_cache.callables) == 2  # one graph per batch size, reused across requests
+
+
+def test_linear_attention_step_sees_weights_written_through_data(dev):
+    """The single-token step projects through one stacked [q; k; v] matrix.  A write that bypasses
+    the version counter (`weight.data.copy_`, what EMA swaps and some optimizers do) must reach
+    it: the projections are views of the stacked storage, not copies."""
+    from based_amd.generation import InferenceParams
+    from based_amd.mixers import LinearAttention, TaylorExp
+
+    torch.manual_seed(4)
+    m = LinearAttention(d_model=256, feature_map=TaylorExp(input_dim=16), num_heads=4, head_dim=64,
+                        layer_idx=0, device=dev, dtype=torch.bfloat16).eval()
+    for p in m.parameters():
+        torch.nn.init.normal_(p, std=0.2)
+
+    def prefill_and_step(x, x1):
+        params = InferenceParams(max_seqlen=64, max_batch_size=2)
+        with torch.inference_mode():
+            m(x, inference_params=params)
+            params.seqlen_offset = x.shape[1]
+            return m(x1, inference_params=params)
+
+    x = torch.randn(2, 20, 256, device=dev, dtype=torch.bfloat16)
+    x1 = torch.randn(2, 1, 256, device=dev, dtype=torch.bfloat16)
+    before = prefill_and_step(x, x1)
+    full = m(torch.cat([x, x1], dim=1))[:, -1:]
+    assert rel_l2(before.float(), full.float()) < 1.5e-2
+    new_q = torch.randn_like(m.proj_q.weight) * 0.2
+    new_v = torch.randn_like(m.proj_v.weight) * 0.2
+    v0 = m.proj_q.weight._version
+    m.proj_q.weight.data.copy_(new_q)
+    m.proj_v.weight.data.copy_(new_v)
+    assert m.proj_q.weight._version == v0          # the write the cache key cannot see
+    after = prefill_and_step(x, x1)
+    full = m(torch.cat([x, x1], dim=1))[:, -1:]   # the parallel path reads the live weights
+    assert rel_l2(after.float(), full.float()) < 1.5e-2
+    assert rel_l2(after.float(), before.float()) > 0.1
+    # a replaced tensor is noticed through its address
+    m.proj_k.weight = torch.nn.Parameter(torch.randn_like(m.proj_k.weight) * 0.2)
+    again = prefill_and_step(x, x1)
+    assert rel_l2(again.float(), m(torch.cat([x, x1], dim=1))[:, -1:].float()) < 1.5e-2
+    assert torch.equal(m.state_dict()["proj_q.weight"], new_q)

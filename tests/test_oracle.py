@@ -285,6 +285,55 @@ def test_rotary_embedding_properties():
         assert abs(float(rx[b, l, h, i]) - z.real) < 1e-5 and abs(float(rx[b, l, h, i + D // 2]) - z.imag) < 1e-5
 
 
+def test_rotary_embedding_partial_and_interleaved():
+    """The two other rotary shapes the reference's constructor admits (rotary_emb_dim < head dim,
+    rotary_emb_interleaved; slide_attention.py:346-355): each against a complex multiplication of
+    ITS pairing, channels past rotary_dim untouched, and the interleaved layout as the half-split
+    one under the channel permutation that maps pair (2i, 2i+1) to (i, i + R/2)."""
+    g = torch.Generator().manual_seed(10)
+    B, L, H, D, R = 2, 9, 2, 48, 32
+    x = torch.randn(B, L, H, D, generator=g)
+    pos = torch.arange(3, 3 + L)
+    part = O.rotary_embedding(x, pos, rotary_dim=R)
+    assert torch.equal(part[..., R:], x[..., R:])
+    assert torch.allclose(part[..., :R], O.rotary_embedding(x[..., :R], pos), atol=1e-6)
+    inter = O.rotary_embedding(x, pos, rotary_dim=R, interleaved=True)
+    assert torch.equal(inter[..., R:], x[..., R:])
+    for (b, l, h, i) in [(0, 0, 0, 0), (1, 8, 1, 15), (0, 4, 1, 7)]:
+        w = 10000.0 ** (-2.0 * i / R)
+        p = int(pos[l])
+        z = complex(float(x[b, l, h, i]), float(x[b, l, h, i + R // 2])) * complex(math.cos(p * w), math.sin(p * w))
+        assert abs(float(part[b, l, h, i]) - z.real) < 1e-5 and abs(float(part[b, l, h, i + R // 2]) - z.imag) < 1e-5
+        z = complex(float(x[b, l, h, 2 * i]), float(x[b, l, h, 2 * i + 1])) * complex(math.cos(p * w), math.sin(p * w))
+        assert abs(float(inter[b, l, h, 2 * i]) - z.real) < 1e-5 and abs(float(inter[b, l, h, 2 * i + 1]) - z.imag) < 1e-5
+    perm = torch.cat([torch.arange(0, R, 2), torch.arange(1, R, 2)])          # half-split position -> interleaved channel
+    half = O.rotary_embedding(x[..., :R][..., perm], pos)
+    assert torch.allclose(half, inter[..., :R][..., perm], atol=1e-6)
+    assert torch.allclose(inter.norm(dim=-1), x.norm(dim=-1), rtol=1e-5)
+
+
+def test_add_layer_norm_against_library_routine():
+    """nn.LayerNorm glue of a config without rms_norm: F.layer_norm on the cast sum, the fp32 stream
+    handed on unrounded, and one row by hand."""
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(3, 5, 32, generator=g)
+    res = torch.randn(3, 5, 32, generator=g)
+    w, b = torch.randn(32, generator=g), torch.randn(32, generator=g)
+    y, r = O.add_layer_norm(x, res, w, b, eps=1e-5)
+    assert torch.allclose(y, F.layer_norm(x + res, (32,), w, b, 1e-5), atol=1e-5) and torch.equal(r, x + res)
+    y, r = O.add_layer_norm(x, None, w, None, eps=1e-5)
+    assert torch.allclose(y, F.layer_norm(x, (32,), w, None, 1e-5), atol=1e-5) and torch.equal(r, x)
+    # bf16 activations on an fp32 stream: normalised from the bf16-rounded sum, stream kept in fp32
+    xb = x.bfloat16()
+    y, r = O.add_layer_norm(xb, res, w.bfloat16(), b.bfloat16(), eps=1e-5)
+    assert y.dtype == torch.bfloat16 and r.dtype == torch.float32 and torch.equal(r, xb.float() + res)
+    want = F.layer_norm((xb.float() + res).bfloat16(), (32,), w.bfloat16(), b.bfloat16(), 1e-5)
+    assert torch.allclose(y.float(), want.float(), atol=4e-2)
+    # by hand: [1, 3] -> mean 2, var 1 -> [-1, 1] * w + b
+    y, _ = O.add_layer_norm(torch.tensor([[1.0, 3.0]]), None, torch.tensor([2.0, 3.0]), torch.tensor([0.5, -0.5]), eps=0.0)
+    assert torch.allclose(y, torch.tensor([[-1.5, 2.5]]), atol=1e-6)
+
+
 def test_add_rms_norm_closed_form_cast_order_and_fp32_stream():
     """The prenorm glue (block.py:134-139): (i) closed form on hand-made rows; (ii) the sum is cast to
     the activation dtype BEFORE the norm (a bf16 activation plus an fp32 residual is normalised from
@@ -419,3 +468,55 @@ def test_stack_forward_against_hand_unrolled_modules():
     ids2 = ids.clone()
     ids2[:, -1] = (ids2[:, -1] + 1) % 96
     assert torch.equal(O.stack_forward(ids2, sd, cfg)[:, :-1], got[:, :-1])
+
+
+def test_stack_forward_layer_norm_config_against_nn_modules():
+    """A reference-format config that omits rms_norm (nn.LayerNorm, gpt.py:352,537) and rotates a
+    part of the head in the interleaved layout: the composition against nn.LayerNorm /
+    nn.Linear building blocks, the mixer (one window layer) unrolled by hand."""
+    import torch.nn as nn
+
+    from based_amd.stack import GPTLMHeadModel, StackConfig
+
+    torch.manual_seed(5)
+    cfg = _tiny_stack_config(n_layer=1, alt_mixer_layers=[], alt_mixer_2_layers=[0], rotary_emb_fraction=0.5,
+                             rotary_emb_interleaved=True, qkv_proj_bias=True, out_proj_bias=True)
+    del cfg["rms_norm"]
+    full = vars(StackConfig.from_reference_dict(cfg))
+    assert full["rms_norm"] is False
+    model = GPTLMHeadModel(StackConfig.from_reference_dict(cfg))
+    assert isinstance(model.transformer.ln_f, nn.LayerNorm)
+    sd = {k: v.detach().clone() for k, v in model.state_dict().items()}
+    for k in sd:
+        if "norm" in k or "ln_f" in k or k.endswith("bias"):
+            sd[k] = (1.0 if k.endswith("weight") else 0.0) + 0.1 * torch.randn_like(sd[k])
+    B, L, D, H = 2, 12, 128, 2
+    ids = torch.randint(0, 96, (B, L))
+    got = O.stack_forward(ids, sd, full)
+
+    def ln(x, name):
+        m = nn.LayerNorm(D, eps=1e-5)
+        m.weight.data.copy_(sd[name + ".weight"])
+        m.bias.data.copy_(sd[name + ".bias"])
+        return m(x)
+
+    pre = "transformer.layers.0."
+    res = F.embedding(ids, sd["transformer.embeddings.word_embeddings.weight"])
+    x = ln(res, pre + "norm1")
+    qkv = (x @ sd[pre + "mixer.Wqkv.weight"].T + sd[pre + "mixer.Wqkv.bias"]).view(B, L, 3, H, 64)
+    q, k, v = qkv[:, :, 0].clone(), qkv[:, :, 1].clone(), qkv[:, :, 2]
+    for t in (q, k):            # interleaved rotary of the first 32 channels, pair by pair
+        for l in range(L):
+            for i in range(16):
+                a = l * 10000.0 ** (-2.0 * i / 32)
+                x0, x1 = t[:, l, :, 2 * i].clone(), t[:, l, :, 2 * i + 1].clone()
+                t[:, l, :, 2 * i] = x0 * math.cos(a) - x1 * math.sin(a)
+                t[:, l, :, 2 * i + 1] = x0 * math.sin(a) + x1 * math.cos(a)
+    o = F.scaled_dot_product_attention(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True)
+    h = o.transpose(1, 2).reshape(B, L, D) @ sd[pre + "mixer.out_proj.weight"].T + sd[pre + "mixer.out_proj.bias"]
+    res = h + res
+    x = ln(res, pre + "norm2")
+    yv, gate = (x @ sd[pre + "mlp.fc1.weight"].T).chunk(2, -1)
+    h = (yv * F.silu(gate)) @ sd[pre + "mlp.fc2.weight"].T
+    ref = ln(h + res, "transformer.ln_f") @ sd["lm_head.weight"].T
+    assert torch.allclose(got, ref, atol=3e-5, rtol=1e-5)

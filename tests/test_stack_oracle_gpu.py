@@ -162,3 +162,55 @@ def test_reference_generation_configs_as_written(dev, config, prefill_size, dtyp
                 want = O.stack_forward(seqs[:, : prefill_size + i].cpu(), sd, full_cfg)[:, -1]
                 _allclose_all(scores[:, i], want, dtype, f"cached step {i} vs oracle")
                 _allclose_all(scores_ref[:, -1], want, dtype, f"parallel step {i} vs oracle")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layer_norm_stack_from_reference_dict(dev, dtype):
+    """A reference-format config WITHOUT `rms_norm` means nn.LayerNorm (gpt.py:352,537): it builds
+    through from_reference_dict, runs (the norms as torch statements, everything else through the
+    kernels) and matches the oracle composition, prefill and cached steps; an odd hidden size
+    for the norm kernel (n_embd 264 is no multiple of 16 heads x 16, so heads of 66 would not do:
+    use 4 heads of 64 + RMSNorm rows the kernel refuses) is covered by the second case below."""
+    from based_amd.stack import GPTLMHeadModel, StackConfig
+
+    cfg = _tiny_cfg(alt_mixer_2_layers=[] if dtype == torch.float32 else [2], n_layer=2 if dtype == torch.float32 else 3)
+    del cfg["rms_norm"]
+    config = StackConfig.from_reference_dict(cfg)
+    assert config.rms_norm is False
+    torch.manual_seed(7)
+    model = GPTLMHeadModel(config, device=dev, dtype=dtype).eval()
+    assert isinstance(model.transformer.layers[0].norm1, torch.nn.LayerNorm)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if "norm" in name or "ln_f" in name:
+                p.copy_((1.0 if name.endswith("weight") else 0.0) + 0.1 * torch.randn_like(p))
+    sd = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    full_cfg = vars(config)
+    B, P, n_new = 2, 40, 8
+    ids = torch.randint(1, 1000, (B, P), dtype=torch.long, device=dev)
+    with torch.inference_mode():
+        logits = model(ids).logits
+    _allclose_all(logits, O.stack_forward(ids.cpu(), sd, full_cfg), dtype, "prefill logits")
+    out = model.generate(input_ids=ids, max_length=P + n_new, return_dict_in_generate=True, output_scores=True, top_k=1)
+    seqs = out.sequences.cpu()
+    for i, sc in enumerate(out.scores):
+        _allclose_all(sc, O.stack_forward(seqs[:, : P + i], sd, full_cfg)[:, -1], dtype, f"cached decode step {i}")
+
+
+def test_rms_norm_rows_the_kernel_refuses_run_as_torch(dev):
+    """A norm weight whose dtype differs from the activations (fp32 norms in a bf16 model) is not
+    something the norm kernel takes; the block then states the norm in torch instead of raising."""
+    from based_amd.stack import RMSNorm, add_norm
+
+    torch.manual_seed(8)
+    norm = RMSNorm(256, eps=1e-5, device=dev, dtype=torch.float32)
+    with torch.no_grad():
+        norm.weight.copy_(1.0 + 0.1 * torch.randn_like(norm.weight))
+    x = torch.randn(6, 256, device=dev, dtype=torch.bfloat16)
+    res = torch.randn(6, 256, device=dev, dtype=torch.float32)
+    y, r = add_norm(norm, x, res, residual_in_fp32=True)
+    want_r = x.float() + res
+    want_y, _ = O.add_rms_norm(want_r.cpu(), None, norm.weight.cpu(), 1e-5)
+    assert torch.equal(r, want_r) and torch.allclose(y.cpu(), want_y, atol=1e-5)
+    with pytest.raises(ValueError):
+        add_norm(norm, x.cpu(), None, True)  # no CPU path
