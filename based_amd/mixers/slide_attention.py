@@ -5,10 +5,11 @@ constructor arguments, parameter names (Wqkv / out_proj), forward and
 allocate_inference_cache signatures and the reference's linear (B, max_seqlen, 2, H, D) KV
 cache.  `window_size=W` means query i attends keys [i - W//2, i] (flash-attn's
 `window_size=(W//2, 0)` with causal=True, slide_attention.py:332-336).
-In scope: self-attention, num_heads_kv == num_heads, head_dim 64 (MFMA kernels; other multiples
-of 8 up to 128 run a plain kernel), window_size up to 256 (128 keys to the left, what the released
-checkpoints use), no dropout / padding / varlen; other arguments
-raise NotImplementedError.  Non-half inputs are computed in bf16
+In scope: self-attention, num_heads_kv == num_heads, head dims that are multiples of 8 up to 128
+(64, 112 and 128 are the released models'), rotary over any leading multiple of 16 channels in
+either pair layout, applied inside the kernels, window_size up to 256 (128 keys to the left, what
+the released checkpoints use), no dropout / padding / varlen; other arguments raise
+NotImplementedError.  Non-half inputs are computed in bf16
 (the reference casts to bf16 for prefill, slide_attention.py:76-78).
 """
 from __future__ import annotations
@@ -39,8 +40,8 @@ class RotaryEmbedding(nn.Module):
         return freqs.cos(), freqs.sin()
 
     def tables(self, n_pos: int, device):
-        """(cos, sin) fp32 (>= n_pos, dim/2) tables for the kernels' in-flight rotation; grown on
-        demand and kept (a captured decode graph holds their addresses)."""
+        """(cos, sin, interleaved): fp32 (>= n_pos, dim/2) tables for the kernels' in-flight rotation
+        and the pair layout; grown on demand and kept (a captured decode graph holds their addresses)."""
         cached = getattr(self, "_tables", None)
         if cached is None or cached[0].shape[0] < n_pos or cached[0].device != device:
             if cached is not None:
@@ -48,7 +49,7 @@ class RotaryEmbedding(nn.Module):
                 # stay correct for the positions they cover)
                 self._retired_tables = getattr(self, "_retired_tables", []) + [cached]
             cos, sin = self._cos_sin(torch.arange(n_pos, device=device))
-            self._tables = (cos.contiguous(), sin.contiguous())
+            self._tables = (cos.contiguous(), sin.contiguous(), self.interleaved)
         return self._tables
 
     def _rotate(self, x, cos, sin):
@@ -125,7 +126,10 @@ class SlidingAttention(nn.Module):
         assert self.embed_dim % num_heads == 0, "embed_dim must be divisible by num_heads"
         self.head_dim = self.embed_dim // num_heads
         if self.head_dim % 8 != 0 or self.head_dim > 128:
-            raise NotImplementedError("the HIP kernels take head dims that are multiples of 8 up to 128 (64: MFMA path)")
+            raise NotImplementedError("the HIP kernels take head dims that are multiples of 8 up to 128")
+        if self.rotary_emb_dim > 0 and (self.rotary_emb_dim % 16 != 0 or self.rotary_emb_dim > self.head_dim):
+            # flash-attn's rotary kernels ask for the same (a multiple of 16, at most the head dim)
+            raise NotImplementedError(f"rotary_emb_dim {self.rotary_emb_dim}: a multiple of 16 up to head_dim {self.head_dim}")
         self.softmax_scale = softmax_scale if softmax_scale is not None else 1.0 / math.sqrt(self.head_dim)
         if self.rotary_emb_dim > 0:
             self.rotary_emb = RotaryEmbedding(self.rotary_emb_dim, base=rotary_emb_base,
@@ -150,10 +154,7 @@ class SlidingAttention(nn.Module):
         return d[self.layer_idx]
 
     def supports_decode_step(self) -> bool:
-        in_kernel_rotary = self.head_dim == 64 and self.rotary_emb_dim == 64 and not self.rotary_emb.interleaved \
-            if self.rotary_emb_dim > 0 else True
-        return (in_kernel_rotary and ops.decode_linear_weight_ok(self.Wqkv.weight)
-                and ops.decode_linear_weight_ok(self.out_proj.weight))
+        return ops.decode_linear_weight_ok(self.Wqkv.weight) and ops.decode_linear_weight_ok(self.out_proj.weight)
 
     def decode_step(self, x, inference_params, **prologue):
         """One token per sequence with the projections as `ops.decode_linear` launches: x (b, hidden)
@@ -189,17 +190,12 @@ class SlidingAttention(nn.Module):
         if qkv.dtype != torch.bfloat16:
             qkv = qkv.to(torch.bfloat16)
         offset = 0 if inference_params is None else inference_params.seqlen_offset
-        # Rotary over the whole head, non-interleaved (the released configurations), happens inside
-        # the kernels; other rotary shapes are applied here with torch ops at host-known positions.
+        # the rotation (whole head or a leading part, either pair layout) happens inside the kernels,
+        # at positions they take from the host or, for a recorded decode step, from the device
         rope = None
         if self.rotary_emb_dim > 0:
-            if self.head_dim == 64 and self.rotary_emb_dim == 64 and not self.rotary_emb.interleaved:
-                n_pos = seqlen if inference_params is None else max(inference_params.max_seqlen, offset + seqlen)
-                rope = self.rotary_emb.tables(n_pos, qkv.device)
-            else:
-                if inference_params is not None and inference_params.lengths_per_sample is not None:
-                    raise NotImplementedError("per-sample positions need the in-kernel rotary (full head, non-interleaved)")
-                qkv = self.rotary_emb(qkv, seqlen_offset=offset)
+            n_pos = seqlen if inference_params is None else max(inference_params.max_seqlen, offset + seqlen)
+            rope = self.rotary_emb.tables(n_pos, qkv.device)
         q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
 
         if inference_params is None:

@@ -203,41 +203,53 @@ def linear_attn_flush_deferred(kv_state, pending) -> None:
                                                                pend_n.data_ptr(), B, H, dv, _stream_ptr(kv_state)))
 
 
-def _rope_tables(rope, device, need_rows):
-    """(cos, sin) fp32 (n_pos, 32) contiguous device tables -> (cos_ptr, sin_ptr, n_pos) or Nones."""
+def _rope_tables(rope, device, need_rows, head_dim):
+    """rope = (cos, sin) or (cos, sin, interleaved): fp32 (n_pos, rotary_dim / 2) contiguous device
+    tables -> (cos_ptr, sin_ptr, n_pos, rotary_dim, interleaved), or Nones / zeros without rotary."""
     if rope is None:
-        return None, None, 0
-    cos, sin = rope
+        return None, None, 0, 0, False
+    cos, sin = rope[0], rope[1]
+    interleaved = bool(rope[2]) if len(rope) > 2 else False
     for t in (cos, sin):
-        if (not t.is_cuda or t.device != device or t.dtype != torch.float32 or t.dim() != 2
-                or t.shape[1] != 32 or not t.is_contiguous()):
-            raise ValueError("rotary tables must be contiguous fp32 (n_pos, 32) tensors on the device of q")
+        if not t.is_cuda or t.device != device or t.dtype != torch.float32 or t.dim() != 2 or not t.is_contiguous():
+            raise ValueError("rotary tables must be contiguous fp32 (n_pos, rotary_dim / 2) tensors on the device of q")
+    rotary_dim = 2 * cos.shape[1]
     if cos.shape != sin.shape or cos.shape[0] < need_rows:
         raise ValueError(f"rotary tables hold {cos.shape[0]} positions, need {need_rows}")
-    return cos.data_ptr(), sin.data_ptr(), cos.shape[0]
+    if rotary_dim % 16 != 0 or not 0 < rotary_dim <= head_dim:
+        raise ValueError(f"rotary_dim {rotary_dim} must be a multiple of 16 and at most the head dim {head_dim}")
+    return cos.data_ptr(), sin.data_ptr(), cos.shape[0], rotary_dim, interleaved
+
+
+def _swa_fast64(D: int, rotary_dim: int, interleaved: bool, impl) -> bool:
+    """Head dim 64 without rotary, or rotated over the whole head in half-split pairs, runs the
+    kernels built for exactly that (two heads per workgroup, 128-byte rows)."""
+    return impl is None and D == 64 and (rotary_dim == 0 or (rotary_dim == 64 and not interleaved))
 
 
 def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=None, kv_cache=None,
-                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out: Optional[torch.Tensor] = None, impl: Optional[str] = None) -> torch.Tensor:
     """Sliding-window causal attention.  q, k, v: (B, L, H, D) bf16 (any strides with the
-    last dim contiguous, e.g. slices of a packed qkv).  Query i sees keys [i - w_left, i], 0 <= w_left <= 128.
-    D = 64 runs the MFMA kernel; other head dims (multiples of 8 up to 128) a plain one-wavefront-per-
-    query kernel without in-kernel rotary.
-    rope: None or (cos, sin) fp32 (n_pos >= L, 32) tables; q and k are then rotated in the kernel
-    (non-interleaved rotary over the whole head, positions 0..L-1).
-    kv_cache: None or a (B, max_seqlen >= L, 2, H, 64) bf16 cache whose rows 0..L-1 receive the
-    (rotated) k and v.  out: None or a (B, L, H, 64) tensor (last dim contiguous) to write into."""
+    last dim contiguous, e.g. slices of a packed qkv), D a multiple of 8 up to 128.  Query i sees
+    keys [i - w_left, i], 0 <= w_left <= 128.
+    rope: None, or (cos, sin[, interleaved]) with fp32 (n_pos >= L, rotary_dim / 2) tables: the
+    first rotary_dim channels of q and k are rotated in the kernel at positions 0..L-1, in
+    half-split pairs (c, c + rotary_dim / 2) or, interleaved, pairs (2i, 2i + 1).
+    kv_cache: None or a (B, max_seqlen >= L, 2, H, D) bf16 cache whose rows 0..L-1 receive the
+    (rotated) k and v.  out: None or a (B, L, H, D) tensor (last dim contiguous) to write into.
+    impl: None (MFMA kernels), "wide" (the general MFMA kernel also where the 64-channel one would
+    do) or "plain" (the one-wavefront-per-query kernel, no rotary: a second statement for tests)."""
     _require_cuda(q, k, v)
     B, L, H, D = q.shape
     if k.shape != q.shape or v.shape != q.shape:
         raise ValueError(f"bad shapes q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
-    if D != 64 and rope is not None:
-        raise ValueError("in-kernel rotary needs head dim 64")
     for t in (q, k, v):
         if t.stride(-1) != 1:
             raise ValueError("innermost dimension must be contiguous")
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
-    cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, L)
+    cos_ptr, sin_ptr, n_pos, rotary_dim, interleaved = _rope_tables(rope, q.device, L, D)
+    if impl == "plain" and rope is not None:
+        raise ValueError("the plain kernel has no in-kernel rotary")
     kc_ptr = vc_ptr = None
     c_strides, max_seqlen = (0, 0, 0), 0
     if kv_cache is not None:
@@ -254,31 +266,34 @@ def swa_prefill(q, k, v, w_left: int = 64, scale: Optional[float] = None, rope=N
         o = out
         if tuple(o.shape) != (B, L, H, D) or o.dtype != q.dtype or o.device != q.device or o.stride(-1) != 1:
             raise ValueError(f"out must be a ({B}, {L}, {H}, {D}) {q.dtype} tensor on {q.device}")
+    strides = (q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+               v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2))
     with _on_device(q.device):
-        if D == 64:
+        if _swa_fast64(D, rotary_dim, interleaved, impl):
             _lib.check(_lib.lib().based_swa_prefill(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L,
-                q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L, *strides,
                 int(w_left), scale, cos_ptr, sin_ptr, n_pos, kc_ptr, vc_ptr, *c_strides, max_seqlen,
                 _dtype_code(q), _stream_ptr(q)))
-        else:
+        elif impl == "plain":
             _lib.check(_lib.lib().based_swa_prefill_anydim(
-                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L, D,
-                q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                v.stride(0), v.stride(1), v.stride(2), o.stride(0), o.stride(1), o.stride(2),
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L, D, *strides,
                 int(w_left), scale, kc_ptr, vc_ptr, *c_strides, max_seqlen, _dtype_code(q), _stream_ptr(q)))
+        else:
+            _lib.check(_lib.lib().based_swa_prefill_wide(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, L, D, *strides,
+                int(w_left), scale, cos_ptr, sin_ptr, n_pos, rotary_dim, int(interleaved), kc_ptr, vc_ptr, *c_strides,
+                max_seqlen, _dtype_code(q), _stream_ptr(q)))
     return o
 
 
 def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[float] = None, rope=None,
-             out: Optional[torch.Tensor] = None) -> torch.Tensor:
+             out: Optional[torch.Tensor] = None, impl: Optional[str] = None) -> torch.Tensor:
     """Decode step.  q, k_new, v_new: (B, 1, H, D) bf16; kv_cache (B, max_seqlen, 2, H, D)
-    bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.  D = 64, or
-    another multiple of 8 up to 128 (plain kernel, no in-kernel rotary).
+    bf16, row `pos` is written in place, then rows [pos - w_left, pos] are attended.  D a multiple
+    of 8 up to 128.
     pos: int (same for the whole batch) or an int32 device tensor of B positions.
-    rope: None or (cos, sin) tables as for swa_prefill: q and k_new are rotated at `pos` first.
-    out: None or a (B, 1, H, 64) tensor (last dim contiguous) to write into."""
+    rope: None or (cos, sin[, interleaved]) tables as for swa_prefill: q and k_new are rotated at `pos` first.
+    out: None or a (B, 1, H, D) tensor (last dim contiguous) to write into.  impl: as for swa_prefill."""
     key = ("swa_step", q.shape, q.stride(), k_new.shape, k_new.stride(), v_new.shape, v_new.stride(), kv_cache.shape,
            kv_cache.stride(), q.dtype, k_new.dtype, v_new.dtype, kv_cache.dtype, q.device, k_new.device, v_new.device,
            kv_cache.device)
@@ -298,16 +313,16 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
         _CHECKED[key] = True
     B, _, H, D = q.shape
     scale = 1.0 / math.sqrt(D) if scale is None else float(scale)
-    if D != 64 and rope is not None:
-        raise ValueError("in-kernel rotary needs head dim 64")
+    if impl == "plain" and rope is not None:
+        raise ValueError("the plain kernel has no in-kernel rotary")
     if isinstance(pos, torch.Tensor):
         if pos.dtype != torch.int32 or not pos.is_cuda or pos.numel() < B or not pos.is_contiguous():
             raise ValueError("cache_seqlens must be a contiguous int32 device tensor with B entries")
         seq_ptr, pos_host = pos.data_ptr(), 0
-        cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, 1)
+        cos_ptr, sin_ptr, n_pos, rotary_dim, interleaved = _rope_tables(rope, q.device, 1, D)
     else:
         seq_ptr, pos_host = None, int(pos)
-        cos_ptr, sin_ptr, n_pos = _rope_tables(rope, q.device, pos_host + 1)
+        cos_ptr, sin_ptr, n_pos, rotary_dim, interleaved = _rope_tables(rope, q.device, pos_host + 1, D)
     if out is None:
         o = torch.empty(B, 1, H, D, dtype=q.dtype, device=q.device)
     else:
@@ -317,22 +332,24 @@ def swa_step(q, k_new, v_new, kv_cache, pos, w_left: int = 64, scale: Optional[f
     c_sb, c_st, _, c_sh, _ = kv_cache.stride()
     kc_ptr = kv_cache.data_ptr()
     vc_ptr = kc_ptr + kv_cache.stride(2) * kv_cache.element_size()
+    strides = (q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
+               v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2), c_sb, c_st, c_sh)
     with _on_device(q.device):
-        if D == 64:
+        if _swa_fast64(D, rotary_dim, interleaved, impl):
             _lib.check(_lib.lib().based_swa_step(
                 q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
-                seq_ptr, pos_host, B, H, kv_cache.shape[1],
-                q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
-                v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
-                c_sb, c_st, c_sh,
+                seq_ptr, pos_host, B, H, kv_cache.shape[1], *strides,
                 int(w_left), scale, cos_ptr, sin_ptr, n_pos, _dtype_code(q), _stream_ptr(q)))
-        else:
+        elif impl == "plain":
             _lib.check(_lib.lib().based_swa_step_anydim(
                 q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
-                seq_ptr, pos_host, B, H, D, kv_cache.shape[1],
-                q.stride(0), q.stride(2), k_new.stride(0), k_new.stride(2),
-                v_new.stride(0), v_new.stride(2), o.stride(0), o.stride(2),
-                c_sb, c_st, c_sh, int(w_left), scale, _dtype_code(q), _stream_ptr(q)))
+                seq_ptr, pos_host, B, H, D, kv_cache.shape[1], *strides, int(w_left), scale, _dtype_code(q),
+                _stream_ptr(q)))
+        else:
+            _lib.check(_lib.lib().based_swa_step_wide(
+                q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), kc_ptr, vc_ptr, o.data_ptr(),
+                seq_ptr, pos_host, B, H, D, kv_cache.shape[1], *strides, int(w_left), scale,
+                cos_ptr, sin_ptr, n_pos, rotary_dim, int(interleaved), _dtype_code(q), _stream_ptr(q)))
     return o
 
 

@@ -122,7 +122,7 @@ def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0):
     return e0.elapsed_time(e1) / steps, wall
 
 
-def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4):
+def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4, replays=12):
     """Recurrent decode step.  Timed twice: COLD over `n_sets` independent (kv_state, k_state) sets
     visited in turn (n_sets x 145 MB at B=128, dv=64: more than the 256 MB last-level cache, and what
     the linear-attention layers of a stack do per token: every layer has its own state), and WARM
@@ -175,31 +175,52 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
                 for _ in range(steps):
                     step()
         torch.cuda.current_stream().wait_stream(side)
-        return _events_ms(torch, graph.replay, 1, 2)[0] / steps
+        graph.replay()
+        graph.replay()
+        torch.cuda.synchronize()
+        # every replay timed by itself: the spread over `replays` samples is part of the result
+        samples = []
+        for _ in range(replays):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            samples.append(e0.elapsed_time(e1) / steps)
+        samples.sort()
+        return {"median": samples[len(samples) // 2], "min": samples[0], "max": samples[-1]}
 
     eager_cold, wall = _events_ms(torch, make_step(n_sets), steps, warmup)
     eager_warm, _ = _events_ms(torch, make_step(1), steps, warmup)
-    ms_cold, ms_warm = in_graph(n_sets), in_graph(1)
+    sp_cold, sp_warm = in_graph(n_sets), in_graph(1)
+    ms_cold, ms_warm = sp_cold["median"], sp_warm["median"]
     bytes_per_launch = B * H * (2 * D_EXP * dv * 4 + 2 * D_EXP * 4 + (2 * 16 + 2 * dv) * 2)
     ms = max(ms_cold, ms_warm)
     gbs = bytes_per_launch / (ms * 1e-3) / 1e9
+    spread = sp_cold if ms_cold >= ms_warm else sp_warm
+    frac_of = lambda t: round(bytes_per_launch / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
     assert torch.isfinite(y.float()).all() and all(torch.isfinite(a).all() for a, _ in states)
     return {
         "tok_s": B / (ms * 1e-3),
         "ms": ms,
         "wall_ms": wall,
-        "cold": {"ms": round(ms_cold, 5), "GBps": round(bytes_per_launch / (ms_cold * 1e-3) / 1e9, 1), "state_sets": n_sets,
+        "cold": {"ms": round(ms_cold, 5), "ms_min": round(sp_cold["min"], 5), "ms_max": round(sp_cold["max"], 5),
+                 "GBps": round(bytes_per_launch / (ms_cold * 1e-3) / 1e9, 1), "state_sets": n_sets,
                  "working_set_MB": round(n_sets * (kv_state.numel() + k_state.numel()) * 4 / 1e6, 1),
                  "launched_one_by_one_ms": round(eager_cold, 5)},
-        "warm": {"ms": round(ms_warm, 5), "GBps": round(bytes_per_launch / (ms_warm * 1e-3) / 1e9, 1), "state_sets": 1,
+        "warm": {"ms": round(ms_warm, 5), "ms_min": round(sp_warm["min"], 5), "ms_max": round(sp_warm["max"], 5),
+                 "GBps": round(bytes_per_launch / (ms_warm * 1e-3) / 1e9, 1), "state_sets": 1,
                  "working_set_MB": round((kv_state.numel() + k_state.numel()) * 4 / 1e6, 1),
                  "launched_one_by_one_ms": round(eager_warm, 5)},
         "roofline": {"kernel": "lin_step_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                     "frac_spread": {"replays": replays, "median": frac_of(spread["median"]),
+                                     "slowest": frac_of(spread["max"]), "fastest": frac_of(spread["min"])},
                      "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else None,
                      "algorithmic_bytes_per_launch": bytes_per_launch,
-                     "timed": "the slower of cold (rotating state sets) and warm (one set); the steps are recorded in "
-                              "one graph and one replay is timed (launched one by one: see decode_cold / decode_warm)"},
+                     "timed": "median over %d replays of a graph of the timed steps, the slower of cold (rotating state "
+                              "sets) and warm (one set); each replay timed by itself, spread in frac_spread (launched one "
+                              "by one: see decode_cold / decode_warm)" % replays},
         "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, "
                     f"bf16 q/k/v, {n_sets} independent state sets visited in turn",
     }

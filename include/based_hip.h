@@ -373,10 +373,52 @@ BASED_API int based_decode_linear(const void* x, int64_t x_row_stride, const int
                         const void* conv_weight, const void* conv_bias, int conv_k, void* stream);
 
 /*
+ * Sliding-window attention for head dimensions other than 64 and for every rotary shape of the
+ * reference's constructor, on the MFMA path: any head dim that is a multiple of 8 up to 128 (112
+ * and 128 are the released 1B / 1.3B models: n_embd 1792 / 2048 over 16 heads,
+ * train/configs/experiment/reference/based-1b.yaml:94-99), rotary over the first `rotary_dim`
+ * channels (a multiple of 16, at most D; slide_attention.py:346-355: RotaryEmbedding(rotary_emb_dim,
+ * interleaved=rotary_emb_interleaved)), half-split pairs (c, c + rotary_dim/2) or, with
+ * rotary_interleaved != 0, pairs (2i, 2i+1).  Replaces the same reference calls as
+ * based_swa_prefill / based_swa_step (flash_attn_qkvpacked_func / flash_attn_kvpacked_func after
+ * _update_kv_cache, slide_attention.py:59-106,150-213,255-281; flash_attn_with_kvcache with its
+ * rotary arguments, slide_attention.py:384-481) with the same argument meaning, plus:
+ *   D                      : head dim; rows of q, k, v, o and the cache hold D contiguous elements
+ *   rope_cos / rope_sin    : fp32 (rope_len, rotary_dim / 2), NULL for no rotary
+ *   rotary_dim, rotary_interleaved : as above (ignored without tables)
+ * All element strides multiples of 8, all tensors 16-byte aligned, 0 <= w_left <= 128, bf16.
+ * A device-side position outside the cache or the rotary table leaves the cache untouched and
+ * writes NaN to that (batch, head) output row.
+ */
+BASED_API int based_swa_prefill_wide(const void* q, const void* k, const void* v, void* o, int64_t B,
+                           int64_t H, int64_t L, int64_t D,
+                           int64_t q_sb, int64_t q_sl, int64_t q_sh,
+                           int64_t k_sb, int64_t k_sl, int64_t k_sh,
+                           int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                           int64_t o_sb, int64_t o_sl, int64_t o_sh,
+                           int w_left, float scale,
+                           const float* rope_cos, const float* rope_sin, int64_t rope_len,
+                           int64_t rotary_dim, int rotary_interleaved,
+                           void* kcache_out, void* vcache_out,
+                           int64_t c_sb, int64_t c_st, int64_t c_sh, int64_t max_seqlen,
+                           int io_dtype, void* stream);
+BASED_API int based_swa_step_wide(const void* q, const void* k_new, const void* v_new,
+                        void* kcache, void* vcache, void* o,
+                        const int32_t* cache_seqlens, int64_t pos_host,
+                        int64_t B, int64_t H, int64_t D, int64_t max_seqlen,
+                        int64_t q_sb, int64_t q_sh, int64_t kn_sb, int64_t kn_sh,
+                        int64_t vn_sb, int64_t vn_sh, int64_t o_sb, int64_t o_sh,
+                        int64_t c_sb, int64_t c_st, int64_t c_sh,
+                        int w_left, float scale,
+                        const float* rope_cos, const float* rope_sin, int64_t rope_len,
+                        int64_t rotary_dim, int rotary_interleaved,
+                        int io_dtype, void* stream);
+
+/*
  * The same sliding-window attention for head dimensions other than 64 (any multiple of 8 up to
- * 128), bf16, fp32 arithmetic, one wavefront per query: not a performance path, it exists so
- * that models with other head sizes (the reference's own test models have 16-dim heads,
- * based/tests/test_generation.py:7-34,69-80) run through the same module.  Same reference lines
+ * 128), bf16, fp32 arithmetic, one wavefront per query: not a performance path; a plain second
+ * statement of the same attention (the reference's own test models have 16-dim heads,
+ * based/tests/test_generation.py:7-34,69-80) that the tests hold the MFMA kernels against.  Same reference lines
  * and argument meaning as based_swa_prefill / based_swa_step, plus the head dimension D; no
  * in-kernel rotary (the caller rotates q and k first).
  */

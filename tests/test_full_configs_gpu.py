@@ -104,17 +104,20 @@ def test_config5_long_context_dv128(dev):
     y2, _, _ = ops.linear_attn_prefill(q, k, v2)
     y12, _, _ = ops.linear_attn_prefill(q, k, (v.float() + v2.float()).to(torch.bfloat16))
     assert rel_l2(y12.float(), y.float() + y2.float()) < 1.5e-2
-    # decode B=64 for 32 of the 512 steps from the tiled state (every batch row must agree)
+    # decode B=64 for all 512 steps of the configuration from the tiled state (every batch row must
+    # agree; the oracle follows two of the heads, its state carried in fp32 like the kernel's)
     Bd = 64
     kvd = kv.repeat(Bd, 1, 1, 1, 1).contiguous()
     ksd = ks.repeat(Bd, 1, 1, 1, 1).contiguous()
-    kv_o, ks_o = kv32[:, :2].cpu().clone(), ks32[:, :2].cpu().clone()
-    for t in range(32):
-        qs, kk, vv = _randn((1, H, 1, 16), 100 + t, dev), _randn((1, H, 1, 16), 200 + t, dev), _randn((1, H, 1, dv), 300 + t, dev)
+    kv_o, ks_o = kv[:, :2].cpu().clone(), ks[:, :2].cpu().clone()
+    for t in range(512):
+        qs, kk, vv = _randn((1, H, 1, 16), 1000 + t, dev), _randn((1, H, 1, 16), 2000 + t, dev), _randn((1, H, 1, dv), 3000 + t, dev)
         yd = ops.linear_attn_step(qs.expand(Bd, H, 1, 16), kk.expand(Bd, H, 1, 16), vv.expand(Bd, H, 1, dv), kvd, ksd)
         y_ref = O.linear_attn_step(kv_o, ks_o, qs[:, :2].float().cpu(), kk[:, :2].float().cpu(), vv[:, :2].float().cpu())
-        assert rel_l2(yd[:1, :2].float(), y_ref) < 1e-2
-        assert torch.equal(yd[0], yd[Bd - 1])
+        assert rel_l2(yd[:1, :2].float(), y_ref) < 1e-2, f"decode step {t}"
+        if t % 64 == 0 or t == 511:
+            assert torch.equal(yd[0], yd[Bd - 1])
+    assert rel_l2(kvd[:1, :2], kv_o) < 5e-3 and rel_l2(ksd[Bd - 1:, :2], ks_o) < 5e-3   # the states after 512 steps
 
 
 def test_config4_full_stack_generation(dev):

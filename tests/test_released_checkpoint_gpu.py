@@ -22,7 +22,7 @@ pytestmark = pytest.mark.gpu
 N_EMBD, N_HEAD, N_LAYER, VOCAB = 256, 4, 4, 1000
 
 
-def released_config():
+def released_config(N_EMBD=N_EMBD, N_HEAD=N_HEAD, N_LAYER=N_LAYER):
     return {
         "alt_mixer_layers": [1], "alt_mixer_2_layers": [2],
         "mixer": {"_target_": "based.models.mixers.convolution.BaseConv", "l_max": 2048, "use_bias": True,
@@ -59,7 +59,10 @@ def released_state_dict(cfg, seed=11):
             sd[p + "mixer.Wqkv.weight"], sd[p + "mixer.out_proj.weight"] = mat(3 * d, d), mat(d, d)
         elif i in cfg["alt_mixer_layers"]:
             h = cfg["alt_mixer"]["num_heads"]
-            sd[p + "mixer.proj_q.weight"], sd[p + "mixer.proj_k.weight"] = 8 * mat(16 * h, d), 8 * mat(16 * h, d)
+            # q, k entries of standard deviation 2.56 at any width (8 x 0.02 x sqrt(256)): scores of a few units
+            qk_gain = 8 * (256 / d) ** 0.5
+            sd[p + "mixer.proj_q.weight"] = (qk_gain * mat(16 * h, d).float()).bfloat16()
+            sd[p + "mixer.proj_k.weight"] = (qk_gain * mat(16 * h, d).float()).bfloat16()
             sd[p + "mixer.proj_v.weight"], sd[p + "mixer.out_proj.weight"] = mat(d, d), mat(d, d)
         else:
             d_inner = 4 * d // 2
@@ -75,7 +78,8 @@ def released_state_dict(cfg, seed=11):
 def _assert_reference_bound(got, want, what):
     got, want = got.float().cpu(), want.float().cpu()
     excess = (got - want).abs() - (5e-2 + 1e-2 * want.abs())
-    assert float(excess.max()) <= 0, f"{what}: a logit is {float(excess.max()):.3e} beyond atol 5e-2 / rtol 1e-2"
+    assert float(excess.max()) <= 0, (f"{what}: a logit is {float(excess.max()):.3e} beyond atol 5e-2 / rtol 1e-2 "
+                                      f"(max |diff| {float((got - want).abs().max()):.3e}, max |want| {float(want.abs().max()):.2f})")
 
 
 def test_released_layout_checkpoint_loads_and_generates(dev, tmp_path):
@@ -93,6 +97,7 @@ def test_released_layout_checkpoint_loads_and_generates(dev, tmp_path):
     swa = model.transformer.layers[2].mixer
     lin = model.transformer.layers[1].mixer
     assert isinstance(swa, SlidingAttention) and swa.window == (128, 0) and swa.rotary_emb_dim == 64
+    assert all(layer.supports_decode_step() for layer in model.transformer.layers)   # single-token steps take the fused path
     assert isinstance(lin, LinearAttention) and lin.eps == 1e-6     # the "fla" regulariser
     assert not hasattr(model.transformer.embeddings, "position_embeddings")
     for k, v in model.state_dict().items():
@@ -143,3 +148,67 @@ def test_released_360m_shape_builds_with_window_256(dev):
         for i in range(3):
             ref = model(out.sequences[:, : 300 + i]).logits[:, -1]
             _assert_reference_bound(out.scores[i], ref, f"cached step {i} vs parallel")
+
+
+def test_released_1b_shape_head_dim_112(dev, tmp_path):
+    """The released 1B / 1.3B shape (train/configs/experiment/reference/based-1b.yaml:72-125:
+    n_embd 1792 over 16 heads = head dim 112 for BOTH attention mixers, window_size 256, rotary over
+    the whole head, n_inner 2 x n_embd), narrow in depth and vocabulary: loaded from the released
+    layout, prefill and every cached step against the oracle composition at the reference's bound,
+    eagerly and through the recorded decode graph.  Head dim 112 must take the MFMA kernels and the
+    fused single-token path (no torch-side rotary, nothing that raises under device positions)."""
+    from based_amd.mixers.linear_attention import LinearAttention
+    from based_amd.mixers.slide_attention import SlidingAttention
+    from based_amd.stack import GPTLMHeadModel
+
+    cfg = released_config(N_EMBD=1792, N_HEAD=16, N_LAYER=4)
+    sd = released_state_dict(cfg, seed=19)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    torch.save({"model." + k: v for k, v in sd.items()}, tmp_path / "pytorch_model.bin")
+    print("1B-shape checkpoint: load", flush=True)
+    model = GPTLMHeadModel.from_pretrained_local(str(tmp_path), device=dev, dtype=torch.bfloat16).eval()
+    swa, lin = model.transformer.layers[2].mixer, model.transformer.layers[1].mixer
+    assert isinstance(swa, SlidingAttention) and swa.head_dim == 112 and swa.rotary_emb_dim == 112 and swa.window == (128, 0)
+    assert isinstance(lin, LinearAttention) and lin.head_dim == 112
+    assert all(layer.supports_decode_step() for layer in model.transformer.layers)
+
+    sd32 = {k: v.float() for k, v in sd.items()}
+    B, P, n_new = 2, 270, 6
+    ids = torch.randint(1, VOCAB, (B, P), generator=torch.Generator().manual_seed(5))
+
+    def check(got, seq, last_only, what):
+        """At this width the logits reach +-4.5, where one bf16 step is 0.03: the element-wise bound
+        of the reference's 256-wide test model is widened by what rounding alone does to the SAME
+        composition evaluated with bf16 activations on the CPU, and the GPU model must sit as close
+        to the fp32 statement as that composition does."""
+        exact = O.stack_forward(seq, sd32, cfg)
+        rounded = O.stack_forward(seq, sd32, cfg, dtype=torch.bfloat16).float()
+        if last_only:
+            exact, rounded = exact[:, -1], rounded[:, -1]
+        got = got.float().cpu()
+        noise = float((rounded - exact).abs().max())
+        excess = (got - exact).abs() - (5e-2 + 1e-2 * exact.abs() + noise)
+        e_gpu = float((got - exact).norm() / exact.norm())
+        e_cpu = float((rounded - exact).norm() / exact.norm())
+        print(f"{what}: rel-L2 to the fp32 statement GPU {e_gpu:.4f} / CPU bf16 composition {e_cpu:.4f}; "
+              f"max |diff| GPU {float((got - exact).abs().max()):.4f} / CPU {noise:.4f}", flush=True)
+        assert float(excess.max()) <= 0, f"{what}: a logit is {float(excess.max()):.3e} beyond the bound"
+        assert e_gpu < 1.5 * e_cpu + 2e-3, f"{what}: rel-L2 {e_gpu:.4f} against {e_cpu:.4f} from rounding alone"
+
+    print("1B-shape checkpoint: prefill", flush=True)
+    with torch.inference_mode():
+        logits = model(ids.to(dev)).logits
+    check(logits, ids, False, "prefill logits")
+    print("1B-shape checkpoint: generate", flush=True)
+    out = model.generate(input_ids=ids.to(dev), max_length=P + n_new, return_dict_in_generate=True, output_scores=True,
+                         top_k=1)
+    seqs = out.sequences.cpu()
+    for i, sc in enumerate(out.scores):
+        check(sc, seqs[:, : P + i], True, f"cached decode step {i}")
+    print("1B-shape checkpoint: graph decode", flush=True)
+    graphed = model.generate(input_ids=ids.to(dev), max_length=P + n_new, return_dict_in_generate=True,
+                             output_scores=True, top_k=1, cg=True)
+    assert torch.equal(graphed.sequences.cpu(), seqs)
+    for i, (a, b) in enumerate(zip(graphed.scores, out.scores)):
+        err = float((a.float() - b.float()).norm() / b.float().norm())
+        assert err < 1e-3, f"graph step {i}: rel-L2 {err:.2e} against eager"

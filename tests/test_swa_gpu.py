@@ -106,7 +106,7 @@ def test_rejects(dev):
         ops.swa_prefill(x, x, x)  # head dim 12 (not a multiple of 8)
     x = torch.zeros(1, 4, 2, 32, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
-        ops.swa_prefill(x, x, x, rope=_rope_tables(4, dev))  # in-kernel rotary is for head dim 64
+        ops.swa_prefill(x, x, x, rope=_rope_tables(4, dev))  # 64 rotated channels do not fit a head of 32
     y = torch.zeros(1, 4, 2, 64, device=dev, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         ops.swa_prefill(y, y, y, w_left=129)
@@ -187,14 +187,19 @@ def _qkv_d(B, L, H, D, seed):
     return torch.randn(B, L, 3, H, D, generator=g).bfloat16()
 
 
+@pytest.mark.parametrize("impl", [None, "plain"])
 @pytest.mark.parametrize("B,L,H,D,w", [(2, 200, 3, 16, 64), (1, 300, 2, 32, 128), (1, 70, 2, 128, 17), (1, 1, 1, 8, 64),
-                                       (2, 130, 4, 16, 0), (1, 257, 2, 96, 100)])
-def test_other_head_dims_prefill_and_cache(dev, B, L, H, D, w):
-    """Head dims other than 64 (the reference's test models have 16): the plain kernel against the oracle,
-    with and without the cache output."""
-    from based_amd import ops
+                                       (2, 130, 4, 16, 0), (1, 257, 2, 96, 100), (2, 300, 3, 112, 128), (1, 1000, 16, 112, 128),
+                                       (1, 129, 2, 128, 128), (1, 500, 2, 72, 64), (1, 333, 2, 112, 64)])
+def test_other_head_dims_prefill_and_cache(dev, B, L, H, D, w, impl):
+    """Head dims other than 64 (112 and 128: the released 1B / 1.3B models; 16: the reference's test
+    models): the general MFMA kernel and the plain kernel against the oracle, with and without the
+    cache output."""
+    from based_amd import ops as ops_mod
+    from types import SimpleNamespace
 
-    print(f"swa any-dim prefill case B={B} L={L} H={H} D={D} w={w}", flush=True)
+    ops = SimpleNamespace(swa_prefill=lambda *a, **kw: ops_mod.swa_prefill(*a, impl=impl, **kw))
+    print(f"swa any-dim prefill case B={B} L={L} H={H} D={D} w={w} impl={impl}", flush=True)
     qkv = _qkv_d(B, L, H, D, seed=23)
     ref = O.sliding_window_attn(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=w)
     qd = qkv.to(dev)
@@ -205,10 +210,15 @@ def test_other_head_dims_prefill_and_cache(dev, B, L, H, D, w):
     assert torch.equal(out, ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w))
 
 
-@pytest.mark.parametrize("D,P,T,w", [(16, 0, 70, 64), (16, 100, 40, 128), (32, 60, 10, 65), (128, 10, 6, 7)])
-def test_other_head_dims_decode(dev, D, P, T, w):
-    from based_amd import ops
+@pytest.mark.parametrize("impl", [None, "plain"])
+@pytest.mark.parametrize("D,P,T,w", [(16, 0, 70, 64), (16, 100, 40, 128), (32, 60, 10, 65), (128, 10, 6, 7),
+                                     (112, 0, 140, 128), (112, 200, 6, 128), (128, 70, 5, 64), (72, 3, 70, 64)])
+def test_other_head_dims_decode(dev, D, P, T, w, impl):
+    from based_amd import ops as ops_mod
+    from types import SimpleNamespace
 
+    ops = SimpleNamespace(swa_prefill=lambda *a, **kw: ops_mod.swa_prefill(*a, impl=impl, **kw),
+                          swa_step=lambda *a, **kw: ops_mod.swa_step(*a, impl=impl, **kw))
     B, H = 2, 3
     L = P + T
     qkv = _qkv_d(B, L, H, D, seed=29)
@@ -243,3 +253,111 @@ def test_plain_kernel_agrees_with_mfma_kernel_at_head_dim_64(dev):
         k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2), slow.stride(0), slow.stride(1),
         slow.stride(2), w, 0.125, None, None, 0, 0, 0, 0, _lib.BASED_BF16, stream))
     assert rel_l2(fast.float(), slow.float()) < 4e-3
+
+
+def _rope_tables_d(n_pos, rotary_dim, dev, interleaved=False, base=10000.0):
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    ang = torch.outer(torch.arange(n_pos).float(), inv_freq)
+    return ang.cos().contiguous().to(dev), ang.sin().contiguous().to(dev), interleaved
+
+
+@pytest.mark.parametrize("D,R,inter", [(112, 112, False), (128, 128, False), (112, 112, True), (128, 64, False),
+                                       (112, 48, True), (64, 32, False), (64, 64, True), (64, 16, True),
+                                       (32, 32, False), (96, 80, False)])
+@pytest.mark.parametrize("B,L,H,w", [(2, 300, 3, 128), (1, 130, 2, 64)])
+def test_wide_prefill_rotary_layouts_and_cache(dev, D, R, inter, B, L, H, w):
+    """The rotary shapes of the reference's constructor (rotary_emb_dim a multiple of 16 up to the
+    head dim, half-split or interleaved pairs; slide_attention.py:346-355) inside the general
+    kernel == rotating q and k first with the oracle; the cache receives the rotated k and v."""
+    from based_amd import ops
+
+    print(f"swa wide rotary case D={D} R={R} interleaved={inter} B={B} L={L} H={H} w={w}", flush=True)
+    qkv = _qkv_d(B, L, H, D, seed=37)
+    pos = torch.arange(L)
+    q_r = O.rotary_embedding(qkv[:, :, 0], pos, rotary_dim=R, interleaved=inter)
+    k_r = O.rotary_embedding(qkv[:, :, 1], pos, rotary_dim=R, interleaved=inter)
+    ref = O.sliding_window_attn(q_r, k_r, qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    rope = _rope_tables_d(L + 3, R, dev, inter)
+    cache = torch.full((B, L + 2, 2, H, D), 3.0, dtype=torch.bfloat16, device=dev)
+    out = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, rope=rope, kv_cache=cache)
+    torch.cuda.synchronize()
+    assert rel_l2(out.float(), ref.float()) < TOL
+    c = cache.cpu()
+    assert torch.equal(c[:, :L, 1], qkv[:, :, 2])
+    assert rel_l2(c[:, :L, 0].float(), k_r.float()) < 3e-3
+    assert torch.equal(c[:, :L, 0][..., R:], qkv[:, :, 1][..., R:])   # channels past rotary_dim pass through
+    assert bool((c[:, L:] == 3.0).all())
+
+
+@pytest.mark.parametrize("D,R,inter,P,T,w", [(112, 112, False, 0, 140, 128), (112, 112, False, 200, 8, 128),
+                                             (128, 128, False, 70, 6, 64), (112, 64, True, 50, 20, 128),
+                                             (64, 32, False, 10, 10, 7), (64, 64, True, 100, 40, 128)])
+def test_wide_decode_rotary_matches_parallel(dev, D, R, inter, P, T, w):
+    """Prefill P tokens into the cache with in-kernel rotary, then rotary decode steps (host and
+    device positions) through the general kernels: every step equals the parallel oracle."""
+    from based_amd import ops
+
+    B, H = 2, 3
+    L = P + T
+    qkv = _qkv_d(B, L, H, D, seed=41)
+    pos = torch.arange(L)
+    q_r = O.rotary_embedding(qkv[:, :, 0], pos, rotary_dim=R, interleaved=inter)
+    k_r = O.rotary_embedding(qkv[:, :, 1], pos, rotary_dim=R, interleaved=inter)
+    ref = O.sliding_window_attn(q_r, k_r, qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    rope = _rope_tables_d(L, R, dev, inter)
+    cache = torch.zeros(B, L, 2, H, D, dtype=torch.bfloat16, device=dev)
+    if P > 0:
+        o0 = ops.swa_prefill(qd[:, :P, 0], qd[:, :P, 1], qd[:, :P, 2], w_left=w, rope=rope, kv_cache=cache)
+        assert rel_l2(o0.float(), ref[:, :P].float()) < TOL
+    for t in range(P, L):
+        print(f"swa wide rotary step case D={D} R={R} P={P} w={w} pos={t}", flush=True)
+        p = t if t % 2 == 0 else torch.full((B,), t, dtype=torch.int32, device=dev)
+        o = ops.swa_step(qd[:, t:t + 1, 0], qd[:, t:t + 1, 1], qd[:, t:t + 1, 2], cache, p, w_left=w, rope=rope)
+        assert rel_l2(o.float(), ref[:, t:t + 1].float()) < TOL
+    assert rel_l2(cache[:, :, 0].float(), k_r.float()) < 3e-3
+    assert torch.equal(cache[:, :, 1].cpu(), qkv[:, :, 2])
+    bad = ops.swa_step(qd[:, :1, 0], qd[:, :1, 1], qd[:, :1, 2], cache, torch.full((B,), L, dtype=torch.int32, device=dev),
+                       w_left=w, rope=rope)
+    assert bool(torch.isnan(bad.float()).all())        # device-side position outside the cache
+
+
+def test_wide_kernel_agrees_with_64_channel_kernel(dev):
+    """At head dim 64 with whole-head half-split rotary both MFMA kernels apply; they agree to bf16
+    noise on outputs and cache, prefill and step."""
+    from based_amd import ops
+
+    B, L, H, w = 2, 333, 4, 128
+    qkv = _qkv(B, L + 1, H, seed=43).to(dev)
+    rope = _rope_tables_d(L + 1, 64, dev)
+    q, k, v = qkv[:, :L, 0], qkv[:, :L, 1], qkv[:, :L, 2]
+    c1 = torch.zeros(B, L + 1, 2, H, 64, dtype=torch.bfloat16, device=dev)
+    c2 = torch.zeros_like(c1)
+    fast = ops.swa_prefill(q, k, v, w_left=w, rope=rope, kv_cache=c1)
+    wide = ops.swa_prefill(q, k, v, w_left=w, rope=rope, kv_cache=c2, impl="wide")
+    assert rel_l2(wide.float(), fast.float()) < 4e-3 and rel_l2(c2.float(), c1.float()) < 1e-3
+    s1 = ops.swa_step(qkv[:, L:, 0], qkv[:, L:, 1], qkv[:, L:, 2], c1, L, w_left=w, rope=rope)
+    s2 = ops.swa_step(qkv[:, L:, 0], qkv[:, L:, 1], qkv[:, L:, 2], c2, L, w_left=w, rope=rope, impl="wide")
+    assert rel_l2(s2.float(), s1.float()) < 4e-3
+
+
+@pytest.mark.parametrize("w", [0, 1, 64, 65, 127, 128])
+def test_wide_window_edges_are_exact(dev, w):
+    """The q = 0 mean test of the window edges on the general kernel (head dim 112)."""
+    from based_amd import ops
+
+    B, L, H, D = 1, 400, 2, 112
+    qkv = _qkv_d(B, L, H, D, seed=47)
+    qkv[:, :, 0] = 0
+    v = qkv[:, :, 2].float()
+    ref = torch.stack([v[:, max(0, i - w): i + 1].mean(dim=1) for i in range(L)], dim=1)
+    qd = qkv.to(dev)
+    out = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w)
+    assert rel_l2(out.float(), ref) < 3e-3
+    cache = torch.zeros(B, L, 2, H, D, dtype=torch.bfloat16, device=dev)
+    cache[:, :, 0] = qd[:, :, 1]
+    cache[:, :, 1] = qd[:, :, 2]
+    for t in sorted({0, 1, max(w - 1, 0), w, w + 1, w + 2, 2 * w + 1, L - 1}):
+        o = ops.swa_step(qd[:, t:t + 1, 0], qd[:, t:t + 1, 1], qd[:, t:t + 1, 2], cache, t, w_left=w)
+        assert rel_l2(o.float(), ref[:, t:t + 1]) < 3e-3, f"step at {t}"
