@@ -194,14 +194,17 @@ __device__ __forceinline__ void interleave() {
       long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh, long v_sl, long y_sb,  \
       long y_sh, long y_sl, float eps, float *__restrict__ ws, int seg_tokens, int n_seg
 
-// chain number of this workgroup.  Workgroups are dealt to the 8 XCDs round-robin by workgroup
-// id.  Chains whose q/k rows share cache lines (neighbouring heads of one batch entry: 32-byte
-// rows, 512 bytes apart) should sit behind the same L2, so consecutive chain numbers are laid
-// along one XCD: chain = (id mod 8) * ceil(n / 8) + id / 8 when that stays in range.
-__device__ __forceinline__ long chain_of_block() {
-  const long n_chain = gridDim.x;
-  const long per_xcd = (n_chain + 7) / 8;
-  if (n_chain % 8 != 0) return blockIdx.x;  // irregular grids keep the identity mapping
+// Work item of this workgroup: item = (batch * H + head) * n_blocks + channel block, n_blocks =
+// ceil(dv / 64).  Workgroups are dealt to the 8 XCDs round-robin by workgroup id.  Items whose rows
+// share cache lines (the channel blocks of one head read the same q and k rows, and for head dims
+// that are no multiple of 64 their v and y rows meet inside 128-byte lines; neighbouring heads of
+// one batch entry: 32-byte q / k rows 512 bytes apart) should sit behind the same L2 at about the
+// same time, so consecutive items are laid along one XCD: item = (id mod 8) * ceil(n / 8) + id / 8
+// when that stays in range.
+__device__ __forceinline__ long item_of_block() {
+  const long n_item = gridDim.x;
+  const long per_xcd = (n_item + 7) / 8;
+  if (n_item % 8 != 0) return blockIdx.x;  // irregular grids keep the identity mapping
   return (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
 }
 
@@ -254,8 +257,10 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
   const int lane = threadIdx.x & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
-  const long bh = chain_of_block();
-  const int eb = blockIdx.y;  // 64-channel block of the value dimension
+  const int n_eb = (dv + 63) >> 6;
+  const long item = item_of_block();
+  const long bh = item / n_eb;
+  const int eb = (int)(item % n_eb);  // 64-channel block of the value dimension
   const int live_ch = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // channels of this block that exist (a multiple of 16)
   const int b = (int)(bh / H), h = (int)(bh % H);
   y += b * y_sb + h * y_sh + 64 * eb;
@@ -476,8 +481,10 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   const int lane = tid & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
-  const long bh = chain_of_block();
-  const int eb = blockIdx.y;  // 64-channel block of the value dimension
+  const int n_eb = (dv + 63) >> 6;
+  const long item = item_of_block();
+  const long bh = item / n_eb;
+  const int eb = (int)(item % n_eb);  // 64-channel block of the value dimension
   const int live_ch = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // channels of this block that exist (a multiple of 16)
   const int b = (int)(bh / H), h = (int)(bh % H);
   q += b * q_sb + h * q_sh;
@@ -506,7 +513,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   const bool last_seg = MODE == kModeFull || seg == n_seg - 1;
   float* ws_mine = nullptr;
   if constexpr (MODE != kModeFull)
-    ws_mine = ws + (((long)bh * gridDim.y + eb) * n_seg + seg) * (long)kSegStateFloats;
+    ws_mine = ws + (item * n_seg + seg) * (long)kSegStateFloats;
   if constexpr (MODE == kModeFrom) {
 #pragma unroll
     for (int i = 0; i < kOwn; ++i)
@@ -1007,7 +1014,8 @@ extern "C" BASED_API int based_linear_attn_prefill(
                     "linear_attn_prefill: bf16 strides must be multiples of 8 elements (16 bytes)");
     BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
                   "linear_attn_prefill: tensors must be 16-byte aligned");
-    dim3 grid((unsigned)(B * H), (unsigned)((dv + 63) / 64)), block(kThreads);
+    BASED_REQUIRE(B * H * ((dv + 63) / 64) < (1ll << 31), BASED_ERR_SHAPE, "linear_attn_prefill: sizes too large");
+    dim3 grid((unsigned)(B * H * ((dv + 63) / 64))), block(kThreads);
     hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFull>, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
                        q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, (float*)nullptr, 0, 1);
@@ -1088,6 +1096,7 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
                 "%s: segment count %ld leaves empty segments (use the plan)", who, (long)n_seg);
   const int64_t eblocks = (dv + 63) / 64;
   const int64_t chains = B * H * eblocks;
+  BASED_REQUIRE(chains < (1ll << 31), BASED_ERR_SHAPE, "%s: sizes too large", who);
   const int64_t need = chains * n_seg * (int64_t)kSegStateFloats * 4;
   if (workspace_limit >= 0)
     BASED_REQUIRE(need <= workspace_limit, BASED_ERR_SHAPE,
@@ -1105,7 +1114,7 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   const int seg_tokens = (int)(seg_chunks * kChunk);
   dim3 block(kThreads);
   // pass 1: every segment but the last accumulates its own contribution to the state
-  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)(B * H), (unsigned)eblocks, (unsigned)(n_seg - 1)),
+  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)chains, 1, (unsigned)(n_seg - 1)),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
@@ -1121,7 +1130,7 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
     rc = check_launch(who);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(fold ? lin_prefill_mfma_kernel<kModeFromSum> : lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)(B * H), (unsigned)eblocks, (unsigned)n_seg),
+  hipLaunchKernelGGL(fold ? lin_prefill_mfma_kernel<kModeFromSum> : lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)chains, 1, (unsigned)n_seg),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);

@@ -106,12 +106,21 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
   const int np = D >> 3;            // live 16-byte pieces of a row
   const int n_ds = (D + 31) >> 5;   // contraction steps of 32 channels
   const int n_et = (D + 15) >> 4;   // output channel tiles of 16
+  const bool whole_lines = (D & 63) == 0 && (o_sh & 63) == 0 && (o_sl & 63) == 0;
 
-  // work item: a run of consecutive query tiles of one (batch, head); the runs of a head are neighbours
+  // Work item: a run of consecutive query tiles of one (batch, head).  The heads of one run of
+  // tokens are consecutive items and consecutive items are laid along one XCD (workgroup ids are
+  // dealt to the 8 XCDs round-robin): a token's rows of all heads are one contiguous piece of
+  // memory, and head rows of 224 bytes (head dim 112) start and end inside 128-byte lines that
+  // two neighbouring heads share; the neighbours then read and write those lines behind the same
+  // L2 at about the same time (measured with a streaming probe: 128-byte accesses into 224-byte
+  // head rows from unrelated workgroups run at 2.4 TB/s, half the rate of aligned rows).
   const int runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
-  const int run = (int)(blockIdx.x % (unsigned)runs_per_seq);
-  const unsigned bh = blockIdx.x / (unsigned)runs_per_seq;
-  const int h = (int)(bh % (unsigned)H), b = (int)(bh / (unsigned)H);
+  const unsigned n_item = gridDim.x;
+  const unsigned item = n_item % 8 == 0 ? (blockIdx.x % 8) * (n_item / 8) + blockIdx.x / 8 : blockIdx.x;
+  const int h = (int)(item % (unsigned)H);
+  const unsigned rest = item / (unsigned)H;
+  const int run = (int)(rest % (unsigned)runs_per_seq), b = (int)(rest / (unsigned)runs_per_seq);
   const int tile_begin = run * run_tiles;
   const int tile_end = tile_begin + run_tiles < n_tiles ? tile_begin + run_tiles : n_tiles;
 
@@ -359,8 +368,13 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
       const int row = 4 * it + (lane >> 4);
       const int piece = lane & 15;
       const u32x4 w4 = *reinterpret_cast<const u32x4*>(q_rows + row * kWRowBytes + (wide_swz_k(row, piece) << 4));
-      if (n0 + row < L && piece < np)
-        __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(o_my + (long)(n0 + row) * o_sl + 8 * piece));
+      if (n0 + row < L && piece < np) {
+        // head rows that end inside a cache line are completed by the neighbouring head's workgroup:
+        // such lines should meet in the L2 (plain store); whole lines stream past it
+        u32x4* dst = reinterpret_cast<u32x4*>(o_my + (long)(n0 + row) * o_sl + 8 * piece);
+        if (whole_lines) __builtin_nontemporal_store(w4, dst);
+        else *dst = w4;
+      }
     }
 
     // ---- the oldest block (and the query rows) take the next tile's rows ----

@@ -86,7 +86,8 @@ def probes():
         lib.bench_probe_stream_qkv.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.c_void_p]
         lib.bench_probe_rmw.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
         lib.bench_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
-        for fn in (lib.bench_probe_stream_qkv, lib.bench_probe_rmw, lib.bench_probe_copy):
+        lib.bench_probe_stream_prefill.argtypes = [C.c_void_p] * 4 + [C.c_int64] * 3 + [C.c_void_p]
+        for fn in (lib.bench_probe_stream_qkv, lib.bench_probe_rmw, lib.bench_probe_copy, lib.bench_probe_stream_prefill):
             fn.restype = C.c_int
         _probes = lib
     return _probes
@@ -354,6 +355,31 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     ms_w128_warm, _ = _events_ms(torch, make_rel(1, False), steps, warmup)
     ms_rel_cold, _ = _events_ms(torch, make_rel(n_sets, True), steps, warmup)
     del caches
+    # the released 1B / 1.3B window layer: head dim 112 (n_embd 1792 over 16 heads), 128 keys to the left,
+    # rotary over the whole head, KV cache filled; the general MFMA kernel
+    D1 = 112
+    x1 = [torch.randn(B, L, 3, H, D1, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
+    o1b = [torch.empty(B, L, H, D1, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+    c1b = [torch.empty(B, L, 2, H, D1, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
+    inv1 = 1.0 / (10000.0 ** (torch.arange(0, D1, 2, dtype=torch.float32) / D1))
+    ang1 = torch.outer(torch.arange(L).float(), inv1)
+    rope1 = (ang1.cos().contiguous().to(dev), ang1.sin().contiguous().to(dev))
+
+    def make_1b(full):
+        def pf():
+            i = it[0] % n_sets
+            it[0] += 1
+            x = x1[i]
+            if full:
+                ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=128, rope=rope1, kv_cache=c1b[i], out=o1b[i])
+            else:
+                ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=128, out=o1b[i])
+        return pf
+
+    ms_1b_plain, _ = _events_ms(torch, make_1b(False), steps, warmup)
+    ms_1b_full, _ = _events_ms(torch, make_1b(True), steps, warmup)
+    byts_1b = B * L * H * 4 * D1 * 2
+    del x1, o1b, c1b
     cache = torch.zeros(B, L + decode_steps, 2, H, 64, dtype=torch.bfloat16, device=dev)
     cache[:, :L] = qkv[:, :, 1:]
     qn = torch.randn(B, 1, 3, H, 64, generator=g).bfloat16().to(dev)
@@ -375,6 +401,13 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
                        "cold_GBps": round(byts / (ms_w128_cold * 1e-3) / 1e9, 1),
                        "with_rotary_and_cache_fill_cold_ms": round(ms_rel_cold, 5),
                        "note": "same inputs, 128 keys to the left (the released checkpoints' window_size 256)"},
+        "head_dim_112": {"kernel": "swa_prefill_wide_kernel", "B": B, "L": L, "H": H, "window_left": 128,
+                         "cold_ms": round(ms_1b_plain, 5), "cold_GBps": round(byts_1b / (ms_1b_plain * 1e-3) / 1e9, 1),
+                         "frac_of_hbm_peak": round(byts_1b / (ms_1b_plain * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                         "with_rotary_and_cache_fill_cold_ms": round(ms_1b_full, 5),
+                         "with_rotary_and_cache_fill_GBps": round(byts_1b * 1.5 / (ms_1b_full * 1e-3) / 1e9, 1),
+                         "note": "the released 1B / 1.3B window layer (based-1b.yaml: n_embd 1792, 16 heads); bytes = q, k, v "
+                                 "read + o written (+ k, v written to the cache: x 1.5)"},
         "roofline": {"kernel": "swa_prefill_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["swa_prefill_kernel"], "algorithmic_bytes_per_launch": byts,
@@ -424,6 +457,18 @@ def bench_machine(torch, steps=20, warmup=4, n_sets=4):
 
         ms, _ = _events_ms(torch, st, steps, warmup)
         out[f"stream_qkv_cold_GBps_{g}_heads"] = round(B * L * H * 512 / (ms * 1e-3) / 1e9, 1)
+    del xs, os_
+    # memory side of the linear-attention prefill (B=96, H=16, L=4096, dv=64: 2.01 GB per launch, cold by size)
+    B, H, L = 96, 16, 4096
+    q = torch.ones(B, L, H * 16, dtype=torch.bfloat16, device=dev)
+    k = torch.ones(B, L, H * 16, dtype=torch.bfloat16, device=dev)
+    v = torch.ones(B, L, H * 64, dtype=torch.bfloat16, device=dev)
+    y = torch.empty(B, L, H * 64, dtype=torch.bfloat16, device=dev)
+    ms, _ = _events_ms(torch, lambda: _probe_ok(lib.bench_probe_stream_prefill(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                                                   y.data_ptr(), B, H, L, stream)), steps, warmup)
+    out["stream_prefill_B96_ms"] = round(ms, 4)
+    out["stream_prefill_B96_GBps"] = round(B * L * H * 320 / (ms * 1e-3) / 1e9, 1)
+    del q, k, v, y
     out["note"] = ("probe kernels of bench_probes.hip over %d rotating buffer sets; GB/s of bytes read + written" % n_sets)
     return out
 
@@ -708,6 +753,8 @@ def main():
             out["decode_deferred"] = bench_decode_deferred(torch, ops)
     if args.only in (None, "prefill"):
         pre = [bench_prefill(torch, ops, 30, 3, B=b) for b in sorted({int(x) for x in args.prefill_batches.split(',')})]
+        if args.only is None or args.prefill_batches == "1,8,32,96":
+            pre.append(bench_prefill(torch, ops, 30, 3, B=32, dv=112))   # the released 1B / 1.3B head dim
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
     if args.only in (None, "prefill"):
         # configs[4]: one 32K-token sequence at head dim 128, and its decode batch of 64
@@ -745,7 +792,7 @@ def main():
                     "ms_per_step": out["stack"]["decode_graph_ms_per_token"], "dtype": "bf16",
                     "config": {"workload": "configs[3]: 27-layer stack, B=4, prefill 2048 + 128 greedy tokens (decode graph)"}})
     if args.only == "prefill":
-        p = out["prefill"][-1]
+        p = [x for x in out["prefill"] if x["dv"] == 64][-1]
         out.update({"value": round(p["tok_s"], 1), "ms_per_step": p["ms"], "dtype": "bf16",
                     "config": {"workload": f"linear-attn prefill B={p['B']} L={p['L']} dv={p['dv']}"}, "roofline": p["roofline"]})
     if args.only == "swa":

@@ -9,6 +9,8 @@
 //                state update of the recurrent decode step.
 //   copy       : plain 16-byte-per-lane copy of known size; the calibration kernel for the
 //                profiler's HBM byte counters.
+//   stream_prefill : the q / k / v reads and y writes of the chunked linear-attention prefill, chunk
+//                by chunk per (batch, head), with no arithmetic: the memory ceiling of that kernel.
 //
 // Every entry point returns 0, or 1 for arguments it does not take.
 #include <hip/hip_runtime.h>
@@ -77,6 +79,48 @@ __global__ __launch_bounds__(256) void probe_rw_kernel(u32x4* dst, const u32x4* 
   }
 }
 
+// stream_prefill: the memory side of the chunked linear-attention prefill with nothing else: one
+// workgroup of 512 threads per (batch, head) walks the sequence in chunks of 64 tokens, fetching the
+// chunk's q and k rows (32 bytes each), v rows (128 bytes) two chunks ahead and storing a y row
+// (128 bytes) per token, in the (B, L, H*d) layout of the projections; 80,000 bytes of LDS are
+// requested so that two workgroups share a compute unit as in the real kernel, and workgroup
+// numbers are laid along the XCDs the same way.
+__global__ __launch_bounds__(512, 4) void probe_stream_prefill_kernel(const u32x4* __restrict__ q, const u32x4* __restrict__ k,
+                                                                       const u32x4* __restrict__ v, u32x4* __restrict__ y,
+                                                                       int H, int L) {
+  extern __shared__ unsigned char probe_lds[];
+  const int t = threadIdx.x;
+  const long n = gridDim.x;
+  const long bh = (n % 8 == 0) ? (blockIdx.x % 8) * (n / 8) + blockIdx.x / 8 : blockIdx.x;
+  const long b = bh / H, h = bh % H;
+  // 16-byte pieces: a token row of q / k holds 2 H, of v / y 8 H
+  const u32x4* qb = q + (b * L * H + h) * 2;
+  const u32x4* kb = k + (b * L * H + h) * 2;
+  const u32x4* vb = v + (b * L * H + h) * 8;
+  u32x4* yb = y + (b * L * H + h) * 8;
+  const int qrow = (t & 127) >> 1, qpc = t & 1;   // threads 0..127 fetch q, 128..255 k
+  const int vrow = t >> 3, vpc = t & 7;
+  const int chunks = L / 64;
+  u32x4 a[3], c[3];
+  auto fetch = [&](int ch, int slot) {
+    const long tq = (long)ch * 64 + qrow, tv = (long)ch * 64 + vrow;
+    a[slot] = t < 256 ? (t < 128 ? qb : kb)[tq * H * 2 + qpc] : u32x4{0, 0, 0, 0};   // 256 threads cover q and k
+    c[slot] = vb[tv * H * 8 + vpc];
+  };
+  if (chunks > 0) fetch(0, 0);
+  if (chunks > 1) fetch(1, 1);
+  for (int ch = 0; ch < chunks; ch += 3) {
+#pragma unroll
+    for (int u = 0; u < 3; ++u) {
+      if (ch + u < chunks) {
+        if (ch + u + 2 < chunks) fetch(ch + u + 2, (u + 2) % 3);
+        __builtin_nontemporal_store(a[u] ^ c[u], yb + ((long)(ch + u) * 64 + vrow) * H * 8 + vpc);
+      }
+    }
+  }
+  if (t == 0 && probe_lds[0] == 123 && L < 0) yb[0] = u32x4{0, 0, 0, 0};  // keeps the LDS request alive
+}
+
 static bool probe_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace bench_probes
@@ -118,5 +162,21 @@ PROBE_API int bench_probe_copy(void* dst, const void* src, int64_t bytes, void* 
   PROBE_REQUIRE(probe_aligned16(dst) && probe_aligned16(src));
   hipLaunchKernelGGL(probe_rw_kernel<true>, dim3(256 * 8), dim3(256), 0, static_cast<hipStream_t>(stream),
                      (u32x4*)dst, (const u32x4*)src, (size_t)(bytes / 16));
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+PROBE_API int bench_probe_stream_prefill(const void* q, const void* k, const void* v, void* y, int64_t B, int64_t H,
+                                         int64_t L, void* stream) {
+  using namespace bench_probes;
+  PROBE_REQUIRE(q && k && v && y && B > 0 && H > 0 && L > 0 && L % 64 == 0 && B * H < (1ll << 31) && L < (1ll << 30));
+  PROBE_REQUIRE(probe_aligned16(q) && probe_aligned16(k) && probe_aligned16(v) && probe_aligned16(y));
+  static bool allowed = false;
+  if (!allowed) {
+    PROBE_REQUIRE(hipFuncSetAttribute(reinterpret_cast<const void*>(probe_stream_prefill_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 80000) == hipSuccess);
+    allowed = true;
+  }
+  hipLaunchKernelGGL(probe_stream_prefill_kernel, dim3((unsigned)(B * H)), dim3(512), 80000, static_cast<hipStream_t>(stream),
+                     (const u32x4*)q, (const u32x4*)k, (const u32x4*)v, (u32x4*)y, (int)H, (int)L);
   return hipGetLastError() == hipSuccess ? 0 : 2;
 }

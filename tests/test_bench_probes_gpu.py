@@ -33,3 +33,29 @@ def test_rmw_and_copy_probes(dev):
     assert torch.equal(a, b)
     assert lib.bench_probe_rmw(a.data_ptr(), 24, stream) == 1        # not a multiple of 16: refused
     assert lib.bench_probe_stream_qkv(a.data_ptr(), b.data_ptr(), 1, 6, 8, 4, stream) == 1   # H % group: refused
+
+
+def test_stream_prefill_probe_moves_what_it_says(dev):
+    """The prefill memory probe reads every q, k, v row of its (batch, head) and writes every y row:
+    y piece (token 64 c + t / 8, piece t % 8) = v piece ^ the q or k piece thread t < 256 fetched."""
+    import bench
+
+    B, H, L = 2, 8, 256
+    q = torch.randint(-2**15, 2**15, (B, L, H, 16), dtype=torch.int16, device=dev)
+    k = torch.randint(-2**15, 2**15, (B, L, H, 16), dtype=torch.int16, device=dev)
+    v = torch.randint(-2**15, 2**15, (B, L, H, 64), dtype=torch.int16, device=dev)
+    y = torch.zeros(B, L, H, 64, dtype=torch.int16, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert bench.probes().bench_probe_stream_prefill(q.data_ptr(), k.data_ptr(), v.data_ptr(), y.data_ptr(), B, H, L, stream) == 0
+    torch.cuda.synchronize()
+    t = torch.arange(512, device=dev)
+    src_row, src_pc = (t & 127) >> 1, t & 1
+    want = torch.empty_like(y)
+    pick = lambda x, rows, n_pc, pc: x[:, rows].view(B, 512, H, n_pc, 8)[:, t, :, pc].permute(1, 0, 2, 3)   # (B, 512, H, 8)
+    for c in range(L // 64):
+        qk = torch.where((t < 128)[None, :, None, None], pick(q, 64 * c + src_row, 2, src_pc), pick(k, 64 * c + src_row, 2, src_pc))
+        qk = torch.where((t < 256)[None, :, None, None], qk, torch.zeros_like(qk))   # threads 256..511 fetch v only
+        vv = pick(v, 64 * c + (t >> 3), 8, t & 7)
+        blk = (qk ^ vv).view(B, 64, 8, H, 8).permute(0, 1, 3, 2, 4).reshape(B, 64, H, 64)    # thread t = (row t / 8, piece t % 8)
+        want[:, 64 * c: 64 * c + 64] = blk
+    assert torch.equal(y, want)
