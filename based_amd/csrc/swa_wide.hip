@@ -7,7 +7,7 @@
 // Prefill.  Four wavefronts cover 64 consecutive queries of one (batch, head); wavefront w owns
 // queries [q0 + 16 w, q0 + 16 w + 16) and sees the staged keys 16 w .. 16 w + 16 NT - 1 of a ring
 // of NB blocks of 64 K rows and 64 V rows (NB = 2: up to 64 keys to the left, NB = 3: up to 128).
-//   S^T = K Q^T   : NT key tiles x ceil(D / 32) MFMA 16x16x32; K and Q rows are staged in LDS
+//   S^T = K Q^T   : NT key tiles x 2 or 4 MFMA 16x16x32 (head dims up to 64 / 128); K and Q rows are staged in LDS
 //                   (rotated on the way in), a lane's operand = 8 consecutive bf16 of one row.
 //   softmax       : whole window in one pass, lane <-> query, registers <-> keys.
 //   O^T = V^T P^T : P from the accumulator registers, V^T by the transposing LDS read; the
@@ -84,7 +84,9 @@ constexpr int wide_lds_bytes(int nb) { return (2 * nb + 1) * kWQTile * kWRowByte
 // tables of R/2 frequencies per position (slide_attention.py:346-355,553-556); kc_out / vc_out
 // (optional): the (rotated) K rows and the V rows of this call also go to a KV cache
 // (_update_kv_cache, slide_attention.py:255-281).
-template <int RMODE, int NB>
+// NDS: contraction steps of 32 channels (head dims up to 32 NDS); a compile-time count keeps the
+// products free of branches, so that the operand reads of one MFMA travel under the others.
+template <int RMODE, int NB, int NDS>
 __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int D, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
@@ -104,8 +106,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
   const int col = lane & 15;
   const int grp = lane >> 4;
   const int np = D >> 3;            // live 16-byte pieces of a row
-  const int n_ds = (D + 31) >> 5;   // contraction steps of 32 channels
-  const int n_et = (D + 15) >> 4;   // output channel tiles of 16
+  constexpr int NET = 2 * NDS;      // output channel tiles of 16 (a tile past the head dim works on zeros)
   const bool whole_lines = (D & 63) == 0 && (o_sh & 63) == 0 && (o_sl & 63) == 0;
 
   // Work item: a run of consecutive query tiles of one (batch, head).  The heads of one run of
@@ -245,6 +246,13 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     store_rows(0, q0, pre, true);
   }
   if (tile_begin + 1 < tile_end) load_rows(q0 + kWQTile, pre, true);  // travels while this tile is computed
+  // The three-block ring leaves room for one workgroup per compute unit (112 KB of LDS), i.e. one
+  // wavefront per SIMD with the whole register file to itself and nobody to cover its memory
+  // round trips: it keeps the rows of TWO tiles in flight (a second register set).
+  constexpr int DEPTH = NB == 3 ? 2 : 1;
+  WideRows pre2;
+  if constexpr (DEPTH == 2)
+    if (tile_begin + 2 < tile_end) load_rows(q0 + 2 * kWQTile, pre2, true);
 
   // lane-constant parts of the operand addresses (a tile's rows start at multiples of 16, so
   // row & 15 == col for the operand rows and row & 7 == vt_row & 7 for the transposed ones)
@@ -255,7 +263,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
 
   const int i_win = w_left >= 64 * (NB - 1) + 15 ? 0 : (64 * (NB - 1) + 30 - w_left) >> 4;
   int own = 0;  // ring block with keys [q0, q0 + 64); block own + 1 (mod NB) is the oldest
-  for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kWQTile, own = own + 1 == NB ? 0 : own + 1) {
+  // one tile; `nxt` holds the rows of tile + 1 and is refilled with those of tile + 1 + DEPTH
+  auto do_tile = [&](int tile, WideRows& nxt) {
     const int oldest = own + 1 == NB ? 0 : own + 1;
     const int n0 = q0 + 16 * wq;
     const int n = n0 + col;
@@ -266,9 +275,9 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     };
     __syncthreads();  // the staged rows are visible
     unsigned char* const q_rows = lds + kOffQ + 16 * wq * kWRowBytes;  // this wavefront's own
-    bf16x8 bq[4];
+    bf16x8 bq[NDS];
 #pragma unroll
-    for (int ds = 0; ds < 4; ++ds)
+    for (int ds = 0; ds < NDS; ++ds)
       bq[ds] = *reinterpret_cast<const bf16x8*>(q_rows + k_lane + (wide_swz_k(col, 4 * ds + grp) << 4));
 
     // ---- S^T tiles: keys (rows) x queries (cols), contraction over the channels ----
@@ -278,10 +287,9 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
       const unsigned char* row = lds + ring_row(16 * wq + 16 * i) * kWRowBytes + k_lane;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ds = 0; ds < 4; ++ds)
-        if (ds < n_ds)
-          acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              *reinterpret_cast<const bf16x8*>(row + (wide_swz_k(col, 4 * ds + grp) << 4)), bq[ds], acc, 0, 0, 0);
+      for (int ds = 0; ds < NDS; ++ds)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            *reinterpret_cast<const bf16x8*>(row + (wide_swz_k(col, 4 * ds + grp) << 4)), bq[ds], acc, 0, 0, 0);
       st[i] = acc;
     }
 
@@ -317,9 +325,9 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     sum += __shfl_xor(sum, 32, 64);
 
     // ---- O^T = V^T P^T: ceil(D / 16) channel tiles x NS key slabs of 32 ----
-    f32x4 ot[8];
+    f32x4 ot[NET];
 #pragma unroll
-    for (int et = 0; et < 8; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int et = 0; et < NET; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
       u32x4 pb4;
@@ -336,16 +344,14 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
       const unsigned char* lo_rows = lds + kOffV + ring_row(16 * wq + 32 * s) * kWRowBytes + v_lane;
       const unsigned char* hi_rows = lds + kOffV + ring_row(s < NS - 1 ? 16 * wq + 32 * s + 16 : 0) * kWRowBytes + v_lane;
 #pragma unroll
-      for (int et = 0; et < 8; ++et) {
-        if (et < n_et) {
-          const int pc = wide_swz_v(vt_row, 2 * et + v_half) << 4;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + pc));
-          s16x4 hi = {0, 0, 0, 0};
-          if (s < NS - 1)
-            hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + pc));
-          const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
-        }
+      for (int et = 0; et < NET; ++et) {
+        const int pc = wide_swz_v(vt_row, 2 * et + v_half) << 4;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + pc));
+        s16x4 hi = {0, 0, 0, 0};
+        if (s < NS - 1)
+          hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + pc));
+        const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
       }
     }
 
@@ -353,13 +359,11 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     // registers, and only this wavefront rewrites them) so that every lane stores 16 bytes of a row ----
     const float inv = 1.0f / sum;
 #pragma unroll
-    for (int et = 0; et < 8; ++et) {
-      if (et < n_et) {
-        const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
-        const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
-        *reinterpret_cast<uint2*>(q_rows + k_lane + (wide_swz_k(col, 2 * et + (grp >> 1)) << 4) + 8 * (grp & 1)) =
-            make_uint2(w0, w1);
-      }
+    for (int et = 0; et < NET; ++et) {
+      const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
+      const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
+      *reinterpret_cast<uint2*>(q_rows + k_lane + (wide_swz_k(col, 2 * et + (grp >> 1)) << 4) + 8 * (grp & 1)) =
+          make_uint2(w0, w1);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -380,8 +384,18 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     // ---- the oldest block (and the query rows) take the next tile's rows ----
     if (tile + 1 < tile_end) {
       __syncthreads();  // every wavefront is done with the oldest block
-      store_rows(oldest, q0 + kWQTile, pre, true);
-      if (tile + 2 < tile_end) load_rows(q0 + 2 * kWQTile, pre, true);  // not waited for here
+      store_rows(oldest, q0 + kWQTile, nxt, true);
+      if (tile + 1 + DEPTH < tile_end) load_rows(q0 + (1 + DEPTH) * kWQTile, nxt, true);  // not waited for here
+    }
+    q0 += kWQTile;
+    own = own + 1 == NB ? 0 : own + 1;
+  };
+  if constexpr (DEPTH == 1) {
+    for (int tile = tile_begin; tile < tile_end; ++tile) do_tile(tile, pre);
+  } else {
+    for (int tile = tile_begin; tile < tile_end; tile += 2) {
+      do_tile(tile, pre);
+      if (tile + 1 < tile_end) do_tile(tile + 1, pre2);
     }
   }
 }
@@ -591,7 +605,7 @@ __global__ __launch_bounds__(256) void swa_step_wide_kernel(
 static bool wide_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 constexpr int kWideMaxDevices = 64;
-static std::atomic<bool> g_wide_lds_allowed[kWideMaxDevices][3 /*RMODE*/][2 /*NB - 2*/];
+static std::atomic<bool> g_wide_lds_allowed[kWideMaxDevices][3 /*RMODE*/][2 /*NB - 2*/][2 /*NDS / 2 - 1*/];
 
 // shared checks of the rotary arguments; returns the layout code or -1 with the error set
 static int wide_rope_mode(const char* who, const float* rope_cos, const float* rope_sin, int64_t rotary_dim,
@@ -668,17 +682,22 @@ extern "C" BASED_API int based_swa_prefill_wide(const void* q, const void* k, co
   using Kern = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int, int, int, int, int, long, long, long,
                         long, long, long, long, long, long, long, long, long, int, float, const float*, const float*, int,
                         __bf16*, __bf16*, long, long, long);
-  static const Kern kerns[3][2] = {
-      {swa_prefill_wide_kernel<kRopeNone, 2>, swa_prefill_wide_kernel<kRopeNone, 3>},
-      {swa_prefill_wide_kernel<kRopeHalf, 2>, swa_prefill_wide_kernel<kRopeHalf, 3>},
-      {swa_prefill_wide_kernel<kRopeInterleaved, 2>, swa_prefill_wide_kernel<kRopeInterleaved, 3>}};
-  const Kern kern = kerns[rmode][nb - 2];
+  // head dims up to 64 contract in two steps of 32 channels, up to 128 in four
+  static const Kern kerns[3][2][2] = {
+      {{swa_prefill_wide_kernel<kRopeNone, 2, 2>, swa_prefill_wide_kernel<kRopeNone, 2, 4>},
+       {swa_prefill_wide_kernel<kRopeNone, 3, 2>, swa_prefill_wide_kernel<kRopeNone, 3, 4>}},
+      {{swa_prefill_wide_kernel<kRopeHalf, 2, 2>, swa_prefill_wide_kernel<kRopeHalf, 2, 4>},
+       {swa_prefill_wide_kernel<kRopeHalf, 3, 2>, swa_prefill_wide_kernel<kRopeHalf, 3, 4>}},
+      {{swa_prefill_wide_kernel<kRopeInterleaved, 2, 2>, swa_prefill_wide_kernel<kRopeInterleaved, 2, 4>},
+       {swa_prefill_wide_kernel<kRopeInterleaved, 3, 2>, swa_prefill_wide_kernel<kRopeInterleaved, 3, 4>}}};
+  const int wide = D > 64 ? 1 : 0;
+  const Kern kern = kerns[rmode][nb - 2][wide];
   const size_t lds = (size_t)wide_lds_bytes(nb);
   {
     int dev = 0;
     BASED_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kWideMaxDevices, BASED_ERR_LAUNCH,
                   "swa_prefill_wide: cannot identify the current device");
-    std::atomic<bool>& allowed = g_wide_lds_allowed[dev][rmode][nb - 2];
+    std::atomic<bool>& allowed = g_wide_lds_allowed[dev][rmode][nb - 2][wide];
     if (!allowed.load(std::memory_order_acquire)) {  // more than 64 KB of LDS has to be asked for once per device
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
