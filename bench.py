@@ -44,10 +44,11 @@ D_EXP = 273
 # the same counter reads for a plain copy of known size (the summaries and the commands that
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": 294355149,   # B=128, H=16, dv=64, rotating state sets: fetch 147,032,269 + write 147,322,880
-    "lin_prefill_mfma_kernel": {96: 2208919860},  # B=96, L=4096, dv=64, states written; keyed by batch
-    "swa_prefill_kernel": 283253146,   # B=8, H=16, L=4096: fetch 216,144,282 + write 67,108,864
-    "decode_linear_kernel_lm_head": 105068544,   # M=4, 50280 x 1024 + closing norm: fetch 104,456,397 + write 612,147
+    "lin_step_kernel": 293108326,   # B=128, H=16, dv=64, rotating state sets: fetch 146,970,214 + write 146,138,112
+    "lin_step_kernel_B64_dv128": 290387149,   # long-context decode: fetch 145,405,952 + write 144,981,197
+    "lin_prefill_mfma_kernel": {96: 2317252301},  # B=96, L=4096, dv=64, states written: fetch 1,402,835,354 + write 914,416,947; keyed by batch
+    "swa_prefill_kernel": 283241574,   # B=8, H=16, L=4096: fetch 216,132,198 + write 67,109,376
+    "decode_linear_kernel_lm_head": 104962356,   # M=4, 50280 x 1024 + closing norm: fetch 104,351,130 + write 611,226
 }
 
 
@@ -217,7 +218,8 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "frac_spread": {"replays": replays, "median": frac_of(spread["median"]),
                                      "slowest": frac_of(spread["max"]), "fastest": frac_of(spread["min"])},
-                     "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else (
+                         MEASURED_TRAFFIC_BYTES["lin_step_kernel_B64_dv128"] if (B, H, dv) == (64, 16, 128) else None),
                      "algorithmic_bytes_per_launch": bytes_per_launch,
                      "timed": "median over %d replays of a graph of the timed steps, the slower of cold (rotating state "
                               "sets) and warm (one set); each replay timed by itself, spread in frac_spread (launched one "
@@ -307,7 +309,8 @@ def bench_prefill(torch, ops, steps, warmup, B=8, H=16, L=4096, dv=64):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES["lin_prefill_mfma_kernel"].get(B) if (L, dv) == (4096, 64) else None,
                      "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": byts,
-                     "hbm_gbs": round(byts / (ms * 1e-3) / 1e9, 1)},
+                     "hbm_gbs": round(byts / (ms * 1e-3) / 1e9, 1),
+                     "hbm_frac": round(byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
     }
 
 
