@@ -88,7 +88,9 @@ def probes():
         lib.bench_probe_rmw.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
         lib.bench_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
         lib.bench_probe_stream_prefill.argtypes = [C.c_void_p] * 4 + [C.c_int64] * 3 + [C.c_void_p]
-        for fn in (lib.bench_probe_stream_qkv, lib.bench_probe_rmw, lib.bench_probe_copy, lib.bench_probe_stream_prefill):
+        lib.bench_probe_mfma.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.POINTER(C.c_double), C.c_void_p]
+        for fn in (lib.bench_probe_stream_qkv, lib.bench_probe_rmw, lib.bench_probe_copy, lib.bench_probe_stream_prefill,
+                   lib.bench_probe_mfma):
             fn.restype = C.c_int
         _probes = lib
     return _probes
@@ -418,6 +420,22 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     }
 
 
+def bench_mfma_rate(torch, steps=20):
+    """TFLOP/s of a loop of nothing but dense bf16 MFMA 16x16x32 (bench_probes.hip), after 30 ms of
+    that load: what the matrix pipes sustain at the clock the board settles at."""
+    import ctypes as C
+
+    lib = probes()
+    dev = torch.device("cuda:0")
+    wgs = 256 * 4
+    buf = torch.empty(wgs * 256, dtype=torch.float32, device=dev)
+    flops = C.c_double(0.0)
+    stream = torch.cuda.current_stream().cuda_stream
+    ms, _ = _events_ms(torch, lambda: _probe_ok(lib.bench_probe_mfma(buf.data_ptr(), wgs, 2000, C.byref(flops), stream)),
+                       steps, 2, warmup_ms=30.0)
+    return flops.value / (ms * 1e-3) / 1e12
+
+
 def bench_machine(torch, steps=20, warmup=4, n_sets=4):
     """What this machine's memory delivers for the access patterns of the HBM-bound kernels, measured
     with the probe kernels of bench_probes.hip (no arithmetic) over rotating buffers beyond the
@@ -472,7 +490,9 @@ def bench_machine(torch, steps=20, warmup=4, n_sets=4):
     out["stream_prefill_B96_ms"] = round(ms, 4)
     out["stream_prefill_B96_GBps"] = round(B * L * H * 320 / (ms * 1e-3) / 1e9, 1)
     del q, k, v, y
-    out["note"] = ("probe kernels of bench_probes.hip over %d rotating buffer sets; GB/s of bytes read + written" % n_sets)
+    out["mfma_bf16_sustained_TFLOPs"] = round(bench_mfma_rate(torch), 1)
+    out["note"] = ("probe kernels of bench_probes.hip over %d rotating buffer sets; GB/s of bytes read + written; "
+                   "mfma: a loop of dense bf16 MFMA only, after 30 ms of that load" % n_sets)
     return out
 
 
@@ -759,6 +779,12 @@ def main():
         if args.only is None or args.prefill_batches == "1,8,32,96":
             pre.append(bench_prefill(torch, ops, 30, 3, B=32, dv=112))   # the released 1B / 1.3B head dim
         out["prefill"] = [{k: (round(v, 3) if isinstance(v, float) else v) for k, v in p.items()} for p in pre]
+        # the same fractions against what a loop of nothing but MFMA sustains on this board (the
+        # published peak assumes the maximum clock, which the board does not hold under that load)
+        sustained = bench_mfma_rate(torch)
+        for p in out["prefill"]:
+            p["roofline"]["mfma_sustained_TFLOPs"] = round(sustained, 1)
+            p["roofline"]["frac_of_sustained_mfma"] = round(p["roofline"]["achieved"] / sustained, 4)
     if args.only in (None, "prefill"):
         # configs[4]: one 32K-token sequence at head dim 128, and its decode batch of 64
         c5 = bench_prefill(torch, ops, 30, 3, B=1, L=32768, dv=128)

@@ -11,6 +11,10 @@
 //                profiler's HBM byte counters.
 //   stream_prefill : the q / k / v reads and y writes of the chunked linear-attention prefill, chunk
 //                by chunk per (batch, head), with no arithmetic: the memory ceiling of that kernel.
+//   mfma       : nothing but independent dense bf16 MFMA 16x16x32 on non-zero register operands,
+//                four workgroups of four wavefronts per compute unit: the rate the matrix pipes
+//                sustain at the clock the board holds under that load (the published peak assumes
+//                the maximum clock).
 //
 // Every entry point returns 0, or 1 for arguments it does not take.
 #include <hip/hip_runtime.h>
@@ -124,6 +128,47 @@ __global__ __launch_bounds__(512, 4) void probe_stream_prefill_kernel(const u32x
 static bool probe_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace bench_probes
+
+namespace bench_probes {
+typedef __attribute__((ext_vector_type(8))) __bf16 probe_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float probe_f32x4;
+constexpr int kMfmaPerIter = 32;   // 4 rounds over 8 independent accumulators
+
+__global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ out, int iters) {
+  probe_f32x4 m[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) m[i] = probe_f32x4{0.f, 0.f, 0.f, 0.f};
+  probe_bf16x8 a, b;
+  unsigned s = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 12345u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    s = s * 1664525u + 1013904223u;
+    a[i] = (__bf16)(((int)(s >> 16) % 2001 - 1000) * 1e-3f);
+    s = s * 1664525u + 1013904223u;
+    b[i] = (__bf16)(((int)(s >> 16) % 2001 - 1000) * 1e-3f);
+  }
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < kMfmaPerIter / 8; ++r)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) m[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, m[i], 0, 0, 0);
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc += m[i][0] + m[i][1] + m[i][2] + m[i][3];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+}  // namespace bench_probes
+
+// `out` takes workgroups * 256 floats; *flops (host) receives the floating-point operations of the launch.
+PROBE_API int bench_probe_mfma(float* out, int64_t workgroups, int64_t iters, double* flops, void* stream) {
+  using namespace bench_probes;
+  PROBE_REQUIRE(out && flops && workgroups > 0 && workgroups < (1ll << 20) && iters > 0 && iters < (1ll << 24));
+  *flops = (double)workgroups * 4.0 * (double)iters * kMfmaPerIter * (2.0 * 16 * 16 * 32);
+  hipLaunchKernelGGL(probe_mfma_kernel, dim3((unsigned)workgroups), dim3(256), 0, static_cast<hipStream_t>(stream), out,
+                     (int)iters);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
 
 PROBE_API int bench_probe_stream_qkv(const void* qkv, void* o, int64_t B, int64_t H, int64_t L,
                                                 int heads_per_group, void* stream) {

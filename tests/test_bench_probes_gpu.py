@@ -59,3 +59,22 @@ def test_stream_prefill_probe_moves_what_it_says(dev):
         blk = (qk ^ vv).view(B, 64, 8, H, 8).permute(0, 1, 3, 2, 4).reshape(B, 64, H, 64)    # thread t = (row t / 8, piece t % 8)
         want[:, 64 * c: 64 * c + 64] = blk
     assert torch.equal(y, want)
+
+
+def test_mfma_probe_counts_its_flops_and_runs(dev):
+    """The MFMA-rate probe reports 32 MFMA 16x16x32 per iteration and wavefront, writes one finite
+    sum per lane (every lane's operands differ, the sums are not all equal) and refuses bad sizes."""
+    import ctypes as C
+    import bench
+
+    lib = bench.probes()
+    wgs, iters = 8, 3
+    out = torch.zeros(wgs * 256, dtype=torch.float32, device=dev)
+    flops = C.c_double(0.0)
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.bench_probe_mfma(out.data_ptr(), wgs, iters, C.byref(flops), stream) == 0
+    torch.cuda.synchronize()
+    assert flops.value == wgs * 4 * iters * 32 * 2 * 16 * 16 * 32
+    assert torch.isfinite(out).all() and out.unique().numel() > wgs
+    assert lib.bench_probe_mfma(out.data_ptr(), 0, iters, C.byref(flops), stream) == 1
+    assert lib.bench_probe_mfma(None, wgs, iters, C.byref(flops), stream) == 1
