@@ -113,21 +113,32 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 //   state image, 2     : bf16 image of the state, [slab][channel tile][lane] x 16 B; chunk c is
 //                        read out from image[c & 1] while image[(c+1) & 1] is being written.
 //   K2, K1, 2 each     : normaliser state (see below).
+// A workgroup carries CT channel tiles of its head: 4 (one block of 64 channels; two workgroups
+// per compute unit) or 8 (two blocks; head dims 65..128: psi(q) and psi(k) are generated once for
+// both blocks, at 142 KB of LDS and up to 256 registers, i.e. one workgroup per compute unit).
+// With two blocks the v rows of a ring slot are two 64 x 128 B arrays, one per block, each laid
+// out as described above.
 constexpr int kRing = 3;
 constexpr int kQkBytes = kChunk * kFeat * 2;       // 2 KB
-constexpr int kVBytes = kChunk * 64 * 2;           // 8 KB
-constexpr int kDataBytes = 2 * kQkBytes + kVBytes; // one ring slot: q | k | v
+constexpr int kVBlockBytes = kChunk * 64 * 2;      // 8 KB: the v rows of one block of 64 channels
 constexpr int kDataK = kQkBytes, kDataV = 2 * kQkBytes;
-constexpr int kImgBytes = 5 * kCTiles * 64 * 16;   // state image: [slab][channel tile][lane] x 16 B
 constexpr int kK2Bytes = 2 * 64 * 8;               // hi and lo halves of the 16x16 second-moment operand
 constexpr int kOffData = 0;
-constexpr int kOffImg = kOffData + kRing * kDataBytes;
-constexpr int kOffK2 = kOffImg + 2 * kImgBytes;
-constexpr int kOffK1 = kOffK2 + 2 * kK2Bytes;      // [2][16] floats: first moment of k
-constexpr int kLdsBytes = kOffK1 + 2 * 16 * 4;
-static_assert(kLdsBytes <= 80 * 1024, "two workgroups must fit the 160 KB of a compute unit");
-static_assert(kOffImg % 16 == 0 && kOffK2 % 16 == 0 && kOffK1 % 16 == 0, "16-byte aligned sections");
-constexpr int kLoadsPerUpdater = 3;   // of the 12 wave-wide direct loads of a chunk: q 2, k 2, v 8
+template <int CT>
+struct PrefillLds {
+  static_assert(CT == 4 || CT == 8, "one or two blocks of 64 channels");
+  static constexpr int kBlocks = CT / 4;
+  static constexpr int kDataBytes = 2 * kQkBytes + kBlocks * kVBlockBytes;  // one ring slot: q | k | v
+  static constexpr int kImgBytes = 5 * CT * 64 * 16;   // state image: [slab][channel tile][lane] x 16 B
+  static constexpr int kOffImg = kOffData + kRing * kDataBytes;
+  static constexpr int kOffK2 = kOffImg + 2 * kImgBytes;
+  static constexpr int kOffK1 = kOffK2 + 2 * kK2Bytes;      // [2][16] floats: first moment of k
+  static constexpr int kBytes = kOffK1 + 2 * 16 * 4;
+  // of the wave-wide direct loads of a chunk (q 2, k 2, v 8 per block) each updater issues
+  static constexpr int kLoadsPerUpdater = (4 + 8 * kBlocks) / kWavesPerChain;
+  static_assert(kOffImg % 16 == 0 && kOffK2 % 16 == 0 && kOffK1 % 16 == 0, "16-byte aligned sections");
+  static_assert(kBytes * (CT == 4 ? 2 : 1) <= 160 * 1024, "must fit the 160 KB of a compute unit");
+};
 
 // One chain = one (batch, head, 64-channel block), scanned in chunks of 64 tokens by a workgroup
 // of EIGHT wavefronts in two kinds of roles that run concurrently and meet at one barrier per
@@ -208,6 +219,27 @@ __device__ __forceinline__ long item_of_block() {
   return (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
 }
 
+// What a workgroup works on: head `bh`, its first block of 64 channels `eb0`, how many of the
+// workgroup's channels exist (`live`, a multiple of 16), and the index of that first block among
+// all (head, block) chains (the unit of the segmented scan's workspace).
+struct PrefillItem {
+  long bh, chain0;
+  int eb0, live;
+};
+template <int CT>
+__device__ __forceinline__ PrefillItem prefill_item(int dv) {
+  constexpr int kBlocks = CT / 4;
+  const int n_eb = (dv + 63) >> 6;
+  const int n_wb = (n_eb + kBlocks - 1) / kBlocks;  // workgroups per head
+  const long item = item_of_block();
+  PrefillItem it;
+  it.bh = item / n_wb;
+  it.eb0 = (int)(item % n_wb) * kBlocks;
+  it.live = dv - 64 * it.eb0 < 64 * kBlocks ? dv - 64 * it.eb0 : 64 * kBlocks;
+  it.chain0 = it.bh * n_eb + it.eb0;
+  return it;
+}
+
 // Transposing 64-bit LDS read pair: inside each group of 16 lanes, lane 4a + b receives element
 // b of what lanes a, a+4, a+8, a+12 loaded.  `p` is the lane's source address for the first four
 // tokens; the second four are `hi_bytes` further on.
@@ -222,8 +254,9 @@ __device__ __forceinline__ bf16x8 load_tr_pair(const unsigned char* p, int hi_by
 // 4j + a of a group fetches channels 16 et + 4a..+3 of token 32 s + 4 grp + j (+16), which sit in
 // 16-byte piece (2 et + a/2) ^ 2j of the row, i.e. at byte ((et ^ j) << 5) + 8a.
 // vt_lane = 128 (4 grp + j) + 8a is the lane's part of the address.
+// Channel tiles 4 and up belong to the second block of 64 channels, whose rows follow the first's.
 __device__ __forceinline__ bf16x8 load_vt(const unsigned char* slot, int vt_lane, int j, int et, int s) {
-  return load_tr_pair(slot + kDataV + vt_lane + (((et ^ j) & 3) << 5) + 4096 * s, 2048);
+  return load_tr_pair(slot + kDataV + (et >> 2) * kVBlockBytes + vt_lane + (((et ^ j) & 3) << 5) + 4096 * s, 2048);
 }
 // k^T operand tile of token slab s (lane <-> feature col) from the row-major 32-byte k rows
 __device__ __forceinline__ bf16x8 load_kt(const unsigned char* slot, int kt_lane, int s) {
@@ -252,16 +285,16 @@ __device__ __forceinline__ void barrier_updater() {
 // ------------------------------------------------------------------------------------------
 // reader of token tile nt
 // ------------------------------------------------------------------------------------------
-template <int nt, int MODE>
+template <int nt, int MODE, int CT>
 __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
+  using LD = PrefillLds<CT>;
   const int lane = threadIdx.x & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
-  const int n_eb = (dv + 63) >> 6;
-  const long item = item_of_block();
-  const long bh = item / n_eb;
-  const int eb = (int)(item % n_eb);  // 64-channel block of the value dimension
-  const int live_ch = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // channels of this block that exist (a multiple of 16)
+  const PrefillItem it = prefill_item<CT>(dv);
+  const long bh = it.bh;
+  const int eb = it.eb0;        // first 64-channel block of this workgroup
+  const int live_ch = it.live;  // channels of this workgroup that exist (a multiple of 16)
   const int b = (int)(bh / H), h = (int)(bh % H);
   y += b * y_sb + h * y_sh + 64 * eb;
   const int seg = blockIdx.z;
@@ -281,15 +314,15 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
   for (int t0 = t_begin; t0 < t_end; t0 += kChunk, buf ^= 1, slot_i = slot_i == kRing - 1 ? 0 : slot_i + 1) {
     if constexpr (MODE != kModeDelta) {
       const int ntok = t_end - t0 < kChunk ? t_end - t0 : kChunk;
-      const unsigned char* slot = lds + kOffData + slot_i * kDataBytes;
+      const unsigned char* slot = lds + kOffData + slot_i * LD::kDataBytes;
       const __bf16* s_q = reinterpret_cast<const __bf16*>(slot);
       const __bf16* s_k = reinterpret_cast<const __bf16*>(slot + kDataK);
-      const unsigned char* s_img = lds + kOffImg + buf * kImgBytes;
+      const unsigned char* s_img = lds + LD::kOffImg + buf * LD::kImgBytes;
 
       // O^T[channel tile]: lane <-> token 16 nt + col, regs <-> channel 4 grp + r
-      f32x4 O[kCTiles];
+      f32x4 O[CT];
 #pragma unroll
-      for (int et = 0; et < kCTiles; ++et) O[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int et = 0; et < CT; ++et) O[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
       // ---- reads of the first stages ----
       // the 16 raw features are exactly the contraction of a 16x16x16 MFMA: lane <-> (row, features 4 grp ..+3)
@@ -299,20 +332,20 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         qx[i] = *reinterpret_cast<const bf16x4*>(s_q + (16 * nt + col) * kFeat + 4 * (((grp + i) & 3) ^ qk_swz));
-      const unsigned char* k2 = lds + kOffK2 + buf * kK2Bytes;
+      const unsigned char* k2 = lds + LD::kOffK2 + buf * kK2Bytes;
       const s16x4 k2hi = *reinterpret_cast<const s16x4*>(k2 + lane * 8);
       const s16x4 k2lo = *reinterpret_cast<const s16x4*>(k2 + 512 + lane * 8);
-      const f32x4 k1 = *reinterpret_cast<const f32x4*>(lds + kOffK1 + buf * 64 + 16 * grp);
+      const f32x4 k1 = *reinterpret_cast<const f32x4*>(lds + LD::kOffK1 + buf * 64 + 16 * grp);
       s16x4 ka[nt + 1];
 #pragma unroll
       for (int mt = 0; mt <= nt; ++mt)
         ka[mt] = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * (grp ^ qk_swz));
-      auto img_load = [&](int sg, bf16x8 (&A)[kCTiles]) {
+      auto img_load = [&](int sg, bf16x8 (&A)[CT]) {
 #pragma unroll
-        for (int et = 0; et < kCTiles; ++et)
-          A[et] = *reinterpret_cast<const bf16x8*>(s_img + ((sg * kCTiles + et) * 64 + lane) * 16);
+        for (int et = 0; et < CT; ++et)
+          A[et] = *reinterpret_cast<const bf16x8*>(s_img + ((sg * CT + et) * 64 + lane) * 16);
       };
-      bf16x8 A[5][kCTiles];
+      bf16x8 A[5][CT];
       img_load(0, A[0]);
       BASED_STAGE_END();
 
@@ -364,7 +397,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       // this lane's share of the normaliser of token 16 nt + col: first the quadratic form over
       // the earlier chunks, then the row sums of the in-chunk weights
       float zpart = 0.f;
-      bf16x8 vt_p[2][kCTiles];
+      bf16x8 vt_p[2][CT];
       bf16x8 bp[2];
       // in-chunk weights 1 + s + s^2/2 (s = a/4) of key tiles 2 s, 2 s + 1, masked on the diagonal
       // tile, packed as the B operand of the V^T A^T product; tiles above the diagonal are zero
@@ -391,14 +424,14 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
         if constexpr (sg + 1 < 5) img_load(sg + 1, A[sg + 1]);
         if constexpr (sg == 3) {
 #pragma unroll
-          for (int et = 0; et < kCTiles; ++et) vt_p[0][et] = load_vt(slot, vt_lane, vt_j, et, 0);
+          for (int et = 0; et < CT; ++et) vt_p[0][et] = load_vt(slot, vt_lane, vt_j, et, 0);
         }
         if constexpr (sg == 4 && nt >= 2) {
 #pragma unroll
-          for (int et = 0; et < kCTiles; ++et) vt_p[1][et] = load_vt(slot, vt_lane, vt_j, et, 1);
+          for (int et = 0; et < CT; ++et) vt_p[1][et] = load_vt(slot, vt_lane, vt_j, et, 1);
         }
 #pragma unroll
-        for (int et = 0; et < kCTiles; ++et) O[et] = mfma(A[sg][et], Bq[sg], O[et]);
+        for (int et = 0; et < CT; ++et) O[et] = mfma(A[sg][et], Bq[sg], O[et]);
         if constexpr (sg + 1 < 5) Bq[sg + 1] = psi_q(integral_constant<int, sg + 1>{});
         if constexpr (sg == 0) {
 #pragma unroll
@@ -407,7 +440,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
           weights(integral_constant<int, 0>{});
         }
         if constexpr (sg == 1 && nt >= 2) weights(integral_constant<int, 1>{});
-        interleave<4, (sg == 0 ? 9 : (sg == 1 && nt >= 2) ? 8 : 3)>();
+        interleave<CT, ((sg == 0 ? 9 : (sg == 1 && nt >= 2) ? 8 : 3) * 4 + CT - 1) / CT>();
         BASED_STAGE_END();
       });
 
@@ -416,7 +449,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       static_for<nt / 2 + 1>([&](auto SS) {
         constexpr int s = decltype(SS)::value;
 #pragma unroll
-        for (int et = 0; et < kCTiles; ++et) O[et] = mfma(vt_p[s][et], bp[s], O[et]);
+        for (int et = 0; et < CT; ++et) O[et] = mfma(vt_p[s][et], bp[s], O[et]);
         if constexpr (s == 0) {
           // the earlier tokens count 1 each, the lane groups hold partial sums of the rest
           const float z = group_allreduce(zpart) + (float)t0;
@@ -429,27 +462,35 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       // A lane holds 4 channels (8 bytes) of each channel tile.  Lane groups g and g ^ 1 trade two
       // tiles (one row swap per dword), after which every lane holds 2 x 8 consecutive channels
       // and stores 16 contiguous bytes twice, straight from registers.
-      uint32_t P[kCTiles][2];
+      uint32_t P[CT][2];
 #pragma unroll
-      for (int et = 0; et < kCTiles; ++et) {
+      for (int et = 0; et < CT; ++et) {
         P[et][0] = pack_bf16(O[et][0] * inv, O[et][1] * inv);
         P[et][1] = pack_bf16(O[et][2] * inv, O[et][3] * inv);
       }
       // The swap must not read a register in the two issue slots after a vector instruction wrote
       // it; the compiler does not look into inline assembly, so each one carries the wait.
 #pragma unroll
-      for (int e = 0; e < 2; ++e)
+      for (int blk = 0; blk < CT / 4; ++blk)
 #pragma unroll
-        for (int d = 0; d < 2; ++d)
-          asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(P[e][d]), "+v"(P[e + 2][d]));
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+          for (int d = 0; d < 2; ++d)
+            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(P[4 * blk + e][d]), "+v"(P[4 * blk + e + 2][d]));
       {
         const int tau = 16 * nt + col;
         if (tau < ntok) {
-          // (in the last block of a head dim that is no multiple of 64 the channels past dv were
+          // (channels past dv, in the last block of a head dim that is no multiple of 64, were
           // computed from stand-in data and are dropped here)
-          __bf16* dst = y + (long)(t0 + tau) * y_sl + out_ch;
-          if (out_ch + 8 <= live_ch) *reinterpret_cast<u32x4*>(dst) = u32x4{P[0][0], P[0][1], P[2][0], P[2][1]};
-          if (out_ch + 24 <= live_ch) *reinterpret_cast<u32x4*>(dst + 16) = u32x4{P[1][0], P[1][1], P[3][0], P[3][1]};
+#pragma unroll
+          for (int blk = 0; blk < CT / 4; ++blk) {
+            const int ch = 64 * blk + out_ch;
+            __bf16* dst = y + (long)(t0 + tau) * y_sl + ch;
+            if (ch + 8 <= live_ch)
+              *reinterpret_cast<u32x4*>(dst) = u32x4{P[4 * blk][0], P[4 * blk][1], P[4 * blk + 2][0], P[4 * blk + 2][1]};
+            if (ch + 24 <= live_ch)
+              *reinterpret_cast<u32x4*>(dst + 16) = u32x4{P[4 * blk + 1][0], P[4 * blk + 1][1], P[4 * blk + 3][0], P[4 * blk + 3][1]};
+          }
         }
       }
     }
@@ -459,7 +500,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
   // the updaters expand the state into the decode layout; readers help to copy it out
   if constexpr (MODE != kModeDelta) {
     if (kv_state != nullptr && last_seg) {
-      const float* blk = reinterpret_cast<const float*>(lds + kOffImg);
+      const float* blk = reinterpret_cast<const float*>(lds + LD::kOffImg);
 #pragma unroll 1
       for (int et = 0; 16 * et < live_ch; ++et) {
         __syncthreads();
@@ -475,17 +516,18 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
 // ------------------------------------------------------------------------------------------
 // updater owning slot tiles own_tile(w, .)
 // ------------------------------------------------------------------------------------------
-template <int w, int MODE>
+template <int w, int MODE, int CT>
 __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
+  using LD = PrefillLds<CT>;
+  constexpr int kLoads = LD::kLoadsPerUpdater;
   const int tid = threadIdx.x - 64 * kWavesPerChain;  // 0..255 among the updaters
   const int lane = tid & 63;
   const int col = lane & 15;
   const int grp = lane >> 4;
-  const int n_eb = (dv + 63) >> 6;
-  const long item = item_of_block();
-  const long bh = item / n_eb;
-  const int eb = (int)(item % n_eb);  // 64-channel block of the value dimension
-  const int live_ch = dv - 64 * eb < 64 ? dv - 64 * eb : 64;  // channels of this block that exist (a multiple of 16)
+  const PrefillItem it = prefill_item<CT>(dv);
+  const long bh = it.bh;
+  const int eb = it.eb0;        // first 64-channel block of this workgroup
+  const int live_ch = it.live;  // channels of this workgroup that exist (a multiple of 16)
   const int b = (int)(bh / H), h = (int)(bh % H);
   q += b * q_sb + h * q_sh;
   k += b * k_sb + h * k_sh;
@@ -496,11 +538,11 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 
   // own share of the running state S[i <-> slot tile own_tile(w, i)][channel tile]:
   // lane <-> channel 16 et + col, regs <-> slot positions 4 grp + r
-  f32x4 S[kOwn][kCTiles];
+  f32x4 S[kOwn][CT];
 #pragma unroll
   for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-    for (int et = 0; et < kCTiles; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int et = 0; et < CT; ++et) S[i][et] = f32x4{0.f, 0.f, 0.f, 0.f};
   // normaliser state (updater kNormWave only), both as MFMA accumulators:
   // K2[4 grp + r][col] (= K2[col][4 grp + r]) and K1[4 grp + r] (the same in every column)
   f32x4 K2 = {0.f, 0.f, 0.f, 0.f};
@@ -511,15 +553,20 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   const int t_begin = MODE == kModeFull ? 0 : seg * seg_tokens;
   const int t_end = MODE == kModeFull ? L : (t_begin + seg_tokens < L ? t_begin + seg_tokens : L);
   const bool last_seg = MODE == kModeFull || seg == n_seg - 1;
+  // workspace entry of this segment for the workgroup's first block; the second block's chain
+  // follows n_seg entries further on
   float* ws_mine = nullptr;
   if constexpr (MODE != kModeFull)
-    ws_mine = ws + (item * n_seg + seg) * (long)kSegStateFloats;
+    ws_mine = ws + (it.chain0 * n_seg + seg) * (long)kSegStateFloats;
+  const long ws_block = (long)n_seg * kSegStateFloats;
+  // offset of accumulator tile (slot tile t, channel tile et) inside the workspace
+  auto ws_tile = [&](int t, int et) { return (et >> 2) * ws_block + ((t * kCTiles + (et & 3)) * 64 + lane) * 4; };
   if constexpr (MODE == kModeFrom) {
 #pragma unroll
     for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-      for (int et = 0; et < kCTiles; ++et)
-        S[i][et] = *reinterpret_cast<const f32x4*>(ws_mine + ((own_tile(w, i) * kCTiles + et) * 64 + lane) * 4);
+      for (int et = 0; et < CT; ++et)
+        S[i][et] = *reinterpret_cast<const f32x4*>(ws_mine + ws_tile(own_tile(w, i), et));
     if constexpr (kNorm) {
       K2 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK2 + lane * 4);
       K1 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK1 + lane * 4);
@@ -532,8 +579,8 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 #pragma unroll
       for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-        for (int et = 0; et < kCTiles; ++et)
-          S[i][et] += *reinterpret_cast<const f32x4*>(src + ((own_tile(w, i) * kCTiles + et) * 64 + lane) * 4);
+        for (int et = 0; et < CT; ++et)
+          S[i][et] += *reinterpret_cast<const f32x4*>(src + ws_tile(own_tile(w, i), et));
       if constexpr (kNorm) {
         K2 += *reinterpret_cast<const f32x4*>(src + kWsK2 + lane * 4);
         K1 += *reinterpret_cast<const f32x4*>(src + kWsK1 + lane * 4);
@@ -555,10 +602,10 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   // (lane <-> row 8j + lane/8, LDS piece lane%8 = global piece (lane%8) ^ 2((lane/8) & 3)).
   // Rows past the end of the sequence are zero-filled instead.
   auto issue_loads = [&](int tc, int slot_index) {
-    unsigned char* slot = lds + kOffData + slot_index * kDataBytes;
+    unsigned char* slot = lds + kOffData + slot_index * LD::kDataBytes;
     const int ntok = t_end - tc < kChunk ? t_end - tc : kChunk;
-    static_for<kLoadsPerUpdater>([&](auto II) {
-      constexpr int id = kLoadsPerUpdater * w + decltype(II)::value;
+    static_for<kLoads>([&](auto II) {
+      constexpr int id = kLoads * w + decltype(II)::value;
       if constexpr (MODE == kModeDelta && id < 2) return;  // no read-out, no q
       int row;
       const __bf16* src;
@@ -568,13 +615,15 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
         src = (id < 2 ? q + (long)(tc + row) * q_sl : k + (long)(tc + row) * k_sl) + 8 * ((lane & 1) ^ ((lane >> 3) & 1));
         dst = slot + (id < 2 ? 0 : kDataK) + 1024 * (id & 1);
       } else {
-        row = 8 * (id - 4) + (lane >> 3);
+        constexpr int vb = (id - 4) / 8, j = (id - 4) % 8;  // block of 64 channels, group of 8 rows
+        row = 8 * j + (lane >> 3);
         // a piece past the head dim (last block of a dv that is no multiple of 64) is fetched from
         // piece 0 instead: channels are independent, so what such channels compute touches no
         // other, and they are never stored
         const int piece = (lane & 7) ^ (2 * ((lane >> 3) & 3));
-        src = v + (long)(tc + row) * v_sl + (8 * piece < live_ch ? 8 * piece : 0);
-        dst = slot + kDataV + 1024 * (id - 4);
+        const int ch = 64 * vb + 8 * piece;
+        src = v + (long)(tc + row) * v_sl + (ch < live_ch ? ch : 0);
+        dst = slot + kDataV + vb * kVBlockBytes + 1024 * j;
       }
       if (ntok == kChunk || row < ntok) {
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
@@ -591,22 +640,22 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   auto publish_pair = [&](int buf) {
     constexpr int t = own_tile(w, 0);
     static_assert(t % 2 == 0 && own_tile(w, 1) == t + 1, "first two own tiles = one slab");
-    unsigned char* img = lds + kOffImg + buf * kImgBytes;
+    unsigned char* img = lds + LD::kOffImg + buf * LD::kImgBytes;
 #pragma unroll
-    for (int et = 0; et < kCTiles; ++et) {
+    for (int et = 0; et < CT; ++et) {
       const u32x4 w4 = {pack_bf16(S[0][et][0], S[0][et][1]), pack_bf16(S[0][et][2], S[0][et][3]),
                         pack_bf16(S[1][et][0], S[1][et][1]), pack_bf16(S[1][et][2], S[1][et][3])};
-      *reinterpret_cast<u32x4*>(img + (((t >> 1) * kCTiles + et) * 64 + lane) * 16) = w4;
+      *reinterpret_cast<u32x4*>(img + (((t >> 1) * CT + et) * 64 + lane) * 16) = w4;
     }
   };
   auto publish_single = [&](int buf) {
     if constexpr (kOwn == 3) {
       constexpr int t = own_tile(w, 2);
-      unsigned char* img = lds + kOffImg + buf * kImgBytes;
+      unsigned char* img = lds + LD::kOffImg + buf * LD::kImgBytes;
 #pragma unroll
-      for (int et = 0; et < kCTiles; ++et) {
+      for (int et = 0; et < CT; ++et) {
         const uint2 w2 = make_uint2(pack_bf16(S[2][et][0], S[2][et][1]), pack_bf16(S[2][et][2], S[2][et][3]));
-        *reinterpret_cast<uint2*>(img + (((t >> 1) * kCTiles + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
+        *reinterpret_cast<uint2*>(img + (((t >> 1) * CT + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
       }
     }
   };
@@ -617,10 +666,10 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       const uint32_t h0 = pack_bf16(K2[0], K2[1]), h1 = pack_bf16(K2[2], K2[3]);
       const float l0 = K2[0] - bf16_bits_to_f32(h0 & 0xFFFFu), l1 = K2[1] - __builtin_bit_cast(float, h0 & 0xFFFF0000u);
       const float l2 = K2[2] - bf16_bits_to_f32(h1 & 0xFFFFu), l3 = K2[3] - __builtin_bit_cast(float, h1 & 0xFFFF0000u);
-      unsigned char* k2 = lds + kOffK2 + buf * kK2Bytes;
+      unsigned char* k2 = lds + LD::kOffK2 + buf * kK2Bytes;
       *reinterpret_cast<uint2*>(k2 + lane * 8) = make_uint2(h0, h1);
       *reinterpret_cast<uint2*>(k2 + 512 + lane * 8) = make_uint2(pack_bf16(l0, l1), pack_bf16(l2, l3));
-      if (col == 0) *reinterpret_cast<f32x4*>(lds + kOffK1 + buf * 64 + 16 * grp) = K1;
+      if (col == 0) *reinterpret_cast<f32x4*>(lds + LD::kOffK1 + buf * 64 + 16 * grp) = K1;
     }
   };
 
@@ -634,24 +683,21 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   }
   // Chunk 0 has landed; chunk 1 may stay in flight when it is a whole chunk (a partial chunk may
   // issue fewer loads than counted on, so then everything is awaited).
+  constexpr int kInFlight = (MODE == kModeDelta && w == 0) ? kLoads - 2 : kLoads;  // this wavefront's loads per chunk
   if (t_begin + 2 * kChunk <= t_end) {
-    if constexpr (MODE == kModeDelta && w == 0) {
-      barrier_updater<1>();
-    } else {
-      barrier_updater<3>();
-    }
+    barrier_updater<kInFlight>();
   } else {
     barrier_updater<0>();
   }
 
   int slot_i = 0, buf = 0;
   for (int t0 = t_begin; t0 < t_end; t0 += kChunk, buf ^= 1, slot_i = slot_i == kRing - 1 ? 0 : slot_i + 1) {
-    const unsigned char* slot = lds + kOffData + slot_i * kDataBytes;
+    const unsigned char* slot = lds + kOffData + slot_i * LD::kDataBytes;
     // operands of the first stage
     bf16x8 kt0 = load_kt(slot, kt_lane, 0);
-    bf16x8 vt_s0[kCTiles], vt_s1[kCTiles];
+    bf16x8 vt_s0[CT], vt_s1[CT];
 #pragma unroll
-    for (int et = 0; et < kCTiles; ++et) vt_s0[et] = load_vt(slot, vt_lane, vt_j, et, 0);
+    for (int et = 0; et < CT; ++et) vt_s0[et] = load_vt(slot, vt_lane, vt_j, et, 0);
     // the rows of the chunk after the next are requested (their slot was last read one chunk ago)
     const bool more2 = t0 + 2 * kChunk < t_end;
     if (more2) issue_loads(t0 + 2 * kChunk, slot_i == 0 ? 2 : slot_i - 1);
@@ -712,10 +758,10 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       constexpr int s = st / kOwn, i = st % kOwn;
       if constexpr (s == 0 && i == kOwn - 1) {
 #pragma unroll
-        for (int et = 0; et < kCTiles; ++et) vt_s1[et] = load_vt(slot, vt_lane, vt_j, et, 1);
+        for (int et = 0; et < CT; ++et) vt_s1[et] = load_vt(slot, vt_lane, vt_j, et, 1);
       }
 #pragma unroll
-      for (int et = 0; et < kCTiles; ++et) S[i][et] = mfma(ak, s == 0 ? vt_s0[et] : vt_s1[et], S[i][et]);
+      for (int et = 0; et < CT; ++et) S[i][et] = mfma(ak, s == 0 ? vt_s0[et] : vt_s1[et], S[i][et]);
       if constexpr (st + 1 < 2 * kOwn) {
         if constexpr (i + 1 == kOwn) {  // the next stage starts slab 1
           unpack_k(kt1);
@@ -729,7 +775,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       if constexpr (MODE != kModeDelta && s == 1 && i == 2) {
         if (more1) publish_pair(buf ^ 1);  // both tiles of the slab are final
       }
-      interleave<4, ((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i == 2) ? 6 : 3)>();
+      interleave<CT, (((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i == 2) ? 6 : 3) * 4 + CT - 1) / CT>();
       BASED_STAGE_END();
     });
     // the rest of the state after this chunk, for the next chunk's readers
@@ -743,11 +789,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
     // The next chunk's rows (requested one chunk ago) must have landed before anyone reads them;
     // the loads requested in this iteration may stay in flight if they were a whole chunk's.
     if (t0 + 3 * kChunk <= t_end) {
-      if constexpr (MODE == kModeDelta && w == 0) {
-        barrier_updater<1>();
-      } else {
-        barrier_updater<3>();
-      }
+      barrier_updater<kInFlight>();
     } else {
       barrier_updater<0>();
     }
@@ -758,11 +800,16 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 #pragma unroll
     for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-      for (int et = 0; et < kCTiles; ++et)
-        *reinterpret_cast<f32x4*>(ws_mine + ((own_tile(w, i) * kCTiles + et) * 64 + lane) * 4) = S[i][et];
+      for (int et = 0; et < CT; ++et)
+        *reinterpret_cast<f32x4*>(ws_mine + ws_tile(own_tile(w, i), et)) = S[i][et];
     if constexpr (kNorm) {
-      *reinterpret_cast<f32x4*>(ws_mine + kWsK2 + lane * 4) = K2;
-      *reinterpret_cast<f32x4*>(ws_mine + kWsK1 + lane * 4) = K1;
+      // (every block's entry gets the normaliser state, so that the prefix pass reads nothing
+      // that was never written; the workgroup takes it from its first block's entry)
+#pragma unroll
+      for (int blk = 0; blk < CT / 4; ++blk) {
+        *reinterpret_cast<f32x4*>(ws_mine + blk * ws_block + kWsK2 + lane * 4) = K2;
+        *reinterpret_cast<f32x4*>(ws_mine + blk * ws_block + kWsK1 + lane * 4) = K1;
+      }
     }
     return;
   }
@@ -773,9 +820,9 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   // with the factor that undoes the packing weights), and the block, which is contiguous in
   // the decode state, leaves with coalesced 16-byte stores by the whole workgroup.
   if (kv_state != nullptr && last_seg) {
-    float* blk = reinterpret_cast<float*>(lds + kOffImg);
-    static_assert(16 * kExp * 4 <= kImgBytes, "expansion block must fit in a state image buffer");
-    static_for<kCTiles>([&](auto ET) {
+    float* blk = reinterpret_cast<float*>(lds + LD::kOffImg);
+    static_assert(16 * kExp * 4 <= LD::kImgBytes, "expansion block must fit in a state image buffer");
+    static_for<CT>([&](auto ET) {
       constexpr int et = decltype(ET)::value;
       if (16 * et >= live_ch) return;  // uniform over the workgroup (the readers count the same rounds)
       __syncthreads();  // the buffer is free (main loop done / previous block copied out)
@@ -826,24 +873,24 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 }
 #undef BASED_STAGE_END
 
-template <int MODE>
-__global__ __launch_bounds__(kThreads, 4) void lin_prefill_mfma_kernel(
+template <int MODE, int CT>
+__global__ __launch_bounds__(kThreads, CT == 4 ? 4 : 2) void lin_prefill_mfma_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
     int dv, long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh,
     long v_sl, long y_sb, long y_sh, long y_sl, float eps, float* __restrict__ ws, int seg_tokens, int n_seg) {
-  __shared__ __align__(16) unsigned char lds[kLdsBytes];
+  __shared__ __align__(16) unsigned char lds[PrefillLds<CT>::kBytes];
 #define BASED_CHAIN_ARGS lds, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh, \
                          k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, ws, seg_tokens, n_seg
   switch (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) {
-    case 0: lin_prefill_reader<0, MODE>(BASED_CHAIN_ARGS); break;
-    case 1: lin_prefill_reader<1, MODE>(BASED_CHAIN_ARGS); break;
-    case 2: lin_prefill_reader<2, MODE>(BASED_CHAIN_ARGS); break;
-    case 3: lin_prefill_reader<3, MODE>(BASED_CHAIN_ARGS); break;
-    case 4: lin_prefill_updater<0, MODE>(BASED_CHAIN_ARGS); break;
-    case 5: lin_prefill_updater<1, MODE>(BASED_CHAIN_ARGS); break;
-    case 6: lin_prefill_updater<2, MODE>(BASED_CHAIN_ARGS); break;
-    default: lin_prefill_updater<3, MODE>(BASED_CHAIN_ARGS); break;
+    case 0: lin_prefill_reader<0, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 1: lin_prefill_reader<1, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 2: lin_prefill_reader<2, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 3: lin_prefill_reader<3, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 4: lin_prefill_updater<0, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 5: lin_prefill_updater<1, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 6: lin_prefill_updater<2, MODE, CT>(BASED_CHAIN_ARGS); break;
+    default: lin_prefill_updater<3, MODE, CT>(BASED_CHAIN_ARGS); break;
   }
 #undef BASED_CHAIN_ARGS
 }
@@ -989,6 +1036,11 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // the last block of a head dim that is no multiple of 64 (112 = 64 + 48, the released 1B / 1.3B
 // models) runs with its missing tiles fed stand-in data and dropped at the stores.
 static bool prefill_mfma_takes(int64_t dv) { return dv >= 16 && dv <= 1024 && dv % 16 == 0; }
+// Head dims of 65..128 channels go to workgroups that carry both blocks of 64 (psi(q) and psi(k)
+// generated once per head instead of once per block).
+static bool prefill_wide(int64_t dv) { return dv > 64 && dv <= 128; }
+// workgroups per (batch, head)
+static int64_t prefill_workgroups_per_head(int64_t dv) { return prefill_wide(dv) ? 1 : (dv + 63) / 64; }
 
 }  // namespace based
 
@@ -1015,8 +1067,9 @@ extern "C" BASED_API int based_linear_attn_prefill(
     BASED_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y), BASED_ERR_ALIGN,
                   "linear_attn_prefill: tensors must be 16-byte aligned");
     BASED_REQUIRE(B * H * ((dv + 63) / 64) < (1ll << 31), BASED_ERR_SHAPE, "linear_attn_prefill: sizes too large");
-    dim3 grid((unsigned)(B * H * ((dv + 63) / 64))), block(kThreads);
-    hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeFull>, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
+    dim3 grid((unsigned)(B * H * prefill_workgroups_per_head(dv))), block(kThreads);
+    auto kern = prefill_wide(dv) ? lin_prefill_mfma_kernel<kModeFull, 8> : lin_prefill_mfma_kernel<kModeFull, 4>;
+    hipLaunchKernelGGL(kern, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
                        q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, (float*)nullptr, 0, 1);
     return check_launch("linear_attn_prefill");
@@ -1114,7 +1167,10 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   const int seg_tokens = (int)(seg_chunks * kChunk);
   dim3 block(kThreads);
   // pass 1: every segment but the last accumulates its own contribution to the state
-  hipLaunchKernelGGL(lin_prefill_mfma_kernel<kModeDelta>, dim3((unsigned)chains, 1, (unsigned)(n_seg - 1)),
+  const bool wide = prefill_wide(dv);
+  const unsigned wgs = (unsigned)(B * H * prefill_workgroups_per_head(dv));  // a wide workgroup carries two chains
+  auto kern_delta = wide ? lin_prefill_mfma_kernel<kModeDelta, 8> : lin_prefill_mfma_kernel<kModeDelta, 4>;
+  hipLaunchKernelGGL(kern_delta, dim3(wgs, 1, (unsigned)(n_seg - 1)),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
@@ -1130,7 +1186,9 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
     rc = check_launch(who);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(fold ? lin_prefill_mfma_kernel<kModeFromSum> : lin_prefill_mfma_kernel<kModeFrom>, dim3((unsigned)chains, 1, (unsigned)n_seg),
+  auto kern_from = fold ? (wide ? lin_prefill_mfma_kernel<kModeFromSum, 8> : lin_prefill_mfma_kernel<kModeFromSum, 4>)
+                        : (wide ? lin_prefill_mfma_kernel<kModeFrom, 8> : lin_prefill_mfma_kernel<kModeFrom, 4>);
+  hipLaunchKernelGGL(kern_from, dim3(wgs, 1, (unsigned)n_seg),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
