@@ -3,7 +3,8 @@
 // Kernels behind the entry points:
 //
 //  * lin_prefill_mfma_kernel (bf16 in/out): chunked scan, 64 tokens per chunk, one workgroup
-//    of EIGHT wavefronts per (batch, head, 64-channel block): four updaters keep the running
+//    of EIGHT wavefronts per (batch, head, 64-channel block) -- or per (batch, head) with both
+//    blocks when the head dim is 65..128 --: four updaters keep the running
 //    state in MFMA accumulators for the length of the sequence, split by feature slots, and
 //    publish a bf16 image of it in LDS once per chunk; four readers, split by tokens, compute
 //    the outputs from the chunk's rows and the image.  Small batches scan every sequence as
@@ -140,8 +141,10 @@ struct PrefillLds {
   static_assert(kBytes * (CT == 4 ? 2 : 1) <= 160 * 1024, "must fit the 160 KB of a compute unit");
 };
 
-// One chain = one (batch, head, 64-channel block), scanned in chunks of 64 tokens by a workgroup
-// of EIGHT wavefronts in two kinds of roles that run concurrently and meet at one barrier per
+// One chain = one (batch, head, 64-channel block); a workgroup scans one chain, or the two chains
+// of a head with 65..128 channels side by side (CT = 8 channel tiles: every per-tile array below
+// is twice as long, the roles and the stages are the same).  The scan runs in chunks of 64 tokens
+// on EIGHT wavefronts in two kinds of roles that run concurrently and meet at one barrier per
 // chunk:
 //   readers  (wavefronts 0..3, one per token tile of the chunk): O^T = V^T A^T + S^T psi(q)^T, the
 //            normaliser, the division and the store.  They read the chunk's rows and the bf16
@@ -205,8 +208,8 @@ __device__ __forceinline__ void interleave() {
       long q_sb, long q_sh, long q_sl, long k_sb, long k_sh, long k_sl, long v_sb, long v_sh, long v_sl, long y_sb,  \
       long y_sh, long y_sl, float eps, float *__restrict__ ws, int seg_tokens, int n_seg
 
-// Work item of this workgroup: item = (batch * H + head) * n_blocks + channel block, n_blocks =
-// ceil(dv / 64).  Workgroups are dealt to the 8 XCDs round-robin by workgroup id.  Items whose rows
+// Work item of this workgroup: item = (batch * H + head) * n_wb + workgroup of the head, n_wb =
+// ceil(dv / 64) workgroups of one channel block each, or 1 that carries both blocks (prefill_item).  Workgroups are dealt to the 8 XCDs round-robin by workgroup id.  Items whose rows
 // share cache lines (the channel blocks of one head read the same q and k rows, and for head dims
 // that are no multiple of 64 their v and y rows meet inside 128-byte lines; neighbouring heads of
 // one batch entry: 32-byte q / k rows 512 bytes apart) should sit behind the same L2 at about the
