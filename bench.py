@@ -44,11 +44,11 @@ D_EXP = 273
 # the same counter reads for a plain copy of known size (the summaries and the commands that
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": 293108326,   # B=128, H=16, dv=64, rotating state sets: fetch 146,970,214 + write 146,138,112
-    "lin_step_kernel_B64_dv128": 290387149,   # long-context decode: fetch 145,405,952 + write 144,981,197
-    "lin_prefill_mfma_kernel": {96: 2317252301},  # B=96, L=4096, dv=64, states written: fetch 1,402,835,354 + write 914,416,947; keyed by batch
+    "lin_step_kernel": 293110784,   # B=128, H=16, dv=64, rotating state sets: fetch 146,972,058 + write 146,138,726
+    "lin_step_kernel_B64_dv128": 290398618,   # long-context decode: fetch 145,408,410 + write 144,990,208
+    "lin_prefill_mfma_kernel": {96: 2197046579},  # B=96, L=4096, dv=64, states written: fetch 1,282,658,099 + write 914,388,480 (the fetch varies by 10 % between runs); keyed by batch
     "swa_prefill_kernel": 283241574,   # B=8, H=16, L=4096: fetch 216,132,198 + write 67,109,376
-    "decode_linear_kernel_lm_head": 104962356,   # M=4, 50280 x 1024 + closing norm: fetch 104,351,130 + write 611,226
+    "decode_linear_kernel_lm_head": 104965018,   # M=4, 50280 x 1024 + closing norm: fetch 104,353,382 + write 611,635
 }
 
 
