@@ -17,9 +17,10 @@
 //                   full 128-byte row.
 // Whole-window softmax in one pass: 80 (144) keys fit in registers, so no online rescaling.
 // A workgroup holds G such wavefront quartets, one per head of G heads that are neighbours in
-// memory (G = 2 when the head stride is 64 elements): their rows of one token are one contiguous
-// 128 G-byte piece, and HBM serves pieces of 256 bytes measurably better than pieces of 128
-// (a plain streaming kernel with this access pattern: 4.4 TB/s at 128 bytes, 4.9 at 256).
+// memory (G = 4 or 2 when the head stride is 64 elements; the launcher says which): their rows of
+// one token are one contiguous 128 G-byte piece, and HBM serves longer pieces measurably better
+// (a plain streaming kernel with this access pattern: 4.5 TB/s at 128 bytes, 5.1 at 256, 5.3 at
+// 512).
 // LDS rows are 128 bytes, unpadded; the 16-byte pieces of a row are XOR-swizzled by the row
 // number so that the operand reads (16 rows x 16 bytes, or 8 rows x 32 bytes for the transposing
 // read) fall on distinct banks.
@@ -86,7 +87,7 @@ constexpr int swa_head_lds_bytes(int nb, int g) { return (2 * nb + (g > 1 ? 1 : 
 // to a KV cache, the job of _update_kv_cache (slide_attention.py:255-281).
 // G > 1 needs q_sh == k_sh == v_sh == o_sh == c_sh == 64 and H % G == 0 (checked by the launcher).
 template <bool ROPE, int NB, int G>
-__global__ __launch_bounds__(256 * G, G == 2 ? 4 : (NB == 3 || ROPE ? 3 : 4)) void swa_prefill_kernel(
+__global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || ROPE ? 3 : 4)) void swa_prefill_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
@@ -759,7 +760,7 @@ static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int kMaxDevices = 64;
 // kernels asking for more than 64 KB of LDS have to be told once per device that they may
-static std::atomic<bool> g_big_lds_allowed[kMaxDevices][2 /*ROPE*/][2 /*NB - 2*/][2 /*G - 1*/];
+static std::atomic<bool> g_big_lds_allowed[kMaxDevices][2 /*ROPE*/][2 /*NB - 2*/][3 /*G = 1, 2, 4*/];
 
 }  // namespace based
 
@@ -805,18 +806,24 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   if (B == 0 || L == 0) return BASED_OK;
   const int64_t n_tiles = (L + kQTile - 1) / kQTile;
   BASED_REQUIRE(B * H * n_tiles < (1ll << 31), BASED_ERR_SHAPE, "swa_prefill: grid too large");
-  // Two heads per workgroup when they are neighbours in every tensor (the packed qkv layout) and
-  // the ring is the two-block one; the three-block ring keeps one head per workgroup (LDS).
+  // Heads that are neighbours in every tensor (the packed qkv layout) share a workgroup, so that
+  // every load and store instruction covers pieces of 128 G bytes.  Two-block ring: four heads
+  // (16 wavefronts, 160 KB of LDS: one workgroup per compute unit; 57.1 -> 53.9 us at B=8, H=16,
+  // L=4096 against two heads in each of two workgroups), else two.  Three-block ring (112 KB for
+  // two heads, one workgroup of 8 wavefronts per unit): two heads when the rows also go to a KV
+  // cache, whose 256-byte stores then pay for the lower occupancy (rotary + cache fill 108.5 ->
+  // 98.7 us), one head otherwise (three workgroups of 4 wavefronts: 64.2 against 66.7 us).
   const bool rope = rope_cos != nullptr;
   const int nb = w_left > 64 ? 3 : 2;
-  const bool pair = nb == 2 && H % 2 == 0 && q_sh == 64 && k_sh == 64 && v_sh == 64 && o_sh == 64 &&
+  const bool pair = H % 2 == 0 && q_sh == 64 && k_sh == 64 && v_sh == 64 && o_sh == 64 &&
                     (!kcache_out || c_sh == 64);
-  const int g = pair ? 2 : 1;
+  const int g = !pair ? 1 : (nb == 2 ? (H % 4 == 0 ? 4 : 2) : (kcache_out ? 2 : 1));
   // Consecutive query tiles of one (batch, head) are walked by one workgroup (the keys to the left
   // of a tile are the previous tile's own keys, already staged).  Runs are as long as still gives
   // every resident slot of the GPU one run: 256 compute units x the wavefront quartets that fit
-  // one (4 by registers; 3 for the three-block ring, by LDS, and for the single-head rotary variant).
-  const int64_t slots = 256 * ((nb == 3 || (g == 1 && rope)) ? 3 : 4);
+  // one (4 by registers; for the three-block ring, by LDS, 3 of one head or 2 of a pair; 3 for the
+  // single-head rotary variant).
+  const int64_t slots = 256 * (nb == 3 ? (g == 2 ? 2 : 3) : ((g == 1 && rope) ? 3 : 4));
   int64_t want_runs = slots / (B * H);
   want_runs = want_runs < 1 ? 1 : (want_runs > n_tiles ? n_tiles : want_runs);
   const int64_t run_tiles = (n_tiles + want_runs - 1) / want_runs;
@@ -826,7 +833,9 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
                         long, long, long, long, long, long, long, long, int, float, const float*, const float*, __bf16*,
                         __bf16*, long, long, long);
   Kern kern;
-  if (nb == 3) kern = rope ? swa_prefill_kernel<true, 3, 1> : swa_prefill_kernel<false, 3, 1>;
+  if (nb == 3 && g == 2) kern = rope ? swa_prefill_kernel<true, 3, 2> : swa_prefill_kernel<false, 3, 2>;
+  else if (nb == 3) kern = rope ? swa_prefill_kernel<true, 3, 1> : swa_prefill_kernel<false, 3, 1>;
+  else if (g == 4) kern = rope ? swa_prefill_kernel<true, 2, 4> : swa_prefill_kernel<false, 2, 4>;
   else if (g == 2) kern = rope ? swa_prefill_kernel<true, 2, 2> : swa_prefill_kernel<false, 2, 2>;
   else kern = rope ? swa_prefill_kernel<true, 2, 1> : swa_prefill_kernel<false, 2, 1>;
   const size_t lds = (size_t)g * swa_head_lds_bytes(nb, g);
@@ -834,7 +843,7 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
     int dev = 0;
     BASED_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices, BASED_ERR_LAUNCH,
                   "swa_prefill: cannot identify the current device");
-    std::atomic<bool>& allowed = g_big_lds_allowed[dev][rope][nb - 2][g - 1];
+    std::atomic<bool>& allowed = g_big_lds_allowed[dev][rope][nb - 2][g == 4 ? 2 : g - 1];
     if (!allowed.load(std::memory_order_acquire)) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -322,6 +322,10 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     last-level cache) and WARM on one; the roofline figure is the lower of the two."""
     dev = torch.device("cuda:0")
     g = torch.Generator(device="cpu").manual_seed(2)
+    # every prefill leg below is timed after 20 ms of its own launches, like the linear-attention
+    # prefill: the first millisecond after an idle period runs at another clock and memory state
+    # than a serving loop sees (head dim 112: 157 us in that transient, 139 us after it)
+    SWA_WARMUP_MS = 20.0
     qkvs = [torch.randn(B, L, 3, H, 64, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
     outs = [torch.empty(B, L, H, 64, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
     qkv = qkvs[0]
@@ -334,8 +338,8 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
             ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=64, out=o)
         return pf
 
-    ms_cold, _ = _events_ms(torch, make_pf(n_sets), steps, warmup)
-    ms_warm, _ = _events_ms(torch, make_pf(1), steps, warmup)
+    ms_cold, _ = _events_ms(torch, make_pf(n_sets), steps, warmup, warmup_ms=SWA_WARMUP_MS)
+    ms_warm, _ = _events_ms(torch, make_pf(1), steps, warmup, warmup_ms=SWA_WARMUP_MS)
     ms = max(ms_cold, ms_warm)
     byts = B * L * H * 4 * 64 * 2
     gbs = byts / (ms * 1e-3) / 1e9
@@ -356,9 +360,9 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
                 ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=128, out=outs[i])
         return pf
 
-    ms_w128_cold, _ = _events_ms(torch, make_rel(n_sets, False), steps, warmup)
-    ms_w128_warm, _ = _events_ms(torch, make_rel(1, False), steps, warmup)
-    ms_rel_cold, _ = _events_ms(torch, make_rel(n_sets, True), steps, warmup)
+    ms_w128_cold, _ = _events_ms(torch, make_rel(n_sets, False), steps, warmup, warmup_ms=SWA_WARMUP_MS)
+    ms_w128_warm, _ = _events_ms(torch, make_rel(1, False), steps, warmup, warmup_ms=SWA_WARMUP_MS)
+    ms_rel_cold, _ = _events_ms(torch, make_rel(n_sets, True), steps, warmup, warmup_ms=SWA_WARMUP_MS)
     del caches
     # the released 1B / 1.3B window layer: head dim 112 (n_embd 1792 over 16 heads), 128 keys to the left,
     # rotary over the whole head, KV cache filled; the general MFMA kernel
@@ -381,8 +385,8 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
                 ops.swa_prefill(x[:, :, 0], x[:, :, 1], x[:, :, 2], w_left=128, out=o1b[i])
         return pf
 
-    ms_1b_plain, _ = _events_ms(torch, make_1b(False), steps, warmup)
-    ms_1b_full, _ = _events_ms(torch, make_1b(True), steps, warmup)
+    ms_1b_plain, _ = _events_ms(torch, make_1b(False), steps, warmup, warmup_ms=SWA_WARMUP_MS)
+    ms_1b_full, _ = _events_ms(torch, make_1b(True), steps, warmup, warmup_ms=SWA_WARMUP_MS)
     byts_1b = B * L * H * 4 * D1 * 2
     del x1, o1b, c1b
     cache = torch.zeros(B, L + decode_steps, 2, H, 64, dtype=torch.bfloat16, device=dev)
