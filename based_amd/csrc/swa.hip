@@ -152,21 +152,32 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
   // instruction covering whole 128 G-byte pieces of memory.
   //   plain: instruction i of 2 moves 8/G rows x G heads x 8 pieces
   //   ROPE : one row per 4 G lanes, pieces p and p + 4 (the channel pairs of the rotation)
+  // V rows are never rotated: with the three-block ring they move in the plain arrangement (whole
+  // rows per load and per cache store) also in the ROPE variant (rotary + cache fill at 128 keys
+  // to the left 99.0 -> 94.8 us); with the two-block ring they follow K's arrangement (the plain
+  // one measures 1 % slower there).
+  constexpr bool kPlainV = !ROPE || NB == 3;
   const int mv_head = ROPE ? (lane >> 2) % G : (lane >> 3) % G;
+  const int mv_head_v = kPlainV ? (lane >> 3) % G : mv_head;
   auto piece_row = [&](int i) {
     return ROPE ? 16 * wq + (16 / G) * hsel + lane / (4 * G) : 16 * wq + (16 / G) * hsel + (8 / G) * i + lane / (8 * G);
   };
   auto piece_idx = [&](int i) { return ROPE ? (lane & 3) + 4 * i : (lane & 7); };
+  auto piece_row_v = [&](int i) {
+    return kPlainV ? 16 * wq + (16 / G) * hsel + (8 / G) * i + lane / (8 * G) : piece_row(i);
+  };
+  auto piece_idx_v = [&](int i) { return kPlainV ? (lane & 7) : piece_idx(i); };
   const __bf16* const q_mv = q + b * q_sb + (head0 + mv_head) * q_sh;
   const __bf16* const k_mv = k + b * k_sb + (head0 + mv_head) * k_sh;
-  const __bf16* const v_mv = v + b * v_sb + (head0 + mv_head) * v_sh;
+  const __bf16* const v_mv = v + b * v_sb + (head0 + mv_head_v) * v_sh;
   __bf16* kc_mv = nullptr;
   __bf16* vc_mv = nullptr;
   if (kc_out != nullptr) {
     kc_mv = kc_out + b * c_sb + (head0 + mv_head) * c_sh;
-    vc_mv = vc_out + b * c_sb + (head0 + mv_head) * c_sh;
+    vc_mv = vc_out + b * c_sb + (head0 + mv_head_v) * c_sh;
   }
   unsigned char* const mv_lds = swa_lds + mv_head * kHeadBytes;
+  unsigned char* const mv_lds_v = swa_lds + mv_head_v * kHeadBytes;
   __bf16* const o_my = o + b * o_sb + (head0 + hsel) * o_sh;
 
   // No load sits under a condition (a load in a branch is waited for at the end of the branch,
@@ -179,7 +190,9 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
       int key = key0 + piece_row(i);
       key = key < 0 ? 0 : (key < L ? key : L - 1);
       r.kp[i] = *reinterpret_cast<const u32x4*>(k_mv + (long)key * k_sl + 8 * piece_idx(i));
-      r.vp[i] = *reinterpret_cast<const u32x4*>(v_mv + (long)key * v_sl + 8 * piece_idx(i));
+      int key_v = key0 + piece_row_v(i);
+      key_v = key_v < 0 ? 0 : (key_v < L ? key_v : L - 1);
+      r.vp[i] = *reinterpret_cast<const u32x4*>(v_mv + (long)key_v * v_sl + 8 * piece_idx_v(i));
       if constexpr (QLDS)
         if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q_mv + (long)key * q_sl + 8 * piece_idx(i));  // a literal at every call
     }
@@ -206,14 +219,28 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
       const int lrow = piece_row(i);
       const int row = blk * kQTile + lrow;
       const int pc = piece_idx(i);
+      const int lrow_v = piece_row_v(i);
       *reinterpret_cast<u32x4*>(mv_lds + row * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.kp[i];
-      *reinterpret_cast<u32x4*>(mv_lds + kOffV + row * kRowBytes + ((pc ^ swz_v(lrow)) << 4)) = r.vp[i];
+      *reinterpret_cast<u32x4*>(mv_lds_v + kOffV + (blk * kQTile + lrow_v) * kRowBytes + ((piece_idx_v(i) ^ swz_v(lrow_v)) << 4)) = r.vp[i];
       if constexpr (QLDS)
         if (own_rows) *reinterpret_cast<u32x4*>(mv_lds + kOffQ + lrow * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.qp[i];
+      // Cache rows leave non-temporally where an instruction writes whole rows (the plain
+      // arrangement); rows in the rotary arrangement leave as two half rows from two instructions,
+      // which the cache has to merge (non-temporal there: 99 -> 103 us at 128 keys to the left).
       const int key = key0 + lrow;
-      if (own_rows && kc_mv != nullptr && key < L) {
-        *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
-        *reinterpret_cast<u32x4*>(vc_mv + (long)key * c_st + 8 * pc) = r.vp[i];
+      if constexpr (!kPlainV) {  // K and V in one arrangement: one condition
+        if (own_rows && kc_mv != nullptr && key < L) {
+          *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
+          *reinterpret_cast<u32x4*>(vc_mv + (long)key * c_st + 8 * pc) = r.vp[i];
+        }
+      } else if (own_rows && kc_mv != nullptr) {
+        const int key_v = key0 + lrow_v;
+        if (key < L) {
+          if constexpr (ROPE) *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
+          else __builtin_nontemporal_store(r.kp[i], reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc));
+        }
+        if (key_v < L)
+          __builtin_nontemporal_store(r.vp[i], reinterpret_cast<u32x4*>(vc_mv + (long)key_v * c_st + 8 * piece_idx_v(i)));
       }
     }
   };
