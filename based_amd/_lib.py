@@ -75,6 +75,7 @@ SIGNATURES = {
         [_P] * 6 + [_P, _I64] + [_I64] * 4 + [_I64] * 8 + [_I64] * 3 + [C.c_int, C.c_float]
         + [_P, _P, _I64, _I64, C.c_int] + [C.c_int, _P],
     ),
+    "based_greedy_step": (C.c_int, [_P, _I64, _I64, _I64, _P, _I64, _P, _I64, _I64, _P, _P, _I64, C.c_int, _P]),
     "based_swa_step_anydim": (
         C.c_int,
         [_P] * 6 + [_P, _I64] + [_I64] * 4 + [_I64] * 8 + [_I64] * 3 + [C.c_int, C.c_float, C.c_int, _P],

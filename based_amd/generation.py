@@ -86,13 +86,18 @@ class DecodingGraphCache:
     mempool: Optional[tuple] = None
     inference_params: Optional[InferenceParams] = None
     run: Optional[Callable] = None
+    # greedy decoding with the sampling inside the graph: recorded graphs keyed by (batch_size,
+    # vocab_size) and the (max_batch_size, max_seqlen) buffer they write the sequences to
+    greedy_graphs: dict = field(default_factory=dict)
+    sequences: Optional[Tensor] = None
 
 
 @torch.inference_mode()
-def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, dtype=None, n_warmups=2):
+def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, dtype=None, n_warmups=2, capture=True):
     """Returns a cache whose graphs fit (batch_size, max_seqlen); a larger batch, a longer
     max_seqlen or another device/dtype throws the old graphs and caches away (reference
-    update_graph_cache, :613-680)."""
+    update_graph_cache, :613-680).  capture=False only sets up the caches (the caller records
+    a graph of its own on them)."""
     if cache is None:
         cache = DecodingGraphCache()
     param = next(iter(model.parameters()))
@@ -101,6 +106,8 @@ def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, dtype=No
     if ((device, dtype) != (cache.device, cache.dtype) or batch_size > cache.max_batch_size
             or max_seqlen > cache.max_seqlen):
         cache.callables = {}
+        cache.greedy_graphs = {}
+        cache.sequences = None
         cache.mempool = None
         cache.inference_params = None
         gc.collect()
@@ -112,7 +119,7 @@ def update_graph_cache(model, cache, batch_size, seqlen_og, max_seqlen, dtype=No
                                                  seqlen_offset=seqlen_og, key_value_memory_dict=inf_cache,
                                                  lengths_per_sample=lengths)
         cache.mempool = torch.cuda.graphs.graph_pool_handle()
-    if (batch_size, 1) not in cache.callables:
+    if capture and (batch_size, 1) not in cache.callables:
         cache.callables[batch_size, 1] = capture_graph(model, cache.inference_params, batch_size, cache.max_seqlen,
                                                        mempool=cache.mempool, n_warmups=n_warmups)
 
@@ -160,14 +167,97 @@ def capture_graph(model, inference_params, batch_size, max_seqlen, mempool=None,
     return run
 
 
+def capture_greedy_graph(model, inference_params, sequences, batch_size, max_seqlen, vocab_size=None, mempool=None,
+                         n_warmups=2):
+    """Records one single-token step of the model TOGETHER with the greedy choice of the next
+    token (`ops.greedy_step`): a replay reads the token in the graph's input buffer at the
+    device-side position `lengths_per_sample`, and leaves the next token in that buffer and in
+    `sequences`, with the positions advanced.  A decoding loop is then one replay per token and
+    nothing else: no argmax kernel, no copies of ids / positions / lengths, no logits clone.
+    Returns (graph, input_ids, position_ids)."""
+    from . import ops
+
+    device = next(iter(model.parameters())).device
+    input_ids = torch.zeros(batch_size, 1, dtype=torch.long, device=device)
+    position_ids = torch.zeros(batch_size, 1, dtype=torch.long, device=device)
+    lengths = inference_params.lengths_per_sample
+    seq = sequences[:batch_size]
+    offset_og = inference_params.seqlen_offset
+    inference_params.seqlen_offset = max_seqlen - 1
+
+    def step():
+        logits = model(input_ids, position_ids=position_ids, inference_params=inference_params,
+                       num_last_tokens=1).logits.squeeze(dim=1)
+        ops.greedy_step(logits, input_ids, lengths[:batch_size], sequences=seq, position_ids=position_ids,
+                        vocab_size=vocab_size)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(n_warmups):
+            lengths[:] = max_seqlen - 1   # (a step at the last position writes no sequence entry)
+            input_ids.zero_()
+            step()
+        side.synchronize()
+    torch.cuda.current_stream().wait_stream(side)
+    lengths[:] = max_seqlen - 1
+    input_ids.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, pool=mempool):
+        step()
+    inference_params.seqlen_offset = offset_og
+    return graph, input_ids, position_ids
+
+
+def _decode_greedy_in_graph(input_ids, model, max_length, vocab_size=None) -> DecodeOutput:
+    """Greedy decoding with one graph replay per token (capture_greedy_graph); same sequences as
+    `decode(..., top_k=1, cg=True)`, no scores."""
+    from . import ops
+
+    batch_size, seqlen_og = input_ids.shape
+    if not hasattr(model, "_decoding_cache"):
+        model._decoding_cache = None
+    cache = model._decoding_cache = update_graph_cache(model, model._decoding_cache, batch_size, seqlen_og, max_length,
+                                                       capture=False)
+    inference_params = cache.inference_params
+    inference_params.reset(max_length, batch_size)
+    if cache.sequences is None:
+        cache.sequences = torch.zeros(cache.max_batch_size, cache.max_seqlen, dtype=torch.long, device=input_ids.device)
+    key = (batch_size, vocab_size)
+    if key not in cache.greedy_graphs:
+        cache.greedy_graphs[key] = capture_greedy_graph(model, inference_params, cache.sequences, batch_size,
+                                                        cache.max_seqlen, vocab_size=vocab_size, mempool=cache.mempool)
+    graph, step_ids, step_pos = cache.greedy_graphs[key]
+    seq = cache.sequences[:batch_size]
+    lengths = inference_params.lengths_per_sample[:batch_size]
+    seq[:, :seqlen_og] = input_ids
+    inference_params.seqlen_offset = 0
+    if max_length > seqlen_og:
+        logits = model(input_ids, inference_params=inference_params, num_last_tokens=1).logits[:, -1]
+        inference_params.seqlen_offset = seqlen_og
+        # the first new token comes from the prefill's logits; from then on the graph feeds itself
+        inference_params.lengths_per_sample[:] = seqlen_og - 1
+        ops.greedy_step(logits.contiguous(), step_ids, lengths, sequences=seq, position_ids=step_pos,
+                        vocab_size=vocab_size)
+        for _ in range(max_length - seqlen_og - 1):
+            graph.replay()
+        inference_params.seqlen_offset = max_length - 1
+    return DecodeOutput(sequences=seq[:, :max(max_length, seqlen_og)].clone(), scores=())
+
+
 @torch.inference_mode()
 def decode(input_ids, model, max_length, top_k=1, top_p=0.0, temperature=1.0, eos_token_id=None,
-           teacher_outputs=None, vocab_size=None, cg=False, **kwargs) -> DecodeOutput:
+           teacher_outputs=None, vocab_size=None, cg=False, output_scores=True, **kwargs) -> DecodeOutput:
     """Prefill on `input_ids` (batch, seq_len), then one token at a time up to max_length.
     Same control flow as the reference's `decode`; cg=True replays a recorded graph for every
-    token after the prefill."""
+    token after the prefill.  Greedy decoding under cg=True that needs no scores, no stopping
+    token and no teacher tokens (output_scores=False) takes the sampling into the graph as well:
+    one replay per token."""
     batch_size, seqlen_og = input_ids.shape
     teacher_len = teacher_outputs.shape[1] if teacher_outputs is not None else 0
+    if (cg and top_k == 1 and not output_scores and eos_token_id is None and teacher_outputs is None
+            and max_length > seqlen_og):
+        return _decode_greedy_in_graph(input_ids, model, max_length, vocab_size=vocab_size)
     if cg:
         if not hasattr(model, "_decoding_cache"):
             model._decoding_cache = None
@@ -218,7 +308,8 @@ class GenerationMixin:
 
     def generate(self, input_ids, max_length, top_k=1, top_p=0.0, temperature=1.0,
                  return_dict_in_generate=False, output_scores=False, **kwargs):
-        out = decode(input_ids, self, max_length, top_k=top_k, top_p=top_p, temperature=temperature, **kwargs)
+        out = decode(input_ids, self, max_length, top_k=top_k, top_p=top_p, temperature=temperature,
+                     output_scores=output_scores, **kwargs)
         if not output_scores:
             out.scores = None
         return out if return_dict_in_generate else out.sequences

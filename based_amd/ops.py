@@ -544,6 +544,41 @@ def swiglu(u) -> torch.Tensor:
     return out.view(*u.shape[:-1], F)
 
 
+def greedy_step(logits, next_ids, lengths, sequences=None, position_ids=None, vocab_size=None) -> None:
+    """Greedy sampling of one decoding step plus the loop's bookkeeping, in one launch (recordable
+    in the decode graph): per row b, tok = argmax(logits[b, :vocab_size]) (first index of the
+    maximum, NaN largest, as torch.argmax), written to next_ids[b] and to
+    sequences[b, lengths[b] + 1]; lengths[b] and position_ids[b] advance by one.
+
+    logits (B, V) bf16 / fp32 with contiguous rows; next_ids (B,) or (B, 1) int64; lengths (B,)
+    int32; sequences (B, max_length) int64 or None; position_ids (B,) or (B, 1) int64 or None."""
+    _require_cuda(logits, next_ids, lengths)
+    if logits.ndim != 2 or logits.stride(-1) != 1:
+        raise ValueError("logits must be (B, V) with contiguous rows")
+    B, V = logits.shape
+    V = V if vocab_size is None else int(vocab_size)
+    if not 0 < V <= logits.shape[1]:
+        raise ValueError(f"vocab_size {V} outside (0, {logits.shape[1]}]")
+    if next_ids.dtype != torch.int64 or next_ids.numel() != B or lengths.dtype != torch.int32 or lengths.numel() != B \
+            or not lengths.is_contiguous():
+        raise ValueError("next_ids must hold B int64 values, lengths B contiguous int32 values")
+    for t, name in ((sequences, "sequences"), (position_ids, "position_ids")):
+        if t is not None and (t.dtype != torch.int64 or t.shape[0] != B or not t.is_cuda):
+            raise ValueError(f"{name} must be an int64 device tensor with B rows")
+    if sequences is not None and (sequences.ndim != 2 or sequences.stride(1) != 1):
+        raise ValueError("sequences must be (B, max_length) with contiguous rows")
+    if position_ids is not None and position_ids.numel() != B:
+        raise ValueError("position_ids must hold B values")
+    with _on_device(logits.device):
+        _lib.check(_lib.lib().based_greedy_step(
+            logits.data_ptr(), B, V, logits.stride(0), next_ids.data_ptr(), next_ids.stride(0),
+            sequences.data_ptr() if sequences is not None else None,
+            sequences.stride(0) if sequences is not None else 0,
+            sequences.shape[1] if sequences is not None else 0, lengths.data_ptr(),
+            position_ids.data_ptr() if position_ids is not None else None,
+            position_ids.stride(0) if position_ids is not None else 0, _dtype_code(logits), _stream_ptr(logits)))
+
+
 DECODE_LINEAR_MAX_ROWS = 32  # BASED_DECODE_LINEAR_MAX_ROWS of include/based_hip.h
 PROLOGUE_NONE, PROLOGUE_ADD_RMS_NORM, PROLOGUE_SWIGLU = 0, 1, 2
 EPILOGUE_NONE, EPILOGUE_SWIGLU, EPILOGUE_GATED_CONV_STEP = 0, 1, 2

@@ -565,6 +565,7 @@ def bench_stack(torch, B=4, prefill_len=2048, new_tokens=128, released=False):
         ms_tok = (total - out["prefill_ms"]) / new_tokens
         out[f"decode_{name}_ms_per_token"] = ms_tok
         out[f"decode_{name}_tok_s"] = B / (ms_tok * 1e-3)
+    out["decode_graph_note"] = "greedy sampling recorded in the graph (based_greedy_step): one replay per token"
     return out
 
 

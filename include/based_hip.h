@@ -441,6 +441,26 @@ BASED_API int based_swa_step_anydim(const void* q, const void* k_new, const void
                           int64_t c_sb, int64_t c_st, int64_t c_sh,
                           int w_left, float scale, int io_dtype, void* stream);
 
+/*
+ * Greedy sampling of one decoding step and the bookkeeping of the loop around it, in one launch
+ * that can be recorded in the same graph as the step: replaces sample(logits, top_k=1) =
+ * logits.argmax(dim=-1) (based/generation.py:64-70), the append of the token to the sequences
+ * and the advance of seqlen_offset (generation.py:190-204), and the copies of the next input ids,
+ * position ids and lengths_per_sample into the recorded graph's static tensors
+ * (generation.py:725-735).  Per batch row b:
+ *   tok = first index of the largest of logits[b, 0..V) (NaN counts as the largest, as torch.argmax)
+ *   p = lengths[b]                       position of the token the step just processed
+ *   next_ids[b * ids_stride] = tok       the next step's input
+ *   sequences[b * seq_stride + p + 1] = tok   (skipped when sequences is NULL or p + 1 >= seq_len)
+ *   lengths[b] = p + 1;  position_ids[b * pos_stride] = p + 1 (position_ids may be NULL)
+ * logits: bf16 or fp32, row stride logits_stride elements (>= V); ids and positions int64,
+ * lengths int32.
+ */
+BASED_API int based_greedy_step(const void* logits, int64_t B, int64_t V, int64_t logits_stride,
+                                int64_t* next_ids, int64_t ids_stride, int64_t* sequences,
+                                int64_t seq_stride, int64_t seq_len, int32_t* lengths,
+                                int64_t* position_ids, int64_t pos_stride, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
