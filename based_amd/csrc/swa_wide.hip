@@ -6,7 +6,9 @@
 //
 // Prefill.  Four wavefronts cover 64 consecutive queries of one (batch, head); wavefront w owns
 // queries [q0 + 16 w, q0 + 16 w + 16) and sees the staged keys 16 w .. 16 w + 16 NT - 1 of a ring
-// of NB blocks of 64 K rows and 64 V rows (NB = 2: up to 64 keys to the left, NB = 3: up to 128).
+// of blocks of 64 K rows and 64 V rows (NB = 2: up to 64 keys to the left, NB = 3: up to 128).
+// With NB = 3 a workgroup is eight wavefronts on two neighbouring tiles that share the blocks to
+// their left (a ring of four blocks).
 //   S^T = K Q^T   : NT key tiles x 2 or 4 MFMA 16x16x32 (head dims up to 64 / 128); K and Q rows are staged in LDS
 //                   (rotated on the way in), a lane's operand = 8 consecutive bf16 of one row.
 //   softmax       : whole window in one pass, lane <-> query, registers <-> keys.
@@ -78,7 +80,8 @@ struct WideRows {
   f32x4 cs[2][2], sn[2][2];            // rotary factors of the row's position (RMODE != 0)
 };
 
-constexpr int wide_lds_bytes(int nb) { return (2 * nb + 1) * kWQTile * kWRowBytes; }
+// ring of nb - 1 + qt blocks of K rows and of V rows, qt blocks of query rows
+constexpr int wide_lds_bytes(int nb, int qt) { return (2 * (nb - 1 + qt) + qt) * kWQTile * kWRowBytes; }
 
 // RMODE: rotary layout (kRopeNone / kRopeHalf / kRopeInterleaved) over the first R channels, cos/sin
 // tables of R/2 frequencies per position (slide_attention.py:346-355,553-556); kc_out / vc_out
@@ -86,8 +89,12 @@ constexpr int wide_lds_bytes(int nb) { return (2 * nb + 1) * kWQTile * kWRowByte
 // (_update_kv_cache, slide_attention.py:255-281).
 // NDS: contraction steps of 32 channels (head dims up to 32 NDS); a compile-time count keeps the
 // products free of branches, so that the operand reads of one MFMA travel under the others.
-template <int RMODE, int NB, int NDS>
-__global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
+// QT: tiles of 64 queries a workgroup of 4 QT wavefronts works on at a time (run_tiles is a
+// multiple of it).  With the three-block window a lone tile's ring fills a compute unit's LDS
+// share with four wavefronts; two tiles side by side share the window's blocks (four ring blocks
+// instead of twice three: 160 KB), so that every SIMD has two wavefronts to switch between.
+template <int RMODE, int NB, int NDS, int QT>
+__global__ __launch_bounds__(256 * QT, QT == 2 || NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ o, int H, int L, int D, int n_tiles, int run_tiles, long q_sb, long q_sl, long q_sh,
     long k_sb, long k_sl, long k_sh, long v_sb, long v_sl, long v_sh, long o_sb, long o_sl, long o_sh,
@@ -95,14 +102,19 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     __bf16* __restrict__ kc_out, __bf16* __restrict__ vc_out, long c_sb, long c_st, long c_sh) {
   constexpr int NT = 4 * (NB - 1) + 1;   // key tiles of 16 a wavefront sees
   constexpr int NS = (NT + 1) / 2;       // key slabs of 32 in the second product (last one half empty)
-  constexpr int kOffV = NB * kWQTile * kWRowBytes;
+  static_assert((NB - 1) % QT == 0, "the keys to the left are loaded in pieces of QT blocks");
+  constexpr int NBR = NB - 1 + QT;       // ring blocks
+  constexpr int kSuper = QT * kWQTile;   // queries (and new key rows) per step of the workgroup
+  constexpr int kOffV = NBR * kWQTile * kWRowBytes;
   constexpr int kOffQ = 2 * kOffV;
   extern __shared__ __align__(16) unsigned char swa_wide_lds[];
   unsigned char* const lds = swa_wide_lds;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wq = __builtin_amdgcn_readfirstlane(tid >> 6);  // which 16 of the tile's 64 queries
+  const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);  // which 16 of the step's 64 QT queries
+  const int wt = w8 >> 2;                                   // which tile of the step
+  const int wq = w8 & 3;                                    // which 16 of the tile's 64 queries
   const int col = lane & 15;
   const int grp = lane >> 4;
   const int np = D >> 3;            // live 16-byte pieces of a row
@@ -125,7 +137,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
   const int tile_begin = run * run_tiles;
   const int tile_end = tile_begin + run_tiles < n_tiles ? tile_begin + run_tiles : n_tiles;
 
-  // Pieces moved by this thread: rows 16 wq + lane / 8 (+ 8), piece pair `slot` = lane % 8.
+  // Pieces moved by this thread: rows 16 w8 + lane / 8 (+ 8) of a step's 64 QT, piece pair `slot` = lane % 8.
   //   half-split rotary: slot s < R/16 is the pair (s, s + R/16) that the rotation combines
   //     (channels c and c + R/2); the other slots carry the unrotated pieces past R, two by two;
   //   otherwise: slot s = pieces 2 s, 2 s + 1 (interleaved pairs sit inside one piece).
@@ -148,7 +160,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
   const bool rot = RMODE != kRopeNone && slot < r16;
   const bool va = pa < np, vb = pb < np;
   const int pa_ld = va ? 8 * pa : 0, pb_ld = vb ? 8 * pb : 0;   // element offsets of the loads (always inside the row)
-  const int row_lo = 16 * wq + (lane >> 3);
+  const int row_lo = 16 * w8 + (lane >> 3);
   const __bf16* const q_mv = q + b * q_sb + h * q_sh;
   const __bf16* const k_mv = k + b * k_sb + h * k_sh;
   const __bf16* const v_mv = v + b * v_sb + h * v_sh;
@@ -186,7 +198,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     }
   };
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
-  // own_rows: the rows are the tile's own keys (they also carry its queries and go to the cache)
+  // own_rows: the rows are the step's own keys (they also carry its queries and go to the cache);
+  // they go to the QT ring blocks from blk on
   auto store_rows = [&](int blk, int key0, WideRows& r, bool own_rows) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -210,7 +223,9 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
       if (!va) r.kp[i][0] = r.vp[i][0] = r.qp[i][0] = zero4;
       if (!vb) r.kp[i][1] = r.vp[i][1] = r.qp[i][1] = zero4;
       const int lrow = row_lo + 8 * i;
-      const int row = blk * kWQTile + lrow;
+      int rblk = blk + (lrow >> 6);
+      rblk = rblk >= NBR ? rblk - NBR : rblk;
+      const int row = rblk * kWQTile + (lrow & (kWQTile - 1));
       *reinterpret_cast<u32x4*>(lds + row * kWRowBytes + (wide_swz_k(lrow, pa) << 4)) = r.kp[i][0];
       *reinterpret_cast<u32x4*>(lds + row * kWRowBytes + (wide_swz_k(lrow, pb) << 4)) = r.kp[i][1];
       *reinterpret_cast<u32x4*>(lds + kOffV + row * kWRowBytes + (wide_swz_v(lrow, pa) << 4)) = r.vp[i][0];
@@ -236,23 +251,26 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
   int q0 = tile_begin * kWQTile;
   WideRows pre;
   {
-    // first tile: own rows in block 0, the keys 64 a to the left in block NB - a (one round trip)
-    WideRows left[NB - 1];
+    // first step: own rows in blocks 0 .. QT - 1, the keys 64 QT a to the left in the blocks from
+    // NBR - QT a on (one round trip)
+    constexpr int kLeft = (NB - 1) / QT;
+    WideRows left[kLeft];
 #pragma unroll
-    for (int a = 1; a < NB; ++a) load_rows(q0 - a * kWQTile, left[a - 1], false);
+    for (int a = 1; a <= kLeft; ++a) load_rows(q0 - a * kSuper, left[a - 1], false);
     load_rows(q0, pre, true);
 #pragma unroll
-    for (int a = 1; a < NB; ++a) store_rows(NB - a, q0 - a * kWQTile, left[a - 1], false);
+    for (int a = 1; a <= kLeft; ++a) store_rows(NBR - a * QT, q0 - a * kSuper, left[a - 1], false);
     store_rows(0, q0, pre, true);
   }
-  if (tile_begin + 1 < tile_end) load_rows(q0 + kWQTile, pre, true);  // travels while this tile is computed
+  if (tile_begin + QT < tile_end) load_rows(q0 + kSuper, pre, true);  // travels while this step is computed
   // The three-block ring leaves room for one workgroup per compute unit (112 KB of LDS), i.e. one
   // wavefront per SIMD with the whole register file to itself and nobody to cover its memory
   // round trips: it keeps the rows of TWO tiles in flight (a second register set).
-  constexpr int DEPTH = NB == 3 ? 2 : 1;
+  // (two wavefronts per SIMD have 256 registers each: the rotary factors of a second set do not fit)
+  constexpr int DEPTH = NB == 3 && !(QT == 2 && RMODE != kRopeNone) ? 2 : 1;
   WideRows pre2;
   if constexpr (DEPTH == 2)
-    if (tile_begin + 2 < tile_end) load_rows(q0 + 2 * kWQTile, pre2, true);
+    if (tile_begin + 2 * QT < tile_end) load_rows(q0 + 2 * kSuper, pre2, true);
 
   // lane-constant parts of the operand addresses (a tile's rows start at multiples of 16, so
   // row & 15 == col for the operand rows and row & 7 == vt_row & 7 for the transposed ones)
@@ -262,19 +280,20 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
   const int v_half = (col & 3) >> 1;
 
   const int i_win = w_left >= 64 * (NB - 1) + 15 ? 0 : (64 * (NB - 1) + 30 - w_left) >> 4;
-  int own = 0;  // ring block with keys [q0, q0 + 64); block own + 1 (mod NB) is the oldest
-  // one tile; `nxt` holds the rows of tile + 1 and is refilled with those of tile + 1 + DEPTH
+  int own = 0;  // ring block with keys [q0, q0 + 64); block own + QT (mod NBR) is the oldest
+  // one step of QT tiles; `nxt` holds the rows of the next step and is refilled with those DEPTH steps later
   auto do_tile = [&](int tile, WideRows& nxt) {
-    const int oldest = own + 1 == NB ? 0 : own + 1;
-    const int n0 = q0 + 16 * wq;
+    const int oldest = own + QT >= NBR ? own + QT - NBR : own + QT;
+    const int x0 = 64 * wt + 16 * wq;   // first staged key this wavefront sees = its first query's place in the step
+    const int n0 = q0 + x0;
     const int n = n0 + col;
-    auto ring_row = [&](int x) {  // staged key index x (0 .. 64 NB - 1 <-> key q0 - 64 (NB - 1) + x) -> ring row
+    auto ring_row = [&](int x) {  // staged key index x (0 .. 64 NBR - 1 <-> key q0 - 64 (NB - 1) + x) -> ring row
       int blk = oldest + (x >> 6);
-      blk = blk >= NB ? blk - NB : blk;
+      blk = blk >= NBR ? blk - NBR : blk;
       return blk * kWQTile + (x & (kWQTile - 1));
     };
     __syncthreads();  // the staged rows are visible
-    unsigned char* const q_rows = lds + kOffQ + 16 * wq * kWRowBytes;  // this wavefront's own
+    unsigned char* const q_rows = lds + kOffQ + 16 * w8 * kWRowBytes;  // this wavefront's own
     bf16x8 bq[NDS];
 #pragma unroll
     for (int ds = 0; ds < NDS; ++ds)
@@ -284,7 +303,7 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
     f32x4 st[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) {
-      const unsigned char* row = lds + ring_row(16 * wq + 16 * i) * kWRowBytes + k_lane;
+      const unsigned char* row = lds + ring_row(x0 + 16 * i) * kWRowBytes + k_lane;
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ds = 0; ds < NDS; ++ds)
@@ -341,8 +360,8 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
         pb4[3] = 0u;
       }
       const bf16x8 bp = __builtin_bit_cast(bf16x8, pb4);
-      const unsigned char* lo_rows = lds + kOffV + ring_row(16 * wq + 32 * s) * kWRowBytes + v_lane;
-      const unsigned char* hi_rows = lds + kOffV + ring_row(s < NS - 1 ? 16 * wq + 32 * s + 16 : 0) * kWRowBytes + v_lane;
+      const unsigned char* lo_rows = lds + kOffV + ring_row(x0 + 32 * s) * kWRowBytes + v_lane;
+      const unsigned char* hi_rows = lds + kOffV + ring_row(s < NS - 1 ? x0 + 32 * s + 16 : 0) * kWRowBytes + v_lane;
 #pragma unroll
       for (int et = 0; et < NET; ++et) {
         const int pc = wide_swz_v(vt_row, 2 * et + v_half) << 4;
@@ -381,21 +400,21 @@ __global__ __launch_bounds__(256, NB == 2 ? 2 : 1) void swa_prefill_wide_kernel(
       }
     }
 
-    // ---- the oldest block (and the query rows) take the next tile's rows ----
-    if (tile + 1 < tile_end) {
-      __syncthreads();  // every wavefront is done with the oldest block
-      store_rows(oldest, q0 + kWQTile, nxt, true);
-      if (tile + 1 + DEPTH < tile_end) load_rows(q0 + (1 + DEPTH) * kWQTile, nxt, true);  // not waited for here
+    // ---- the oldest QT blocks (and the query rows) take the next step's rows ----
+    if (tile + QT < tile_end) {
+      __syncthreads();  // every wavefront is done with the oldest blocks
+      store_rows(oldest, q0 + kSuper, nxt, true);
+      if (tile + QT * (1 + DEPTH) < tile_end) load_rows(q0 + (1 + DEPTH) * kSuper, nxt, true);  // not waited for here
     }
-    q0 += kWQTile;
-    own = own + 1 == NB ? 0 : own + 1;
+    q0 += kSuper;
+    own = oldest;   // (own + QT) mod NBR
   };
   if constexpr (DEPTH == 1) {
-    for (int tile = tile_begin; tile < tile_end; ++tile) do_tile(tile, pre);
+    for (int tile = tile_begin; tile < tile_end; tile += QT) do_tile(tile, pre);
   } else {
-    for (int tile = tile_begin; tile < tile_end; tile += 2) {
+    for (int tile = tile_begin; tile < tile_end; tile += 2 * QT) {
       do_tile(tile, pre);
-      if (tile + 1 < tile_end) do_tile(tile + 1, pre2);
+      if (tile + QT < tile_end) do_tile(tile + QT, pre2);
     }
   }
 }
@@ -605,7 +624,7 @@ __global__ __launch_bounds__(256) void swa_step_wide_kernel(
 static bool wide_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 constexpr int kWideMaxDevices = 64;
-static std::atomic<bool> g_wide_lds_allowed[kWideMaxDevices][3 /*RMODE*/][2 /*NB - 2*/][2 /*NDS / 2 - 1*/];
+static std::atomic<bool> g_wide_lds_allowed[kWideMaxDevices][3 /*RMODE*/][3 /*NB 2, NB 3, NB 3 two tiles*/][2 /*NDS / 2 - 1*/];
 
 // shared checks of the rotary arguments; returns the layout code or -1 with the error set
 static int wide_rope_mode(const char* who, const float* rope_cos, const float* rope_sin, int64_t rotary_dim,
@@ -671,33 +690,40 @@ extern "C" BASED_API int based_swa_prefill_wide(const void* q, const void* k, co
   const int64_t n_tiles = (L + kWQTile - 1) / kWQTile;
   BASED_REQUIRE(B * H * n_tiles < (1ll << 31), BASED_ERR_SHAPE, "swa_prefill_wide: grid too large");
   const int nb = w_left > 64 ? 3 : 2;
+  // the three-block window: two tiles side by side per workgroup (a sequence of one tile has nothing for the second)
+  const int qt = nb == 3 && n_tiles > 1 ? 2 : 1;
   // runs of consecutive tiles, as long as still gives every resident slot one run: 256 compute
-  // units x the workgroups whose LDS fits one (80 KB: two; 112 KB: one)
+  // units x the workgroups whose LDS fits one (80 KB: two; 112 KB and 160 KB: one)
   const int64_t slots = 256 * (nb == 3 ? 1 : 2);
   int64_t want_runs = slots / (B * H);
   want_runs = want_runs < 1 ? 1 : (want_runs > n_tiles ? n_tiles : want_runs);
-  const int64_t run_tiles = (n_tiles + want_runs - 1) / want_runs;
+  int64_t run_tiles = (n_tiles + want_runs - 1) / want_runs;
+  run_tiles = (run_tiles + qt - 1) / qt * qt;
   const int64_t runs_per_seq = (n_tiles + run_tiles - 1) / run_tiles;
-  dim3 grid((unsigned)(B * H * runs_per_seq)), block(256);
+  dim3 grid((unsigned)(B * H * runs_per_seq)), block(256 * qt);
   using Kern = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int, int, int, int, int, long, long, long,
                         long, long, long, long, long, long, long, long, long, int, float, const float*, const float*, int,
                         __bf16*, __bf16*, long, long, long);
   // head dims up to 64 contract in two steps of 32 channels, up to 128 in four
-  static const Kern kerns[3][2][2] = {
-      {{swa_prefill_wide_kernel<kRopeNone, 2, 2>, swa_prefill_wide_kernel<kRopeNone, 2, 4>},
-       {swa_prefill_wide_kernel<kRopeNone, 3, 2>, swa_prefill_wide_kernel<kRopeNone, 3, 4>}},
-      {{swa_prefill_wide_kernel<kRopeHalf, 2, 2>, swa_prefill_wide_kernel<kRopeHalf, 2, 4>},
-       {swa_prefill_wide_kernel<kRopeHalf, 3, 2>, swa_prefill_wide_kernel<kRopeHalf, 3, 4>}},
-      {{swa_prefill_wide_kernel<kRopeInterleaved, 2, 2>, swa_prefill_wide_kernel<kRopeInterleaved, 2, 4>},
-       {swa_prefill_wide_kernel<kRopeInterleaved, 3, 2>, swa_prefill_wide_kernel<kRopeInterleaved, 3, 4>}}};
+  static const Kern kerns[3][3][2] = {
+      {{swa_prefill_wide_kernel<kRopeNone, 2, 2, 1>, swa_prefill_wide_kernel<kRopeNone, 2, 4, 1>},
+       {swa_prefill_wide_kernel<kRopeNone, 3, 2, 1>, swa_prefill_wide_kernel<kRopeNone, 3, 4, 1>},
+       {swa_prefill_wide_kernel<kRopeNone, 3, 2, 2>, swa_prefill_wide_kernel<kRopeNone, 3, 4, 2>}},
+      {{swa_prefill_wide_kernel<kRopeHalf, 2, 2, 1>, swa_prefill_wide_kernel<kRopeHalf, 2, 4, 1>},
+       {swa_prefill_wide_kernel<kRopeHalf, 3, 2, 1>, swa_prefill_wide_kernel<kRopeHalf, 3, 4, 1>},
+       {swa_prefill_wide_kernel<kRopeHalf, 3, 2, 2>, swa_prefill_wide_kernel<kRopeHalf, 3, 4, 2>}},
+      {{swa_prefill_wide_kernel<kRopeInterleaved, 2, 2, 1>, swa_prefill_wide_kernel<kRopeInterleaved, 2, 4, 1>},
+       {swa_prefill_wide_kernel<kRopeInterleaved, 3, 2, 1>, swa_prefill_wide_kernel<kRopeInterleaved, 3, 4, 1>},
+       {swa_prefill_wide_kernel<kRopeInterleaved, 3, 2, 2>, swa_prefill_wide_kernel<kRopeInterleaved, 3, 4, 2>}}};
   const int wide = D > 64 ? 1 : 0;
-  const Kern kern = kerns[rmode][nb - 2][wide];
-  const size_t lds = (size_t)wide_lds_bytes(nb);
+  const int variant = nb - 2 + (qt - 1);
+  const Kern kern = kerns[rmode][variant][wide];
+  const size_t lds = (size_t)wide_lds_bytes(nb, qt);
   {
     int dev = 0;
     BASED_REQUIRE(hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kWideMaxDevices, BASED_ERR_LAUNCH,
                   "swa_prefill_wide: cannot identify the current device");
-    std::atomic<bool>& allowed = g_wide_lds_allowed[dev][rmode][nb - 2][wide];
+    std::atomic<bool>& allowed = g_wide_lds_allowed[dev][rmode][variant][wide];
     if (!allowed.load(std::memory_order_acquire)) {  // more than 64 KB of LDS has to be asked for once per device
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

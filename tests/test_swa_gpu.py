@@ -290,6 +290,38 @@ def test_wide_prefill_rotary_layouts_and_cache(dev, D, R, inter, B, L, H, w):
     assert bool((c[:, L:] == 3.0).all())
 
 
+@pytest.mark.parametrize("D,R,inter,L", [(112, 0, False, 1100), (112, 112, False, 1100), (128, 64, True, 1237),
+                                         (96, 96, False, 700)])
+def test_wide_prefill_long_runs_of_tile_pairs(dev, D, R, inter, L):
+    """128 heads and 128 keys to the left: every workgroup walks a run of many steps of two query
+    tiles (both register sets of rows in flight, the four-block ring going round several times, a
+    last step whose second tile is past the sequence)."""
+    from based_amd import ops
+
+    B, H, w = 8, 16, 128
+    print(f"swa wide long-run case D={D} R={R} interleaved={inter} L={L}", flush=True)
+    qkv = _qkv_d(B, L, H, D, seed=53)
+    q_r, k_r = qkv[:, :, 0], qkv[:, :, 1]
+    rope = None
+    if R:
+        pos = torch.arange(L)
+        q_r = O.rotary_embedding(q_r, pos, rotary_dim=R, interleaved=inter)
+        k_r = O.rotary_embedding(k_r, pos, rotary_dim=R, interleaved=inter)
+        rope = _rope_tables_d(L, R, dev, inter)
+    ref = O.sliding_window_attn(q_r, k_r, qkv[:, :, 2], w_left=w)
+    qd = qkv.to(dev)
+    cache = torch.full((B, L + 1, 2, H, D), 3.0, dtype=torch.bfloat16, device=dev)
+    out = ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, rope=rope, kv_cache=cache, impl="wide")
+    torch.cuda.synchronize()
+    per_tile = (out.float().cpu() - ref.float()).flatten(2).norm(dim=2) / ref.float().flatten(2).norm(dim=2)
+    assert float(per_tile.max()) < 1.5e-2, f"worst token at {int(per_tile.argmax()) % L}"
+    assert rel_l2(out.float(), ref.float()) < TOL
+    c = cache.cpu()
+    assert torch.equal(c[:, :L, 1], qkv[:, :, 2]) and bool((c[:, L:] == 3.0).all())
+    assert rel_l2(c[:, :L, 0].float(), k_r.float()) < 3e-3
+    assert torch.equal(out, ops.swa_prefill(qd[:, :, 0], qd[:, :, 1], qd[:, :, 2], w_left=w, rope=rope, impl="wide"))
+
+
 @pytest.mark.parametrize("D,R,inter,P,T,w", [(112, 112, False, 0, 140, 128), (112, 112, False, 200, 8, 128),
                                              (128, 128, False, 70, 6, 64), (112, 64, True, 50, 20, 128),
                                              (64, 32, False, 10, 10, 7), (64, 64, True, 100, 40, 128)])
