@@ -296,151 +296,43 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
 
   // key tiles i < i_win reach below the window of the wavefront's last query (see the softmax)
   const int i_win = w_left >= 64 * (NB - 1) + 15 ? 0 : (64 * (NB - 1) + 30 - w_left) >> 4;
-  int own = 0;  // ring block with keys [q0, q0+64); block own + 1 (mod NB) is the oldest
-  for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile, own = own + 1 == NB ? 0 : own + 1) {
-    const int oldest = own + 1 == NB ? 0 : own + 1;
-    const int n0 = q0 + 16 * wq;              // first query of this wavefront
-    const int n = n0 + col;                   // this lane's query
-    // staged key index x (0..64 NB - 1 <-> key q0 - 64 (NB - 1) + x) -> row of the ring
-    auto ring_row = [&](int x) {
-      int blk = oldest + (x >> 6);
-      blk = blk >= NB ? blk - NB : blk;
-      return blk * kQTile + (x & (kQTile - 1));
-    };
-    __syncthreads();  // the staged rows are visible
-    // 16 rows of LDS that are this wavefront's own at the time it stages its output tile
-    unsigned char* const q_rows = QLDS ? my + kOffQ + 16 * wq * kRowBytes : my + (oldest * kQTile + 16 * wq) * kRowBytes;
-    if constexpr (QLDS) {
-#pragma unroll
-      for (int ds = 0; ds < 2; ++ds)
-        bq[ds] = *reinterpret_cast<const bf16x8*>(q_rows + k_lane + (((4 * ds + grp) ^ k_sw) << 4));
-    }
-
-    // ---- S^T tiles: keys (rows) x queries (cols), contraction over the 64 channels ----
-    // wavefront w sees staged keys 16 w .. 16 w + 16 NT - 1 (tile i = keys 16 w + 16 i ..)
-    f32x4 st[NT];
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
-      const unsigned char* row = my + ring_row(16 * wq + 16 * i) * kRowBytes + k_lane;
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ds = 0; ds < 2; ++ds)
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            *reinterpret_cast<const bf16x8*>(row + (((4 * ds + grp) ^ k_sw) << 4)), bq[ds], acc, 0, 0, 0);
-      st[i] = acc;
-    }
-
-    // ---- masked softmax over keys; lane holds keys 16 i + 4 grp + r of query n ----
-    // Only three kinds of key tile contain a masked (key, query) pair, and which they are is the
-    // same for the whole wavefront: the diagonal tile (causality), the tiles that reach below
-    // n0 + 15 - w_left (the far edge of the window), and tiles before the start of the sequence.
-    // All other tiles skip the mask arithmetic.  The scale is applied inside the exponent.
-    float mx = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < NT; ++i) {
-      const int klo = n0 - 64 * (NB - 1) + 16 * i;  // first key of the tile
-      if (i == NT - 1 || i < i_win || klo < 0) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int key = klo + 4 * grp + r;
-          const bool keep = key >= 0 && key <= n && key >= n - w_left;
-          st[i][r] = keep ? st[i][r] : -INFINITY;
-        }
+  // With 128 keys to the left the arithmetic, not the memory, sets the pace (144 keys per
+  // wavefront and tile), a good part of it the addresses of the operand reads.  Paired heads there
+  // run two wavefronts per SIMD and have registers to spare: their loop is unrolled over the three
+  // positions of the ring, so that where a wavefront's tiles of 16 staged keys sit in LDS is, but
+  // for the tiles whose wrap round the ring depends on the wavefront (their addresses wait in
+  // registers), an immediate offset of the operand reads (B=8, H=16, L=4096, cold: rotary + cache
+  // fill 95.0 -> 90.3 us; plain 63.8 -> 61.8 and rotary 78.4 -> 73.4 against one head per
+  // workgroup).  The other variants lose what they gain to register spills, or have nothing to gain
+  // because they wait for memory.
+  constexpr bool kStaticRing = NB == 3 && G == 2;
+  if constexpr (kStaticRing) {
+    // a run starts with the own keys in block 0: the oldest block is 1, then 2, then 0
+    for (int tile = tile_begin;;) {
+      {
+        constexpr int oldest = 1;
+#include "swa_tile.inc"
       }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, st[i][r]);
+      q0 += kQTile;
+      if (++tile == tile_end) break;
+      {
+        constexpr int oldest = 2;
+#include "swa_tile.inc"
+      }
+      q0 += kQTile;
+      if (++tile == tile_end) break;
+      {
+        constexpr int oldest = 0;
+#include "swa_tile.inc"
+      }
+      q0 += kQTile;
+      if (++tile == tile_end) break;
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mxs = mx * scale_log2e;
-    float sum = 0.f;
-#pragma unroll
-    for (int i = 0; i < NT; ++i)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i][r], scale_log2e, -mxs));  // exp2(-inf) = 0 for masked keys
-        st[i][r] = p;
-        sum += p;
-      }
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
-
-    // ---- O^T = V^T P^T: 4 channel tiles x NS key slabs of 32 (last slab half empty) ----
-    // V^T operand tiles come from the row-major V rows with the transposing 64-bit LDS read:
-    // in each group of 16 lanes, lane 4a + b receives element b of what lanes a, a+4, a+8, a+12
-    // loaded, so source lane 4j + a fetches channels 4a..4a+3 of key j of the group's four.
-    f32x4 ot[4];
-#pragma unroll
-    for (int et = 0; et < 4; ++et) ot[et] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      // B operand: slots 0..3 <- tile 2s rows 4grp+r, slots 4..7 <- tile 2s+1 (absent in the last slab)
-      u32x4 pb;
-      pb[0] = pack_bf16(st[2 * s][0], st[2 * s][1]);
-      pb[1] = pack_bf16(st[2 * s][2], st[2 * s][3]);
-      if (s < NS - 1) {
-        pb[2] = pack_bf16(st[2 * s + 1][0], st[2 * s + 1][1]);
-        pb[3] = pack_bf16(st[2 * s + 1][2], st[2 * s + 1][3]);
-      } else {
-        pb[2] = 0u;
-        pb[3] = 0u;
-      }
-      const bf16x8 bp = __builtin_bit_cast(bf16x8, pb);
-      const unsigned char* lo_rows = my + kOffV + ring_row(16 * wq + 32 * s) * kRowBytes + v_lane;
-      const unsigned char* hi_rows = my + kOffV + ring_row(s < NS - 1 ? 16 * wq + 32 * s + 16 : 0) * kRowBytes + v_lane;
-#pragma unroll
-      for (int et = 0; et < 4; ++et) {
-        const int pc = ((2 * et + v_half) ^ v_sw) << 4;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(lo_rows + pc));
-        s16x4 hi = {0, 0, 0, 0};
-        if (s < NS - 1)
-          hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(hi_rows + pc));
-        const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        ot[et] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), bp, ot[et], 0, 0, 0);
-      }
-    }
-
-    // ---- normalise; the 16 x 64 tile goes through the wavefront's own query rows (read above, not
-    // needed again, and rewritten only after the barrier below) so that every lane stores 16
-    // bytes of a full 128-byte row ----
-    const float inv = 1.0f / sum;
-    if constexpr (!QLDS) __syncthreads();  // every wavefront is done with the oldest block, whose rows stage the tile
-#pragma unroll
-    for (int et = 0; et < 4; ++et) {
-      const uint32_t w0 = pack_bf16(ot[et][0] * inv, ot[et][1] * inv);
-      const uint32_t w1 = pack_bf16(ot[et][2] * inv, ot[et][3] * inv);
-      *reinterpret_cast<uint2*>(q_rows + k_lane + (((2 * et + (grp >> 1)) ^ k_sw) << 4) + 8 * (grp & 1)) = make_uint2(w0, w1);
-    }
-    // the tile is re-read below in another lane layout: order the wavefront's own LDS accesses
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int hlf = 0; hlf < 2; ++hlf) {
-      const int row = 8 * hlf + (lane >> 3);
-      const u32x4 w4 = *reinterpret_cast<const u32x4*>(q_rows + row * kRowBytes + (((lane & 7) ^ swz_k(row)) << 4));
-      if (n0 + row < L) __builtin_nontemporal_store(w4, reinterpret_cast<u32x4*>(o_my + (long)(n0 + row) * o_sl + 8 * (lane & 7)));
-    }
-
-    // ---- the oldest block takes the next tile's rows ----
-    if (tile + 1 < tile_end) {
-      if constexpr (QLDS) {
-        __syncthreads();  // every wavefront is done with the oldest block
-      } else {
-        // the staged tile has been read back (same wavefront, same rows: program order suffices)
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        bq[0] = bq_next[0];
-        bq[1] = bq_next[1];
-      }
-      store_rows(oldest, q0 + kQTile, pre, true);
-      if (tile + 2 < tile_end) {
-        load_rows(q0 + 2 * kQTile, pre, true);
-        if constexpr (!QLDS) load_q(q0 + 2 * kQTile, bq_next);
-        // These loads are not waited for here: they travel under the next tile's arithmetic and
-        // are first needed by its store_rows.  (That only works because no load sits in a branch;
-        // measured: warm 49.8 -> 47.6 us, cold unchanged at the rate the memory system gives
-        // this access pattern.)
-      }
+  } else {
+    int own = 0;  // ring block with keys [q0, q0+64); block own + 1 (mod NB) is the oldest
+    for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile, own = own + 1 == NB ? 0 : own + 1) {
+      const int oldest = own + 1 == NB ? 0 : own + 1;
+#include "swa_tile.inc"
     }
   }
 }
@@ -836,15 +728,15 @@ extern "C" BASED_API int based_swa_prefill(const void* q, const void* k, const v
   // Heads that are neighbours in every tensor (the packed qkv layout) share a workgroup, so that
   // every load and store instruction covers pieces of 128 G bytes.  Two-block ring: four heads
   // (16 wavefronts, 160 KB of LDS: one workgroup per compute unit; 57.1 -> 53.9 us at B=8, H=16,
-  // L=4096 against two heads in each of two workgroups), else two.  Three-block ring (112 KB for
-  // two heads, one workgroup of 8 wavefronts per unit): two heads when the rows also go to a KV
-  // cache, whose 256-byte stores then pay for the lower occupancy (rotary + cache fill 108.5 ->
-  // 98.7 us), one head otherwise (three workgroups of 4 wavefronts: 64.2 against 66.7 us).
+  // L=4096 against two heads in each of two workgroups), else two.  Three-block ring: two heads
+  // (112 KB, one workgroup of 8 wavefronts per unit, whose registers allow the loop unrolled over
+  // the ring's positions: see the kernel), one head (three workgroups of 4 wavefronts) only where
+  // the heads are not neighbours.
   const bool rope = rope_cos != nullptr;
   const int nb = w_left > 64 ? 3 : 2;
   const bool pair = H % 2 == 0 && q_sh == 64 && k_sh == 64 && v_sh == 64 && o_sh == 64 &&
                     (!kcache_out || c_sh == 64);
-  const int g = !pair ? 1 : (nb == 2 ? (H % 4 == 0 ? 4 : 2) : (kcache_out ? 2 : 1));
+  const int g = !pair ? 1 : (nb == 2 && H % 4 == 0 ? 4 : 2);
   // Consecutive query tiles of one (batch, head) are walked by one workgroup (the keys to the left
   // of a tile are the previous tile's own keys, already staged).  Runs are as long as still gives
   // every resident slot of the GPU one run: 256 compute units x the wavefront quartets that fit
