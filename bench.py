@@ -324,7 +324,7 @@ def bench_swa(torch, ops, steps, warmup, B=8, H=16, L=4096, decode_steps=256, n_
     g = torch.Generator(device="cpu").manual_seed(2)
     # every prefill leg below is timed after 20 ms of its own launches, like the linear-attention
     # prefill: the first millisecond after an idle period runs at another clock and memory state
-    # than a serving loop sees (head dim 112: 157 us in that transient, 139 us after it)
+    # than a serving loop sees (head dim 112 at one point: 157 us in that transient, 139 us after it)
     SWA_WARMUP_MS = 20.0
     qkvs = [torch.randn(B, L, 3, H, 64, generator=g).bfloat16().to(dev) for _ in range(n_sets)]
     outs = [torch.empty(B, L, H, 64, dtype=torch.bfloat16, device=dev) for _ in range(n_sets)]
