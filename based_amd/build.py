@@ -6,7 +6,9 @@ from __future__ import annotations
 
 import concurrent.futures as cf
 import glob
+import json
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -33,17 +35,36 @@ FLAGS = [
 ]
 
 
-def _compile(src: str) -> str:
+RESOURCES = os.path.join(OBJDIR, "resource_usage.json")
+_REMARK = re.compile(r"remark:\s+(Function Name|VGPRs|AGPRs|VGPRs Spill|SGPRs Spill|ScratchSize \[bytes/lane\]|"
+                     r"Occupancy \[waves/SIMD\]|LDS Size \[bytes/block\]):\s+(\S+)")
+
+
+_SNIPPET = re.compile(r"^\s*\d*\s*\|")   # the source lines clang shows under a remark
+
+
+def _compile(src: str):
+    """Compiles one source; returns (object file, {kernel: resource figures the compiler reports})."""
     obj = os.path.join(OBJDIR, os.path.basename(src).rsplit(".", 1)[0] + ".o")
-    cmd = [HIPCC, *FLAGS, "-c", src, "-o", obj]
+    cmd = [HIPCC, *FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
     noise = "unknown target-feature"  # host pass does not know the gfx feature name; harmless
-    warn = "\n".join(l for l in r.stderr.splitlines() if l.strip() and noise not in l and "packed-fp32-ops" not in l)
-    if warn:
-        sys.stderr.write(warn + "\n")
-    return obj
+    usage, cur, other = {}, None, []
+    for line in r.stderr.splitlines():
+        m = _REMARK.search(line)
+        if m:
+            if m.group(1) == "Function Name":
+                cur = usage.setdefault(m.group(2), {})
+            elif cur is not None:
+                cur[m.group(1)] = int(m.group(2))
+        elif ("-Rpass-analysis" not in line and line.strip() and noise not in line and "packed-fp32-ops" not in line
+              and not _SNIPPET.match(line)):
+            other.append(line)
+    if other:
+        sys.stderr.write("\n".join(other) + "\n")
+    return obj, usage
 
 
 def build(verbose: bool = False) -> str:
@@ -52,7 +73,18 @@ def build(verbose: bool = False) -> str:
     if not srcs:
         raise RuntimeError("no HIP sources found")
     with cf.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
+        done = list(ex.map(_compile, srcs))
+    objs = [o for o, _ in done]
+    # what the compiler says each kernel needs (registers, spills, LDS): kept beside the objects; a
+    # kernel that spills vector registers is named, because a few spilled registers in a loop have
+    # cost a hot kernel 5 % here without any other sign
+    usage = {os.path.basename(src): u for src, (_, u) in zip(srcs, done)}
+    with open(RESOURCES, "w") as f:
+        json.dump(usage, f, indent=1, sort_keys=True)
+    for src, kernels in usage.items():
+        for name, u in kernels.items():
+            if u.get("VGPRs Spill", 0) > 0:
+                sys.stderr.write(f"note: {src}: {name} spills {u['VGPRs Spill']} vector registers\n")
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
