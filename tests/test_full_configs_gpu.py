@@ -83,6 +83,55 @@ def test_config3_sliding_window_full(dev):
     assert torch.equal(cache[:, L:], qkv[:, L:, 1:])
 
 
+@pytest.mark.parametrize("D", [64, 112])
+def test_released_window_full_size(dev, D):
+    """configs[2]'s size with the released checkpoints' window (128 keys to the left), rotary over the
+    whole head and the KV-cache fill in the launch; head dim 64 (paired heads, the loop unrolled over
+    the ring) and 112 (two query tiles per workgroup).  The oracle on three 512-token blocks with
+    their halo; then what needs no CPU pass: the first half of the sequences alone gives the same
+    bits, keys and values further back than the window do not reach an output (bit-exact), the
+    cache holds v exactly and the rotated k of the oracle, and q = 0 gives the window mean of v."""
+    from based_amd import ops
+
+    B, H, L, w = 8, 16, 4096, 128
+    print(f"released window at full size, head dim {D}", flush=True)
+    qkv = _randn((B, L, 3, H, D), 40 + D, dev)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, D, 2, dtype=torch.float32) / D))
+    ang = torch.outer(torch.arange(L).float(), inv_freq)
+    rope = (ang.cos().contiguous().to(dev), ang.sin().contiguous().to(dev))
+    cache = torch.full((B, L + 2, 2, H, D), 3.0, dtype=torch.bfloat16, device=dev)
+    out = ops.swa_prefill(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=w, rope=rope, kv_cache=cache)
+    assert torch.isfinite(out.float()).all()
+    for start in (0, 1472, 3584):
+        lo = max(0, start - w)
+        blk = qkv[:2, lo:start + 512].cpu()
+        pos = torch.arange(lo, start + 512)
+        q_r = O.rotary_embedding(blk[:, :, 0], pos, rotary_dim=D)
+        k_r = O.rotary_embedding(blk[:, :, 1], pos, rotary_dim=D)
+        ref = O.sliding_window_attn(q_r, k_r, blk[:, :, 2], w_left=w)[:, start - lo:]
+        assert rel_l2(out[:2, start:start + 512].float().cpu(), ref.float()) < 1e-2
+        assert rel_l2(cache[:2, lo:start + 512, 0].float().cpu(), k_r.float()) < 3e-3
+    assert torch.equal(cache[:, :L, 1], qkv[:, :, 2]) and bool((cache[:, L:] == 3.0).all())
+    # the first half alone: same bits
+    half = ops.swa_prefill(qkv[:, :L // 2, 0], qkv[:, :L // 2, 1], qkv[:, :L // 2, 2], w_left=w, rope=rope)
+    assert torch.equal(half, out[:, :L // 2])
+    # keys and values more than 128 positions back do not reach the outputs from token 2048 on
+    far = qkv.clone()
+    far[:, :2048 - w, 1:] = _randn((B, 2048 - w, 2, H, D), 7, dev)
+    out_far = ops.swa_prefill(far[:, :, 0], far[:, :, 1], far[:, :, 2], w_left=w, rope=rope)
+    assert torch.equal(out_far[:, 2048:], out[:, 2048:])
+    assert not torch.equal(out_far[:, :1024], out[:, :1024])
+    del far, out_far, half
+    # q = 0: the window mean of v (the rotation of a zero query is zero)
+    o0 = ops.swa_prefill(torch.zeros_like(qkv[:, :, 0]), qkv[:, :, 1], qkv[:, :, 2], w_left=w, rope=rope).float()
+    vf = qkv[:, :, 2].float()
+    cs = torch.cat([torch.zeros_like(vf[:, :1]), vf.cumsum(1)], dim=1)
+    i = torch.arange(L, device=dev)
+    lo = (i - w).clamp_min(0)
+    mean = (cs[:, i + 1] - cs[:, lo]) / (i + 1 - lo)[None, :, None, None].float()
+    assert rel_l2(o0, mean) < 1e-2
+
+
 def test_config5_long_context_dv128(dev):
     """B=1, H=16, L=32768, dv=128 bf16: MFMA scan vs the independent fp32 recurrent kernel, the
     oracle on the first 2048 tokens, linearity in v; then decode at B=64 from the tiled state."""

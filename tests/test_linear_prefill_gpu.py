@@ -243,3 +243,47 @@ def test_split_plan(dev):
     assert n.value >= 2 and w.value == 32 * n.value * 43008  # dv 112: two channel blocks per (batch, head)
     assert lib.based_linear_attn_prefill_plan(1, 16, 4096, 72, 0, ctypes.byref(n), ctypes.byref(w)) == 0
     assert n.value == 1 and w.value == 0                     # not whole 16-channel tiles: the fp32 kernel, never split
+
+
+@pytest.mark.parametrize("B", [32, 96])
+def test_full_size_prefill_properties(dev, B):
+    """The bench's prefill sizes (H=16, L=4096, dv=64, bf16; B=96 is the 1536-chain launch) through
+    properties that need no CPU pass: the first half of every sequence does not depend on the
+    second (bit-exact: same chunks, same order), a sequence does not depend on its place in the
+    batch (bit-exact), the output is linear in v (the normaliser does not see v), the states equal
+    those of the fp32 recurrent kernel on four sequences, and the segmented small-batch scan agrees
+    with the single pass on the same rows."""
+    from based_amd import ops
+
+    H, L, dv = 16, 4096, 64
+    g = torch.Generator(device="cpu").manual_seed(1000 + B)
+    print(f"full-size prefill properties B={B}", flush=True)
+    q = torch.randn(B, L, H, 16, generator=g).bfloat16().to(dev).transpose(1, 2)
+    k = torch.randn(B, L, H, 16, generator=g).bfloat16().to(dev).transpose(1, 2)
+    v = torch.randn(B, L, H, dv, generator=g).bfloat16().to(dev).transpose(1, 2)
+    y, kv, ks = ops.linear_attn_prefill(q, k, v, return_state=True, split=False)
+    assert bool(torch.isfinite(y.float()).all())
+    assert torch.all(ks[..., 0] == L)
+    # causality: the first half alone
+    y_half, _, _ = ops.linear_attn_prefill(q[:, :, :L // 2], k[:, :, :L // 2], v[:, :, :L // 2], split=False)
+    assert torch.equal(y_half, y[:, :, :L // 2])
+    # batch order: reversed batch
+    y_rev, kv_rev, _ = ops.linear_attn_prefill(q.flip(0), k.flip(0), v.flip(0), return_state=True, split=False)
+    assert torch.equal(y_rev.flip(0), y) and torch.equal(kv_rev.flip(0), kv)
+    del y_rev, kv_rev, y_half
+    # linearity in v: y(v) + y(v2) = y(v + v2) up to the bf16 rounding of the three outputs
+    v2 = torch.randn(B, L, H, dv, generator=g).bfloat16().to(dev).transpose(1, 2)
+    vs = (v.float() + v2.float()).bfloat16()
+    y2, _, _ = ops.linear_attn_prefill(q, k, v2, split=False)
+    y_sum, _, _ = ops.linear_attn_prefill(q, k, vs, split=False)
+    assert rel_l2(y_sum.float(), y.float() + y2.float()) < 1e-2
+    del v2, vs, y2, y_sum
+    # four sequences against the fp32 recurrent kernel (outputs and states) and through the segmented scan
+    rows = [0, 1, B // 2, B - 1]
+    qs, ks_, vs_ = q[rows], k[rows], v[rows]
+    y32, kv32, ks32 = ops.linear_attn_prefill(qs.float(), ks_.float(), vs_.float(), return_state=True)
+    assert rel_l2(y[rows].float(), y32) < 1e-2
+    assert rel_l2(kv[rows], kv32) < 5e-3 and rel_l2(ks[rows], ks32) < 5e-3
+    y_seg, kv_seg, ks_seg = ops.linear_attn_prefill(qs, ks_, vs_, return_state=True, split=4)
+    assert rel_l2(y_seg.float(), y[rows].float()) < 5e-3
+    assert rel_l2(kv_seg, kv[rows]) < 2e-3 and rel_l2(ks_seg, ks[rows]) < 2e-3
