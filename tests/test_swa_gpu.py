@@ -124,7 +124,10 @@ def _rope_tables(n_pos, dev):
 
 
 @pytest.mark.parametrize("B,L,H,w", [(2, 256, 3, 64), (1, 1, 2, 64), (1, 100, 2, 64), (1, 333, 4, 20), (1, 1024, 8, 64),
-                                     (2, 257, 3, 128), (1, 129, 2, 128), (1, 1024, 8, 128), (1, 333, 4, 90)])
+                                     (2, 257, 3, 128), (1, 129, 2, 128), (1, 1024, 8, 128), (1, 333, 4, 90),
+                                     # paired heads under the three-block ring, runs of 2+2+2+1, 3+3+3+3 and 5+4 tiles
+                                     # (every exit of the loop that is unrolled over the ring's positions)
+                                     (8, 448, 16, 128), (8, 709, 16, 128), (16, 576, 16, 100)])
 def test_prefill_with_rotary_and_cache_output(dev, B, L, H, w):
     """Rotary inside the kernel == rotating q, k first (oracle RoPE, rounded to bf16 like the
     reference's rotated tensors); the optional cache output holds the rotated k and v."""
