@@ -44,11 +44,11 @@ D_EXP = 273
 # the same counter reads for a plain copy of known size (the summaries and the commands that
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": 293108531,   # B=128, H=16, dv=64, rotating state sets: fetch 146,969,600 + write 146,138,931
-    "lin_step_kernel_B64_dv128": 290398413,   # long-context decode: fetch 145,405,747 + write 144,992,666
-    "lin_prefill_mfma_kernel": {96: 2295008256},  # B=96, L=4096, dv=64, states written: fetch 1,380,576,051 + write 914,432,205 (the fetch varies by 10 % between runs); keyed by batch
-    "swa_prefill_kernel": 283322266,   # B=8, H=16, L=4096, four heads per workgroup: fetch 216,145,306 + write 67,176,960
-    "decode_linear_kernel_lm_head": 104974234,   # M=4, 50280 x 1024 + closing norm: fetch 104,362,598 + write 611,635
+    "lin_step_kernel": 293110681,   # B=128, H=16, dv=64, rotating state sets: fetch 146,971,238 + write 146,139,443
+    "lin_step_kernel_B64_dv128": 290398106,   # long-context decode: fetch 145,408,205 + write 144,989,901
+    "lin_prefill_mfma_kernel": {96: 2290955981},  # B=96, L=4096, dv=64, states written: fetch 1,376,494,592 + write 914,461,389 (the fetch varies by 10 % between runs); keyed by batch
+    "swa_prefill_kernel": 283344384,   # B=8, H=16, L=4096, four heads per workgroup: fetch 216,140,186 + write 67,204,198
+    "decode_linear_kernel_lm_head": 104981504,   # M=4, 50280 x 1024 + closing norm: fetch 104,370,176 + write 611,328
 }
 
 
