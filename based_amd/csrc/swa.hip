@@ -224,23 +224,67 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
       *reinterpret_cast<u32x4*>(mv_lds_v + kOffV + (blk * kQTile + lrow_v) * kRowBytes + ((piece_idx_v(i) ^ swz_v(lrow_v)) << 4)) = r.vp[i];
       if constexpr (QLDS)
         if (own_rows) *reinterpret_cast<u32x4*>(mv_lds + kOffQ + lrow * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.qp[i];
-      // Cache rows leave non-temporally where an instruction writes whole rows (the plain
-      // arrangement); rows in the rotary arrangement leave as two half rows from two instructions,
-      // which the cache has to merge (non-temporal there: 99 -> 103 us at 128 keys to the left).
+      // Cache rows leave non-temporally, an instruction writing whole rows: as they are in the
+      // plain arrangement, after an exchange between lanes in the rotary one (below; the two-block
+      // rotary variants still write half rows from two instructions, which the cache has to merge:
+      // non-temporal stores of half rows were slower, 99 -> 103 us).
       const int key = key0 + lrow;
-      if constexpr (!kPlainV) {  // K and V in one arrangement: one condition
-        if (own_rows && kc_mv != nullptr && key < L) {
-          *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
-          *reinterpret_cast<u32x4*>(vc_mv + (long)key * c_st + 8 * pc) = r.vp[i];
-        }
+      if constexpr (!kPlainV) {
+        // (both in the rotary arrangement: after the loop)
       } else if (own_rows && kc_mv != nullptr) {
         const int key_v = key0 + lrow_v;
-        if (key < L) {
-          if constexpr (ROPE) *reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc) = r.kp[i];
-          else __builtin_nontemporal_store(r.kp[i], reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc));
+        if constexpr (!ROPE) {
+          if (key < L) __builtin_nontemporal_store(r.kp[i], reinterpret_cast<u32x4*>(kc_mv + (long)key * c_st + 8 * pc));
         }
         if (key_v < L)
           __builtin_nontemporal_store(r.vp[i], reinterpret_cast<u32x4*>(vc_mv + (long)key_v * c_st + 8 * piece_idx_v(i)));
+      }
+    }
+    if constexpr (ROPE) {
+      // Rotated K rows for the cache (and, where V moves in the rotary arrangement too, the V rows).  In the rotary arrangement four lanes hold a row (lane q:
+      // pieces q and q + 4), so a store instruction would write half rows.  Neighbouring groups of
+      // four (the next head, or with one head per workgroup the next row) swap halves first
+      // (lower group gives its pieces 4..7, upper group its pieces 0..3, through a mirror of the
+      // eight lanes): then eight lanes hold one whole row per register and both stores write whole
+      // 128-byte rows, non-temporally like the V rows.
+      if (own_rows && kc_mv != nullptr) {
+        const bool upper = (lane >> 2) & 1;
+        const int ql = lane & 3;
+        u32x4 row_lo, row_hi;  // the lower group's row: pieces q | 7 - q; the upper group's: pieces 3 - q | q + 4
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t give = upper ? r.kp[0][d] : r.kp[1][d];
+          const uint32_t got = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)give, 0x141 /* row_half_mirror */, 0xf, 0xf, false);
+          row_lo[d] = upper ? got : r.kp[0][d];
+          row_hi[d] = upper ? r.kp[1][d] : got;
+        }
+        const int key = key0 + piece_row(0);
+        __bf16* base_lo = kc_mv;
+        __bf16* base_hi = kc_mv;
+        int key_lo = key, key_hi = key;
+        if constexpr (G >= 2) {
+          base_lo = upper ? kc_mv - c_sh : kc_mv;
+          base_hi = upper ? kc_mv : kc_mv + c_sh;
+        } else {
+          key_lo = upper ? key - 1 : key;
+          key_hi = upper ? key : key + 1;
+        }
+        const int piece_lo = upper ? 7 - ql : ql, piece_hi = upper ? ql + 4 : 3 - ql;
+        if (key_lo < L) __builtin_nontemporal_store(row_lo, reinterpret_cast<u32x4*>(base_lo + (long)key_lo * c_st + 8 * piece_lo));
+        if (key_hi < L) __builtin_nontemporal_store(row_hi, reinterpret_cast<u32x4*>(base_hi + (long)key_hi * c_st + 8 * piece_hi));
+        if constexpr (!kPlainV) {
+          u32x4 v_lo, v_hi;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const uint32_t give = upper ? r.vp[0][d] : r.vp[1][d];
+            const uint32_t got = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)give, 0x141, 0xf, 0xf, false);
+            v_lo[d] = upper ? got : r.vp[0][d];
+            v_hi[d] = upper ? r.vp[1][d] : got;
+          }
+          const long k_to_v = vc_mv - kc_mv;  // the V rows of the cache lie at a fixed distance from the K rows
+          if (key_lo < L) __builtin_nontemporal_store(v_lo, reinterpret_cast<u32x4*>(base_lo + k_to_v + (long)key_lo * c_st + 8 * piece_lo));
+          if (key_hi < L) __builtin_nontemporal_store(v_hi, reinterpret_cast<u32x4*>(base_hi + k_to_v + (long)key_hi * c_st + 8 * piece_hi));
+        }
       }
     }
   };
