@@ -225,9 +225,9 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
       if constexpr (QLDS)
         if (own_rows) *reinterpret_cast<u32x4*>(mv_lds + kOffQ + lrow * kRowBytes + ((pc ^ swz_k(lrow)) << 4)) = r.qp[i];
       // Cache rows leave non-temporally, an instruction writing whole rows: as they are in the
-      // plain arrangement, after an exchange between lanes in the rotary one (below; the two-block
-      // rotary variants still write half rows from two instructions, which the cache has to merge:
-      // non-temporal stores of half rows were slower, 99 -> 103 us).
+      // plain arrangement, after an exchange between lanes in the rotary one (below; half rows
+      // from two instructions have to be merged by the cache, and non-temporal half rows were
+      // slower still, 99 -> 103 us).
       const int key = key0 + lrow;
       if constexpr (!kPlainV) {
         // (both in the rotary arrangement: after the loop)
