@@ -118,7 +118,10 @@ typedef __attribute__((ext_vector_type(8))) short s16x8;
 // per compute unit) or 8 (two blocks; head dims 65..128: psi(q) and psi(k) are generated once for
 // both blocks, at 142 KB of LDS and up to 256 registers, i.e. one workgroup per compute unit).
 // With two blocks the v rows of a ring slot are two 64 x 128 B arrays, one per block, each laid
-// out as described above.
+// out as described above.  CTL <= CT of the tiles are live: for head dims 97..112 (112 is the
+// released 1B / 1.3B shape) the eighth tile's products, operand reads and image stores are
+// compiled out (the layouts keep eight tiles; B=4, L=4096, dv=112: 63 -> 59 us; large batches wait
+// for their rows and gain nothing).
 constexpr int kRing = 3;
 constexpr int kQkBytes = kChunk * kFeat * 2;       // 2 KB
 constexpr int kVBlockBytes = kChunk * 64 * 2;      // 8 KB: the v rows of one block of 64 channels
@@ -288,7 +291,7 @@ __device__ __forceinline__ void barrier_updater() {
 // ------------------------------------------------------------------------------------------
 // reader of token tile nt
 // ------------------------------------------------------------------------------------------
-template <int nt, int MODE, int CT>
+template <int nt, int MODE, int CT, int CTL>
 __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
   using LD = PrefillLds<CT>;
   const int lane = threadIdx.x & 63;
@@ -345,7 +348,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
         ka[mt] = *reinterpret_cast<const s16x4*>(s_k + (16 * mt + col) * kFeat + 4 * (grp ^ qk_swz));
       auto img_load = [&](int sg, bf16x8 (&A)[CT]) {
 #pragma unroll
-        for (int et = 0; et < CT; ++et)
+        for (int et = 0; et < CTL; ++et)
           A[et] = *reinterpret_cast<const bf16x8*>(s_img + ((sg * CT + et) * 64 + lane) * 16);
       };
       bf16x8 A[5][CT];
@@ -427,14 +430,14 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
         if constexpr (sg + 1 < 5) img_load(sg + 1, A[sg + 1]);
         if constexpr (sg == 3) {
 #pragma unroll
-          for (int et = 0; et < CT; ++et) vt_p[0][et] = load_vt(slot, vt_lane, vt_j, et, 0);
+          for (int et = 0; et < CTL; ++et) vt_p[0][et] = load_vt(slot, vt_lane, vt_j, et, 0);
         }
         if constexpr (sg == 4 && nt >= 2) {
 #pragma unroll
-          for (int et = 0; et < CT; ++et) vt_p[1][et] = load_vt(slot, vt_lane, vt_j, et, 1);
+          for (int et = 0; et < CTL; ++et) vt_p[1][et] = load_vt(slot, vt_lane, vt_j, et, 1);
         }
 #pragma unroll
-        for (int et = 0; et < CT; ++et) O[et] = mfma(A[sg][et], Bq[sg], O[et]);
+        for (int et = 0; et < CTL; ++et) O[et] = mfma(A[sg][et], Bq[sg], O[et]);
         if constexpr (sg + 1 < 5) Bq[sg + 1] = psi_q(integral_constant<int, sg + 1>{});
         if constexpr (sg == 0) {
 #pragma unroll
@@ -443,7 +446,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
           weights(integral_constant<int, 0>{});
         }
         if constexpr (sg == 1 && nt >= 2) weights(integral_constant<int, 1>{});
-        interleave<CT, ((sg == 0 ? 9 : (sg == 1 && nt >= 2) ? 8 : 3) * 4 + CT - 1) / CT>();
+        interleave<CTL, ((sg == 0 ? 9 : (sg == 1 && nt >= 2) ? 8 : 3) * 4 + CTL - 1) / CTL>();
         BASED_STAGE_END();
       });
 
@@ -452,7 +455,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       static_for<nt / 2 + 1>([&](auto SS) {
         constexpr int s = decltype(SS)::value;
 #pragma unroll
-        for (int et = 0; et < CT; ++et) O[et] = mfma(vt_p[s][et], bp[s], O[et]);
+        for (int et = 0; et < CTL; ++et) O[et] = mfma(vt_p[s][et], bp[s], O[et]);
         if constexpr (s == 0) {
           // the earlier tokens count 1 each, the lane groups hold partial sums of the rest
           const float z = group_allreduce(zpart) + (float)t0;
@@ -468,8 +471,12 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
       uint32_t P[CT][2];
 #pragma unroll
       for (int et = 0; et < CT; ++et) {
-        P[et][0] = pack_bf16(O[et][0] * inv, O[et][1] * inv);
-        P[et][1] = pack_bf16(O[et][2] * inv, O[et][3] * inv);
+        if (et < CTL) {
+          P[et][0] = pack_bf16(O[et][0] * inv, O[et][1] * inv);
+          P[et][1] = pack_bf16(O[et][2] * inv, O[et][3] * inv);
+        } else {
+          P[et][0] = P[et][1] = 0;  // a tile past the head dim: never stored
+        }
       }
       // The swap must not read a register in the two issue slots after a vector instruction wrote
       // it; the compiler does not look into inline assembly, so each one carries the wait.
@@ -519,7 +526,7 @@ __device__ __forceinline__ void lin_prefill_reader(BASED_CHAIN_PARAMS) {
 // ------------------------------------------------------------------------------------------
 // updater owning slot tiles own_tile(w, .)
 // ------------------------------------------------------------------------------------------
-template <int w, int MODE, int CT>
+template <int w, int MODE, int CT, int CTL>
 __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   using LD = PrefillLds<CT>;
   constexpr int kLoads = LD::kLoadsPerUpdater;
@@ -568,7 +575,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 #pragma unroll
     for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-      for (int et = 0; et < CT; ++et)
+      for (int et = 0; et < CTL; ++et)
         S[i][et] = *reinterpret_cast<const f32x4*>(ws_mine + ws_tile(own_tile(w, i), et));
     if constexpr (kNorm) {
       K2 = *reinterpret_cast<const f32x4*>(ws_mine + kWsK2 + lane * 4);
@@ -582,7 +589,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 #pragma unroll
       for (int i = 0; i < kOwn; ++i)
 #pragma unroll
-        for (int et = 0; et < CT; ++et)
+        for (int et = 0; et < CTL; ++et)
           S[i][et] += *reinterpret_cast<const f32x4*>(src + ws_tile(own_tile(w, i), et));
       if constexpr (kNorm) {
         K2 += *reinterpret_cast<const f32x4*>(src + kWsK2 + lane * 4);
@@ -645,7 +652,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
     static_assert(t % 2 == 0 && own_tile(w, 1) == t + 1, "first two own tiles = one slab");
     unsigned char* img = lds + LD::kOffImg + buf * LD::kImgBytes;
 #pragma unroll
-    for (int et = 0; et < CT; ++et) {
+    for (int et = 0; et < CTL; ++et) {
       const u32x4 w4 = {pack_bf16(S[0][et][0], S[0][et][1]), pack_bf16(S[0][et][2], S[0][et][3]),
                         pack_bf16(S[1][et][0], S[1][et][1]), pack_bf16(S[1][et][2], S[1][et][3])};
       *reinterpret_cast<u32x4*>(img + (((t >> 1) * CT + et) * 64 + lane) * 16) = w4;
@@ -656,7 +663,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       constexpr int t = own_tile(w, 2);
       unsigned char* img = lds + LD::kOffImg + buf * LD::kImgBytes;
 #pragma unroll
-      for (int et = 0; et < CT; ++et) {
+      for (int et = 0; et < CTL; ++et) {
         const uint2 w2 = make_uint2(pack_bf16(S[2][et][0], S[2][et][1]), pack_bf16(S[2][et][2], S[2][et][3]));
         *reinterpret_cast<uint2*>(img + (((t >> 1) * CT + et) * 64 + lane) * 16 + (t & 1) * 8) = w2;
       }
@@ -700,7 +707,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
     bf16x8 kt0 = load_kt(slot, kt_lane, 0);
     bf16x8 vt_s0[CT], vt_s1[CT];
 #pragma unroll
-    for (int et = 0; et < CT; ++et) vt_s0[et] = load_vt(slot, vt_lane, vt_j, et, 0);
+    for (int et = 0; et < CTL; ++et) vt_s0[et] = load_vt(slot, vt_lane, vt_j, et, 0);
     // the rows of the chunk after the next are requested (their slot was last read one chunk ago)
     const bool more2 = t0 + 2 * kChunk < t_end;
     if (more2) issue_loads(t0 + 2 * kChunk, slot_i == 0 ? 2 : slot_i - 1);
@@ -761,10 +768,10 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       constexpr int s = st / kOwn, i = st % kOwn;
       if constexpr (s == 0 && i == kOwn - 1) {
 #pragma unroll
-        for (int et = 0; et < CT; ++et) vt_s1[et] = load_vt(slot, vt_lane, vt_j, et, 1);
+        for (int et = 0; et < CTL; ++et) vt_s1[et] = load_vt(slot, vt_lane, vt_j, et, 1);
       }
 #pragma unroll
-      for (int et = 0; et < CT; ++et) S[i][et] = mfma(ak, s == 0 ? vt_s0[et] : vt_s1[et], S[i][et]);
+      for (int et = 0; et < CTL; ++et) S[i][et] = mfma(ak, s == 0 ? vt_s0[et] : vt_s1[et], S[i][et]);
       if constexpr (st + 1 < 2 * kOwn) {
         if constexpr (i + 1 == kOwn) {  // the next stage starts slab 1
           unpack_k(kt1);
@@ -778,7 +785,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
       if constexpr (MODE != kModeDelta && s == 1 && i == 2) {
         if (more1) publish_pair(buf ^ 1);  // both tiles of the slab are final
       }
-      interleave<CT, (((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i == 2) ? 6 : 3) * 4 + CT - 1) / CT>();
+      interleave<CTL, (((i + 1 == kOwn && s == 0) ? 7 : (s == 1 && i == 2) ? 6 : 3) * 4 + CTL - 1) / CTL>();
       BASED_STAGE_END();
     });
     // the rest of the state after this chunk, for the next chunk's readers
@@ -825,7 +832,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
   if (kv_state != nullptr && last_seg) {
     float* blk = reinterpret_cast<float*>(lds + LD::kOffImg);
     static_assert(16 * kExp * 4 <= LD::kImgBytes, "expansion block must fit in a state image buffer");
-    static_for<CT>([&](auto ET) {
+    static_for<CTL>([&](auto ET) {
       constexpr int et = decltype(ET)::value;
       if (16 * et >= live_ch) return;  // uniform over the workgroup (the readers count the same rounds)
       __syncthreads();  // the buffer is free (main loop done / previous block copied out)
@@ -876,7 +883,7 @@ __device__ __forceinline__ void lin_prefill_updater(BASED_CHAIN_PARAMS) {
 }
 #undef BASED_STAGE_END
 
-template <int MODE, int CT>
+template <int MODE, int CT, int CTL = CT>
 __global__ __launch_bounds__(kThreads, CT == 4 ? 4 : 2) void lin_prefill_mfma_kernel(
     const __bf16* __restrict__ q, const __bf16* __restrict__ k, const __bf16* __restrict__ v,
     __bf16* __restrict__ y, float* __restrict__ kv_state, float* __restrict__ k_state, int H, int L,
@@ -886,14 +893,14 @@ __global__ __launch_bounds__(kThreads, CT == 4 ? 4 : 2) void lin_prefill_mfma_ke
 #define BASED_CHAIN_ARGS lds, q, k, v, y, kv_state, k_state, H, L, dv, q_sb, q_sh, q_sl, k_sb, k_sh, \
                          k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, ws, seg_tokens, n_seg
   switch (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) {
-    case 0: lin_prefill_reader<0, MODE, CT>(BASED_CHAIN_ARGS); break;
-    case 1: lin_prefill_reader<1, MODE, CT>(BASED_CHAIN_ARGS); break;
-    case 2: lin_prefill_reader<2, MODE, CT>(BASED_CHAIN_ARGS); break;
-    case 3: lin_prefill_reader<3, MODE, CT>(BASED_CHAIN_ARGS); break;
-    case 4: lin_prefill_updater<0, MODE, CT>(BASED_CHAIN_ARGS); break;
-    case 5: lin_prefill_updater<1, MODE, CT>(BASED_CHAIN_ARGS); break;
-    case 6: lin_prefill_updater<2, MODE, CT>(BASED_CHAIN_ARGS); break;
-    default: lin_prefill_updater<3, MODE, CT>(BASED_CHAIN_ARGS); break;
+    case 0: lin_prefill_reader<0, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    case 1: lin_prefill_reader<1, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    case 2: lin_prefill_reader<2, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    case 3: lin_prefill_reader<3, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    case 4: lin_prefill_updater<0, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    case 5: lin_prefill_updater<1, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    case 6: lin_prefill_updater<2, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
+    default: lin_prefill_updater<3, MODE, CT, CTL>(BASED_CHAIN_ARGS); break;
   }
 #undef BASED_CHAIN_ARGS
 }
@@ -1042,6 +1049,8 @@ static bool prefill_mfma_takes(int64_t dv) { return dv >= 16 && dv <= 1024 && dv
 // Head dims of 65..128 channels go to workgroups that carry both blocks of 64 (psi(q) and psi(k)
 // generated once per head instead of once per block).
 static bool prefill_wide(int64_t dv) { return dv > 64 && dv <= 128; }
+// head dims 97..112 (the released 1B / 1.3B models have 112): seven live channel tiles in the wide workgroup
+static bool prefill_live7(int64_t dv) { return dv > 96 && dv <= 112; }
 // workgroups per (batch, head)
 static int64_t prefill_workgroups_per_head(int64_t dv) { return prefill_wide(dv) ? 1 : (dv + 63) / 64; }
 
@@ -1071,7 +1080,8 @@ extern "C" BASED_API int based_linear_attn_prefill(
                   "linear_attn_prefill: tensors must be 16-byte aligned");
     BASED_REQUIRE(B * H * ((dv + 63) / 64) < (1ll << 31), BASED_ERR_SHAPE, "linear_attn_prefill: sizes too large");
     dim3 grid((unsigned)(B * H * prefill_workgroups_per_head(dv))), block(kThreads);
-    auto kern = prefill_wide(dv) ? lin_prefill_mfma_kernel<kModeFull, 8> : lin_prefill_mfma_kernel<kModeFull, 4>;
+    auto kern = prefill_live7(dv) ? lin_prefill_mfma_kernel<kModeFull, 8, 7>
+                : prefill_wide(dv) ? lin_prefill_mfma_kernel<kModeFull, 8> : lin_prefill_mfma_kernel<kModeFull, 4>;
     hipLaunchKernelGGL(kern, grid, block, 0, s, (const __bf16*)q, (const __bf16*)k,
                        (const __bf16*)v, (__bf16*)y, kv_state, k_state, (int)H, (int)L, (int)dv, q_sb,
                        q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb, y_sh, y_sl, eps, (float*)nullptr, 0, 1);
@@ -1172,7 +1182,9 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
   // pass 1: every segment but the last accumulates its own contribution to the state
   const bool wide = prefill_wide(dv);
   const unsigned wgs = (unsigned)(B * H * prefill_workgroups_per_head(dv));  // a wide workgroup carries two chains
-  auto kern_delta = wide ? lin_prefill_mfma_kernel<kModeDelta, 8> : lin_prefill_mfma_kernel<kModeDelta, 4>;
+  const bool live7 = prefill_live7(dv);
+  auto kern_delta = live7 ? lin_prefill_mfma_kernel<kModeDelta, 8, 7>
+                    : wide ? lin_prefill_mfma_kernel<kModeDelta, 8> : lin_prefill_mfma_kernel<kModeDelta, 4>;
   hipLaunchKernelGGL(kern_delta, dim3(wgs, 1, (unsigned)(n_seg - 1)),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
@@ -1189,8 +1201,10 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
     rc = check_launch(who);
     if (rc) return rc;
   }
-  auto kern_from = fold ? (wide ? lin_prefill_mfma_kernel<kModeFromSum, 8> : lin_prefill_mfma_kernel<kModeFromSum, 4>)
-                        : (wide ? lin_prefill_mfma_kernel<kModeFrom, 8> : lin_prefill_mfma_kernel<kModeFrom, 4>);
+  auto kern_from = fold ? (live7 ? lin_prefill_mfma_kernel<kModeFromSum, 8, 7>
+                           : wide ? lin_prefill_mfma_kernel<kModeFromSum, 8> : lin_prefill_mfma_kernel<kModeFromSum, 4>)
+                        : (live7 ? lin_prefill_mfma_kernel<kModeFrom, 8, 7>
+                           : wide ? lin_prefill_mfma_kernel<kModeFrom, 8> : lin_prefill_mfma_kernel<kModeFrom, 4>);
   hipLaunchKernelGGL(kern_from, dim3(wgs, 1, (unsigned)n_seg),
                      block, 0, s, (const __bf16*)q, (const __bf16*)k, (const __bf16*)v, (__bf16*)y, kv_state,
                      k_state, (int)H, (int)L, (int)dv, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl, y_sb,
