@@ -130,8 +130,23 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
   // (59.7 -> 58.0 us).  With the rotary (65.7 against 68.6 us; with the cache fill as well the two
   // orders are equal) and with one head per workgroup (the other order is 2 % slower, 7 % with
   // rotary and cache fill): the runs of one head group are neighbours.
+  // Runs in both directions (paired heads, two-block ring, no rotary, no cache fill): the first
+  // tile of a run needs the 64 keys before it, which are the last tile's own keys of the run
+  // before.  Even runs walk their tiles downwards, odd runs upwards, and all runs of a head group
+  // sit behind one L2 (workgroup ids 8 apart): run 2m starts with its last tile at the moment
+  // run 2m + 1 fetches that tile's keys as its halo, and run 2m + 1 ends with its last tile when
+  // run 2m + 2, coming down, needs it: the second fetch of those rows is served by the L2
+  // (B=8, H=16, L=4096, 64 keys to the left: 216.1 -> 201.5 MB fetched per launch, which is q, k
+  // and v once; 54.0 -> 53.3 us).  The results do not depend on the direction.
+  constexpr bool kBidir = !ROPE && G > 1 && NB == 2;
+  const int n_hg = gridDim.x / runs_per_seq;  // head groups of the whole batch
+  const bool bidir = kBidir && kc_out == nullptr && runs_per_seq > 1 && n_hg % 8 == 0;
   int hg, run, b;
-  if constexpr (G > 1 && !ROPE) {
+  if (bidir) {
+    const int bhg = (int)(blockIdx.x % (unsigned)n_hg);
+    run = (int)(blockIdx.x / (unsigned)n_hg);
+    hg = bhg % (H / G), b = bhg / (H / G);
+  } else if constexpr (G > 1 && !ROPE) {
     hg = (int)(blockIdx.x % (unsigned)(H / G));
     const unsigned rest = blockIdx.x / (unsigned)(H / G);
     run = (int)(rest % (unsigned)runs_per_seq), b = (int)(rest / (unsigned)runs_per_seq);
@@ -142,6 +157,12 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
   }
   const int tile_begin = run * run_tiles;
   const int tile_end = tile_begin + run_tiles < n_tiles ? tile_begin + run_tiles : n_tiles;
+  const bool down = bidir && (run & 1) == 0;
+  // from one tile to the next: the queries move by q_step; the rows fetched are the next tile's
+  // own (upwards) or the block of keys at the far left of its window (downwards), q_ahead tokens
+  // before its queries
+  const int q_step = down ? -kQTile : kQTile;
+  const int q_ahead = down ? kQTile * (NB - 1) : 0;
 
   // rows are moved by lane-dependent heads (head0 + mv_head); the products are per wavefront (head0 + hsel)
   const long head0 = (long)hg * G;
@@ -184,17 +205,19 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
   // which would also end any overlap with the arithmetic): rows outside the sequence are fetched
   // from its nearest row instead.  Keys before the start are masked, keys and queries past the end
   // belong to rows that are never stored, so what is fetched for them does not matter.
-  auto load_rows = [&](int key0, SwaRows& r, bool with_q) {
+  auto load_rows = [&](int key0, SwaRows& r, bool with_q, int q_off = 0) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       int key = key0 + piece_row(i);
+      int qrow = key + q_off;
+      qrow = qrow < 0 ? 0 : (qrow < L ? qrow : L - 1);
       key = key < 0 ? 0 : (key < L ? key : L - 1);
       r.kp[i] = *reinterpret_cast<const u32x4*>(k_mv + (long)key * k_sl + 8 * piece_idx(i));
       int key_v = key0 + piece_row_v(i);
       key_v = key_v < 0 ? 0 : (key_v < L ? key_v : L - 1);
       r.vp[i] = *reinterpret_cast<const u32x4*>(v_mv + (long)key_v * v_sl + 8 * piece_idx_v(i));
       if constexpr (QLDS)
-        if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q_mv + (long)key * q_sl + 8 * piece_idx(i));  // a literal at every call
+        if (with_q) r.qp[i] = *reinterpret_cast<const u32x4*>(q_mv + (long)qrow * q_sl + 8 * piece_idx(i));  // a literal at every call
     }
     if constexpr (ROPE) {
       int key = key0 + piece_row(0);
@@ -311,7 +334,7 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
     bq[1] = __builtin_bit_cast(bf16x8, x[1]);
   };
 
-  int q0 = tile_begin * kQTile;
+  int q0 = (down ? tile_end - 1 : tile_begin) * kQTile;
   SwaRows pre;
   bf16x8 bq[2], bq_next[2];
   {
@@ -326,7 +349,7 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
     store_rows(0, q0, pre, true);
   }
   if (tile_begin + 1 < tile_end) {  // the next tile's rows travel while this one is computed
-    load_rows(q0 + kQTile, pre, true);
+    load_rows(q0 + q_step - q_ahead, pre, true, q_ahead);
     if constexpr (!QLDS) load_q(q0 + kQTile, bq_next);
   }
 
@@ -374,9 +397,12 @@ __global__ __launch_bounds__(256 * G, G >= 2 ? (NB == 3 ? 2 : 4) : (NB == 3 || R
     }
   } else {
     int own = 0;  // ring block with keys [q0, q0+64); block own + 1 (mod NB) is the oldest
-    for (int tile = tile_begin; tile < tile_end; ++tile, q0 += kQTile, own = own + 1 == NB ? 0 : own + 1) {
+    for (int tile = tile_begin; tile < tile_end; ++tile, q0 += q_step) {
       const int oldest = own + 1 == NB ? 0 : own + 1;
 #include "swa_tile.inc"
+      // upwards the oldest block has taken the next tile's own rows; downwards the block of this
+      // tile's own rows has taken the keys at the far left of the next tile's window
+      own = down ? (own == 0 ? NB - 1 : own - 1) : oldest;
     }
   }
 }

@@ -34,6 +34,30 @@ def test_prefill_matches_oracle(dev, B, L, H, w):
     assert rel_l2(out.float(), ref.float()) < TOL
 
 
+@pytest.mark.parametrize("B,L,H,w", [(8, 1500, 16, 64), (8, 1100, 16, 33), (4, 2000, 8, 64), (8, 2000, 6, 64),
+                                     (8, 601, 16, 0)])
+def test_prefill_runs_in_both_directions(dev, B, L, H, w):
+    """Batches whose head groups come in multiples of eight and whose runs hold several tiles: even
+    runs walk their tiles downwards, odd runs upwards (four heads per workgroup, and two for H = 6).
+    The cache fill keeps every run upwards: both must give the oracle's rows, and each other's."""
+    from based_amd import ops
+
+    print(f"swa prefill, runs in both directions: B={B} L={L} H={H} w={w}", flush=True)
+    qkv = _qkv(B, L, H, seed=11)
+    ref = O.sliding_window_attn(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], w_left=w)
+    qkv_d = qkv.to(dev)
+    out = ops.swa_prefill(qkv_d[:, :, 0], qkv_d[:, :, 1], qkv_d[:, :, 2], w_left=w)
+    cache = torch.zeros(B, L, 2, H, 64, dtype=torch.bfloat16, device=dev)
+    out_up = ops.swa_prefill(qkv_d[:, :, 0], qkv_d[:, :, 1], qkv_d[:, :, 2], w_left=w, kv_cache=cache)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert rel_l2(out.float(), ref.float()) < TOL
+    for b in range(B):  # no run may have gone wrong alone
+        assert rel_l2(out[b].float(), ref[b].float()) < TOL, f"batch entry {b}"
+    assert torch.equal(out, out_up)
+    assert torch.equal(cache[:, :, 0], qkv_d[:, :, 1]) and torch.equal(cache[:, :, 1], qkv_d[:, :, 2])
+
+
 @pytest.mark.parametrize("w", [0, 1, 63, 64, 65, 100, 127, 128])
 def test_window_edges_are_exact(dev, w):
     """q = 0 makes every visible key weigh the same, so the output is the plain mean of the V rows in
