@@ -1105,7 +1105,10 @@ extern "C" BASED_API int based_linear_attn_prefill(
 // Workgroup slots of one full wave of the MFMA prefill kernel on MI355X (256 CUs x 2 resident
 // workgroups); segment counts are chosen to fill about one such wave.
 static constexpr int64_t kPrefillSlots = 512;
-static constexpr int64_t kFoldSegments = 4;   // up to this many segments the second pass sums the earlier ones itself
+// Up to this many segments the second pass sums the earlier ones itself (measured: B=2, L=4096 as
+// 8 segments 32.0 -> 28.7 us, B=1 as 16 segments 24.9 -> 23.9 us without the prefix launch; the
+// planned segment counts beyond it belong to long sequences)
+static constexpr int64_t kFoldSegments = 16;
 
 extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, int64_t L, int64_t dv,
                                                         int io_dtype, int64_t* n_seg,
@@ -1121,7 +1124,7 @@ extern "C" BASED_API int based_linear_attn_prefill_plan(int64_t B, int64_t H, in
   // 48..128 -> 4, and from 192 chains on the single pass wins (one workgroup alone on a compute
   // unit is only 12 % slower per chunk than two sharing it, so filling the second slot does not
   // pay for the second pass over k and v).  Hence: about one workgroup per compute unit, at least
-  // four segments (up to four need no prefix launch), and for long sequences segments of at most
+  // four segments (up to kFoldSegments need no prefix launch), and for long sequences segments of at most
   // 32 chunks while that still fits the resident slots.
   if (chains > kPrefillSlots / 4 || chunks < 2) return BASED_OK;
   int64_t want = chains <= 16 ? 16 : (chains <= 32 ? 8 : 4);
@@ -1191,9 +1194,10 @@ static int launch_prefill_split(const char* who, const void* q, const void* k, c
                      y_sh, y_sl, eps, ws, seg_tokens, (int)n_seg);
   int rc = check_launch(who);
   if (rc) return rc;
-  // With few segments every workgroup of the second pass adds up the contributions before its
-  // own (at most kFoldSegments - 1 reads of 42 KB, mostly from L2); with many, a prefix pass over
-  // the workspace is cheaper than every workgroup reading half of its chain's entries.
+  // With up to kFoldSegments segments every workgroup of the second pass adds up the contributions
+  // before its own (reads of 42 KB each, mostly from L2: cheaper than one more launch); with more,
+  // a prefix pass over the workspace is cheaper than every workgroup reading half of its chain's
+  // entries.
   const bool fold = n_seg <= kFoldSegments;
   if (!fold) {
     hipLaunchKernelGGL(lin_prefill_prefix_kernel, dim3((unsigned)chains, (kSegStateFloats / 4 + 255) / 256), dim3(256), 0,

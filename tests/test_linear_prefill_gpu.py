@@ -198,7 +198,9 @@ def test_input_magnitudes(dev, scale, split):
 
 
 @pytest.mark.parametrize("B,H,L,dv,split", [(1, 2, 1000, 64, 4), (1, 2, 1200, 64, 5), (1, 1, 128, 64, 2), (2, 2, 700, 128, 3),
-                                            (1, 3, 4096, 64, 64), (1, 16, 4096, 64, None)])
+                                            (1, 3, 4096, 64, 64), (1, 16, 4096, 64, None),
+                                            # 8 and 16 segments summed by the second pass itself, 32 through the prefix launch
+                                            (2, 2, 2048, 64, 8), (1, 2, 4096, 112, 16), (1, 2, 4096, 128, 32)])
 def test_segmented_scan_matches_single_pass(dev, B, H, L, dv, split):
     """Sequences scanned as concurrent segments (small-batch path) against the single-pass kernel
     and the oracle, outputs and decode states; split=None lets the library plan the segments."""

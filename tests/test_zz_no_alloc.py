@@ -40,8 +40,9 @@ def _run(dev, B, H, L, dv, n_seg, seed, static):
 
 
 def test_static_scratch_matches_workspace_variant(dev):
-    # first call: 2*4 chains x 6 segments; second: fewer chains, fewer segments, shorter, ragged
-    for (B, H, L, dv, n_seg, seed) in [(2, 4, 1536, 64, 6, 11), (1, 2, 700, 128, 3, 12)]:
+    # first call: 2*4 chains x 24 segments (the prefix launch between the two passes); then fewer segments (the second
+    # pass sums them itself), then fewer chains, shorter, ragged
+    for (B, H, L, dv, n_seg, seed) in [(2, 4, 1536, 64, 24, 11), (2, 4, 1536, 64, 6, 13), (1, 2, 700, 128, 3, 12)]:
         print(f"no-alloc prefill case B={B} H={H} L={L} dv={dv} n_seg={n_seg}", flush=True)
         (q, k, v), y_s, kv_s, ks_s = _run(dev, B, H, L, dv, n_seg, seed, static=True)
         _, y_w, kv_w, ks_w = _run(dev, B, H, L, dv, n_seg, seed, static=False)
