@@ -44,11 +44,11 @@ D_EXP = 273
 # the same counter reads for a plain copy of known size (the summaries and the commands that
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": 293108530,   # B=128, H=16, dv=64, rotating state sets: fetch 146,972,795 + write 146,135,735
-    "lin_step_kernel_B64_dv128": 290398502,   # long-context decode: fetch 145,410,057 + write 144,988,445
-    "lin_prefill_mfma_kernel": {96: 2248581301},  # B=96, L=4096, dv=64, states written: fetch 1,334,153,864 + write 914,427,437 (the fetch varies by 10 % between runs); keyed by batch
-    "swa_prefill_kernel": 268705677,   # B=8, H=16, L=4096, four heads per workgroup, runs in both directions: fetch 201,530,551 + write 67,175,126
-    "decode_linear_kernel_lm_head": 104720207,   # M=4, 50280 x 1024 + closing norm: fetch 104,108,726 + write 611,481
+    "lin_step_kernel": 293112401,   # B=128, H=16, dv=64, rotating state sets
+    "lin_step_kernel_B64_dv128": 290399347,   # long-context decode
+    "lin_prefill_mfma_kernel": {96: 2255789451},  # B=96, L=4096, dv=64, states written: fetch 1,341,367,653 + write 914,421,798 (the fetch varies by 10 % between runs); keyed by batch
+    "swa_prefill_kernel": 268667517,   # B=8, H=16, L=4096, four heads per workgroup, runs in both directions: fetch 201,512,366 + write 67,155,151
+    "decode_linear_kernel_lm_head": 105002256,   # M=4, 50280 x 1024 + closing norm: fetch 104,390,516 + write 611,740
 }
 
 
