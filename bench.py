@@ -101,7 +101,7 @@ def _probe_ok(rc):
         raise RuntimeError(f"bench probe refused its arguments or failed to launch (code {rc})")
 
 
-def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0):
+def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0, pilot=4):
     """Average milliseconds per call of fn(), HIP events on the current stream.  warmup_ms > 0
     keeps launching (untimed) until that much wall time has passed: the board's power management
     needs ~20 ms of sustained MFMA load to settle (boost clock -> overshoot -> steady state), and
@@ -117,16 +117,25 @@ def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0):
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    # a few more untimed calls right in front of the timed ones, with no synchronisation in between:
+    # the stream is busy when the first event is recorded, so the timed region starts when they end,
+    # with its own launches already queued, and holds `steps` launches back to back (after a
+    # synchronisation the first launch would count the host's launch latency, 5 - 20 us, as its own)
+    for _ in range(pilot):
+        fn()
     e0.record()
     for _ in range(steps):
         fn()
     e1.record()
     torch.cuda.synchronize()
-    wall = (time.perf_counter() - t0) * 1e3 / steps
+    wall = (time.perf_counter() - t0) * 1e3 / (steps + pilot)
     return e0.elapsed_time(e1) / steps, wall
 
 
-def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4, replays=12):
+LONG_REGION = 256  # steps of the decode leg's second timed region when fewer are asked for
+
+
+def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4, replays=12, long_region_too=False):
     """Recurrent decode step.  Timed twice: COLD over `n_sets` independent (kv_state, k_state) sets
     visited in turn (n_sets x 145 MB at B=128, dv=64: more than the 256 MB last-level cache, and what
     the linear-attention layers of a stack do per token: every layer has its own state), and WARM
@@ -164,7 +173,7 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
                 _lib.check(rc)
         return step
 
-    def in_graph(sets):
+    def in_graph(sets, steps=steps):
         """The same `steps` launches recorded once and replayed, as the decoding loop issues them
         (generation.py: capture_graph); one replay is timed."""
         step = make_step(sets)
@@ -174,6 +183,12 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
             for _ in range(warmup):
                 step()
             side.synchronize()
+            # the untimed steps that run right in front of every timed replay (recorded first: the
+            # timed steps continue their rotation over the state sets)
+            lead = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(lead, stream=side):
+                for _ in range(max(warmup, 4)):
+                    step()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=side):
                 for _ in range(steps):
@@ -182,15 +197,23 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
         graph.replay()
         graph.replay()
         torch.cuda.synchronize()
-        # every replay timed by itself: the spread over `replays` samples is part of the result
-        samples = []
+        # Every replay timed by itself: the spread over `replays` samples is part of the result.
+        # The samples are queued in one go: max(warmup, 4) untimed steps, an event, the `steps`
+        # timed ones, an event, and the next sample's untimed steps right behind, with one
+        # synchronisation at the end.  Every timed region thus starts when untimed steps end, with
+        # its own launches already queued, on a GPU that has not been idle: a replay into an idle
+        # stream counts the host's graph-launch latency (10 - 20 us) among its steps, and the first
+        # millisecond after an idle period runs 2 - 3 % slower, which is all there is to 20 steps.
+        pairs = []
         for _ in range(replays):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            lead.replay()
             e0.record()
             graph.replay()
             e1.record()
-            torch.cuda.synchronize()
-            samples.append(e0.elapsed_time(e1) / steps)
+            pairs.append((e0, e1))
+        torch.cuda.synchronize()
+        samples = [e0.elapsed_time(e1) / steps for e0, e1 in pairs]
         samples.sort()
         return {"median": samples[len(samples) // 2], "min": samples[0], "max": samples[-1]}
 
@@ -203,8 +226,19 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
     gbs = bytes_per_launch / (ms * 1e-3) / 1e9
     spread = sp_cold if ms_cold >= ms_warm else sp_warm
     frac_of = lambda t: round(bytes_per_launch / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+    # A timed region of few steps also holds one boundary between two graph launches (about 14 us:
+    # 0.7 us per step of 20, 0.05 of 256), which is no part of the kernel's launch duration: with
+    # fewer than LONG_REGION steps the same measurement is repeated on LONG_REGION steps and
+    # reported beside the figure of the region asked for (which stays `value` and `frac`).
+    long_region = None
+    if long_region_too and steps < LONG_REGION:
+        lc, lw = in_graph(n_sets, LONG_REGION), in_graph(1, LONG_REGION)
+        lsp = lc if lc["median"] >= lw["median"] else lw  # the slower leg, as for the region asked for
+        long_region = {"steps": LONG_REGION, "cold_ms": round(lc["median"], 5), "warm_ms": round(lw["median"], 5),
+                       "frac": frac_of(lsp["median"]), "slowest": frac_of(lsp["max"]), "fastest": frac_of(lsp["min"])}
     assert torch.isfinite(y.float()).all() and all(torch.isfinite(a).all() for a, _ in states)
     return {
+        "long_region": long_region,
         "tok_s": B / (ms * 1e-3),
         "ms": ms,
         "wall_ms": wall,
@@ -224,8 +258,10 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
                          MEASURED_TRAFFIC_BYTES["lin_step_kernel_B64_dv128"] if (B, H, dv) == (64, 16, 128) else None),
                      "algorithmic_bytes_per_launch": bytes_per_launch,
                      "timed": "median over %d replays of a graph of the timed steps, the slower of cold (rotating state "
-                              "sets) and warm (one set); each replay timed by itself, spread in frac_spread (launched one "
-                              "by one: see decode_cold / decode_warm)" % replays},
+                              "sets) and warm (one set); each replay timed by itself between two events, with the "
+                              "untimed warm-up steps in a graph of their own right in front of it and all samples "
+                              "queued back to back; spread in frac_spread (launched one by one: see decode_cold / "
+                              "decode_warm)" % replays},
         "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, "
                     f"bf16 q/k/v, {n_sets} independent state sets visited in turn",
     }
@@ -772,7 +808,9 @@ def main():
         "data": "synthetic",
     }
     if args.only in (None, "decode"):
-        d = bench_decode(torch, ops, args.steps, args.warmup)
+        d = bench_decode(torch, ops, args.steps, args.warmup, long_region_too=True)
+        if d["long_region"] is not None:
+            d["roofline"]["long_region"] = d["long_region"]
         out.update({"value": round(d["tok_s"], 1), "ms_per_step": round(d["ms"], 5),
                     "config": {"workload": "configs[1]: " + d["workload"], "layers": 1},
                     "roofline": d["roofline"], "wall_ms_per_step": round(d["wall_ms"], 5),
