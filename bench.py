@@ -44,11 +44,11 @@ D_EXP = 273
 # the same counter reads for a plain copy of known size (the summaries and the commands that
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": 293112401,   # B=128, H=16, dv=64, rotating state sets
-    "lin_step_kernel_B64_dv128": 290399347,   # long-context decode
-    "lin_prefill_mfma_kernel": {96: 2255789451},  # B=96, L=4096, dv=64, states written: fetch 1,341,367,653 + write 914,421,798 (the fetch varies by 10 % between runs); keyed by batch
-    "swa_prefill_kernel": 268667517,   # B=8, H=16, L=4096, four heads per workgroup, runs in both directions: fetch 201,512,366 + write 67,155,151
-    "decode_linear_kernel_lm_head": 105002256,   # M=4, 50280 x 1024 + closing norm: fetch 104,390,516 + write 611,740
+    "lin_step_kernel": 293106116,   # B=128, H=16, dv=64, rotating state sets
+    "lin_step_kernel_B64_dv128": 290395163,   # long-context decode
+    "lin_prefill_mfma_kernel": {96: 2291264886},  # B=96, L=4096, dv=64, states written: fetch 1,376,849,071 + write 914,415,815 (the fetch varies by 10 % between runs); keyed by batch
+    "swa_prefill_kernel": 268706889,   # B=8, H=16, L=4096, four heads per workgroup, runs in both directions: fetch 201,529,540 + write 67,177,349
+    "decode_linear_kernel_lm_head": 104938864,   # M=4, 50280 x 1024 + closing norm: fetch 104,327,441 + write 611,423
 }
 
 
