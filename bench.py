@@ -89,6 +89,10 @@ def probes():
         lib.bench_probe_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
         lib.bench_probe_stream_prefill.argtypes = [C.c_void_p] * 4 + [C.c_int64] * 3 + [C.c_void_p]
         lib.bench_probe_mfma.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.POINTER(C.c_double), C.c_void_p]
+        lib.bench_probe_timestamp.argtypes = [C.c_void_p, C.c_void_p]
+        lib.bench_probe_timestamp.restype = C.c_int
+        lib.bench_probe_clock_khz.argtypes = []
+        lib.bench_probe_clock_khz.restype = C.c_int64
         for fn in (lib.bench_probe_stream_qkv, lib.bench_probe_rmw, lib.bench_probe_copy, lib.bench_probe_stream_prefill,
                    lib.bench_probe_mfma):
             fn.restype = C.c_int
@@ -174,48 +178,51 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
         return step
 
     def in_graph(sets, steps=steps):
-        """The same `steps` launches recorded once and replayed, as the decoding loop issues them
-        (generation.py: capture_graph); one replay is timed."""
+        """`replays` samples of exactly `steps` launches each, recorded in ONE graph as the decoding
+        loop records its launches (generation.py: capture_graph): per sample the untimed warm-up
+        steps, a timestamp launch, the `steps` timed launches, a timestamp launch (bench_probes.hip:
+        one lane stores the device's constant-rate clock).  The graph is replayed once untimed and
+        once for the figures: the GPU is never idle between the samples, and the difference of a
+        sample's two timestamps is the time of its `steps` launches and nothing else (both stamps
+        trail the launch before them by the same launch latency).  HIP events cannot be recorded
+        inside a graph on this platform, and events around a graph of just the timed steps also
+        count the boundary between two graph launches (about 14 us: 0.7 us per step of 20).
+        Cross-check in the result: HIP events around the whole replay, per launch of the hot kernel
+        (the 2 x `replays` timestamp launches add about 0.1 %)."""
         step = make_step(sets)
+        lead_n = max(warmup, 4)
+        lib_p = probes()
+        khz = lib_p.bench_probe_clock_khz()
+        if khz <= 0:
+            raise RuntimeError("the device clock rate is not available")
+        stamps = torch.zeros(2 * replays, dtype=torch.int64, device=dev)
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for _ in range(warmup):
                 step()
             side.synchronize()
-            # the untimed steps that run right in front of every timed replay (recorded first: the
-            # timed steps continue their rotation over the state sets)
-            lead = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(lead, stream=side):
-                for _ in range(max(warmup, 4)):
-                    step()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=side):
-                for _ in range(steps):
-                    step()
+                sp = torch.cuda.current_stream().cuda_stream
+                for r in range(replays):
+                    for _ in range(lead_n):
+                        step()
+                    _probe_ok(lib_p.bench_probe_timestamp(stamps.data_ptr() + 16 * r, sp))
+                    for _ in range(steps):
+                        step()
+                    _probe_ok(lib_p.bench_probe_timestamp(stamps.data_ptr() + 16 * r + 8, sp))
         torch.cuda.current_stream().wait_stream(side)
         graph.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         graph.replay()
+        e1.record()
         torch.cuda.synchronize()
-        # Every replay timed by itself: the spread over `replays` samples is part of the result.
-        # The samples are queued in one go: max(warmup, 4) untimed steps, an event, the `steps`
-        # timed ones, an event, and the next sample's untimed steps right behind, with one
-        # synchronisation at the end.  Every timed region thus starts when untimed steps end, with
-        # its own launches already queued, on a GPU that has not been idle: a replay into an idle
-        # stream counts the host's graph-launch latency (10 - 20 us) among its steps, and the first
-        # millisecond after an idle period runs 2 - 3 % slower, which is all there is to 20 steps.
-        pairs = []
-        for _ in range(replays):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            lead.replay()
-            e0.record()
-            graph.replay()
-            e1.record()
-            pairs.append((e0, e1))
-        torch.cuda.synchronize()
-        samples = [e0.elapsed_time(e1) / steps for e0, e1 in pairs]
-        samples.sort()
-        return {"median": samples[len(samples) // 2], "min": samples[0], "max": samples[-1]}
+        t = stamps.cpu().tolist()
+        samples = sorted((t[2 * r + 1] - t[2 * r]) / khz / steps for r in range(replays))  # ticks / kHz = ms
+        return {"median": samples[len(samples) // 2], "min": samples[0], "max": samples[-1],
+                "events_whole_replay": e0.elapsed_time(e1) / (replays * (lead_n + steps))}
 
     eager_cold, wall = _events_ms(torch, make_step(n_sets), steps, warmup)
     eager_warm, _ = _events_ms(torch, make_step(1), steps, warmup)
@@ -226,10 +233,9 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
     gbs = bytes_per_launch / (ms * 1e-3) / 1e9
     spread = sp_cold if ms_cold >= ms_warm else sp_warm
     frac_of = lambda t: round(bytes_per_launch / (t * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
-    # A timed region of few steps also holds one boundary between two graph launches (about 14 us:
-    # 0.7 us per step of 20, 0.05 of 256), which is no part of the kernel's launch duration: with
-    # fewer than LONG_REGION steps the same measurement is repeated on LONG_REGION steps and
-    # reported beside the figure of the region asked for (which stays `value` and `frac`).
+    # With fewer than LONG_REGION steps the same measurement is repeated on LONG_REGION steps and
+    # reported beside the figure of the region asked for (which stays `value` and `frac`): samples
+    # of 1 ms spread more than samples of 13 ms.
     long_region = None
     if long_region_too and steps < LONG_REGION:
         lc, lw = in_graph(n_sets, LONG_REGION), in_graph(1, LONG_REGION)
@@ -245,11 +251,13 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
         "cold": {"ms": round(ms_cold, 5), "ms_min": round(sp_cold["min"], 5), "ms_max": round(sp_cold["max"], 5),
                  "GBps": round(bytes_per_launch / (ms_cold * 1e-3) / 1e9, 1), "state_sets": n_sets,
                  "working_set_MB": round(n_sets * (kv_state.numel() + k_state.numel()) * 4 / 1e6, 1),
-                 "launched_one_by_one_ms": round(eager_cold, 5)},
+                 "launched_one_by_one_ms": round(eager_cold, 5),
+                 "events_around_the_whole_replay_ms": round(sp_cold["events_whole_replay"], 5)},
         "warm": {"ms": round(ms_warm, 5), "ms_min": round(sp_warm["min"], 5), "ms_max": round(sp_warm["max"], 5),
                  "GBps": round(bytes_per_launch / (ms_warm * 1e-3) / 1e9, 1), "state_sets": 1,
                  "working_set_MB": round((kv_state.numel() + k_state.numel()) * 4 / 1e6, 1),
-                 "launched_one_by_one_ms": round(eager_warm, 5)},
+                 "launched_one_by_one_ms": round(eager_warm, 5),
+                 "events_around_the_whole_replay_ms": round(sp_warm["events_whole_replay"], 5)},
         "roofline": {"kernel": "lin_step_kernel", "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                      "frac_spread": {"replays": replays, "median": frac_of(spread["median"]),
@@ -257,11 +265,11 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
                      "traffic": MEASURED_TRAFFIC_BYTES["lin_step_kernel"] if (B, H, dv) == (128, 16, 64) else (
                          MEASURED_TRAFFIC_BYTES["lin_step_kernel_B64_dv128"] if (B, H, dv) == (64, 16, 128) else None),
                      "algorithmic_bytes_per_launch": bytes_per_launch,
-                     "timed": "median over %d replays of a graph of the timed steps, the slower of cold (rotating state "
-                              "sets) and warm (one set); each replay timed by itself between two events, with the "
-                              "untimed warm-up steps in a graph of their own right in front of it and all samples "
-                              "queued back to back; spread in frac_spread (launched one by one: see decode_cold / "
-                              "decode_warm)" % replays},
+                     "timed": "median over %d samples of exactly the timed steps, the slower of cold (rotating state "
+                              "sets) and warm (one set); all samples recorded in one graph (warm-up steps, timestamp "
+                              "launch, the timed steps, timestamp launch) and replayed back to back; a sample = the "
+                              "difference of its two device timestamps; spread in frac_spread; HIP events around the "
+                              "whole replay and the launches issued one by one: see decode_cold / decode_warm" % replays},
         "workload": f"linear-attn recurrent decode, B={B} H={H} d=16 dv={dv}, fp32 state from a {prefill_len}-token prefill, "
                     f"bf16 q/k/v, {n_sets} independent state sets visited in turn",
     }

@@ -16,6 +16,12 @@
 //                sustain at the clock the board holds under that load (the published peak assumes
 //                the maximum clock).
 //
+//   timestamp  : one lane stores the constant-rate device clock (wall_clock64).  Recorded in a graph in
+//                front of and behind a run of launches, two of them time exactly that run from
+//                inside the stream, where HIP events cannot be recorded (a graph holds no timing
+//                events on this platform) and events around a whole graph launch also count the
+//                boundary between two graph launches.
+//
 // Every entry point returns 0, or 1 for arguments it does not take.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -158,7 +164,26 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float* __restrict__ out
   for (int i = 0; i < 8; ++i) acc += m[i][0] + m[i][1] + m[i][2] + m[i][3];
   out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
 }
+__global__ __launch_bounds__(64) void probe_timestamp_kernel(uint64_t* out) {
+  if (threadIdx.x == 0) *out = wall_clock64();
+}
 }  // namespace bench_probes
+
+// Stores the device's constant-rate clock at *out (device memory, 8-byte aligned) when the launch runs.
+PROBE_API int bench_probe_timestamp(void* out, void* stream) {
+  using namespace bench_probes;
+  PROBE_REQUIRE(out && (reinterpret_cast<uintptr_t>(out) & 7) == 0);
+  hipLaunchKernelGGL(probe_timestamp_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), (uint64_t*)out);
+  return hipGetLastError() == hipSuccess ? 0 : 2;
+}
+
+// Rate of that clock in kHz (0 if the runtime cannot tell).
+PROBE_API int64_t bench_probe_clock_khz() {
+  int dev = 0, khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+  return khz;
+}
 
 // `out` takes workgroups * 256 floats; *flops (host) receives the floating-point operations of the launch.
 PROBE_API int bench_probe_mfma(float* out, int64_t workgroups, int64_t iters, double* flops, void* stream) {

@@ -78,3 +78,44 @@ def test_mfma_probe_counts_its_flops_and_runs(dev):
     assert torch.isfinite(out).all() and out.unique().numel() > wgs
     assert lib.bench_probe_mfma(out.data_ptr(), 0, iters, C.byref(flops), stream) == 1
     assert lib.bench_probe_mfma(None, wgs, iters, C.byref(flops), stream) == 1
+
+
+def test_timestamp_probe_agrees_with_events(dev):
+    """Two timestamp launches around a run of copy launches, recorded in a graph: their difference in
+    ticks of the device clock is the run's duration as HIP events around the replay see it (events
+    also see the launch of the graph: they may read a little more, never less than the stamps by
+    more than the resolution)."""
+    import bench
+
+    lib = bench.probes()
+    khz = lib.bench_probe_clock_khz()
+    assert khz > 0
+    n = 64 << 20
+    a = torch.zeros(n // 4, dtype=torch.int32, device=dev)
+    b = torch.zeros_like(a)
+    stamps = torch.zeros(2, dtype=torch.int64, device=dev)
+    assert lib.bench_probe_timestamp(stamps.data_ptr() + 4, torch.cuda.current_stream().cuda_stream) == 1   # misaligned: refused
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            sp = torch.cuda.current_stream().cuda_stream
+            assert lib.bench_probe_copy(b.data_ptr(), a.data_ptr(), n, sp) == 0
+            assert lib.bench_probe_timestamp(stamps.data_ptr(), sp) == 0
+            for _ in range(40):
+                assert lib.bench_probe_copy(b.data_ptr(), a.data_ptr(), n, sp) == 0
+            assert lib.bench_probe_timestamp(stamps.data_ptr() + 8, sp) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t0, t1 = stamps.cpu().tolist()
+        ms_stamps = (t1 - t0) / khz
+        ms_events = e0.elapsed_time(e1) * 40 / 41
+        print(f"timestamp probe: {ms_stamps:.4f} ms by the stamps, {ms_events:.4f} ms by events (scaled to 40 of 41 copies)", flush=True)
+        assert t1 > t0
+        assert 0.9 * ms_events < ms_stamps < 1.05 * ms_events
