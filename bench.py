@@ -44,11 +44,11 @@ D_EXP = 273
 # the same counter reads for a plain copy of known size (the summaries and the commands that
 # produced them are the text files under profiles/); None until such a run exists for the kernel.
 MEASURED_TRAFFIC_BYTES = {
-    "lin_step_kernel": 293106116,   # B=128, H=16, dv=64, rotating state sets
-    "lin_step_kernel_B64_dv128": 290395163,   # long-context decode
-    "lin_prefill_mfma_kernel": {96: 2291264886},  # B=96, L=4096, dv=64, states written: fetch 1,376,849,071 + write 914,415,815 (the fetch varies by 10 % between runs); keyed by batch
-    "swa_prefill_kernel": 268706889,   # B=8, H=16, L=4096, four heads per workgroup, runs in both directions: fetch 201,529,540 + write 67,177,349
-    "decode_linear_kernel_lm_head": 104938864,   # M=4, 50280 x 1024 + closing norm: fetch 104,327,441 + write 611,423
+    "lin_step_kernel": 293110357,   # B=128, H=16, dv=64, rotating state sets
+    "lin_step_kernel_B64_dv128": 290402458,   # long-context decode
+    "lin_prefill_mfma_kernel": {96: 2275537424},  # B=96, L=4096, dv=64, states written: fetch 1,361,103,382 + write 914,434,042 (the fetch varies by 10 % between runs); keyed by batch
+    "swa_prefill_kernel": 268706329,   # B=8, H=16, L=4096, four heads per workgroup, runs in both directions: fetch 201,524,085 + write 67,182,244
+    "decode_linear_kernel_lm_head": 104920711,   # M=4, 50280 x 1024 + closing norm: fetch 104,309,135 + write 611,576
 }
 
 
@@ -139,7 +139,8 @@ def _events_ms(torch, fn, steps, warmup, warmup_ms=0.0, pilot=4):
 LONG_REGION = 256  # steps of the decode leg's second timed region when fewer are asked for
 
 
-def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4, replays=12, long_region_too=False):
+def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512, n_sets=4, replays=12, long_region_too=False,
+                 use_graph=True):
     """Recurrent decode step.  Timed twice: COLD over `n_sets` independent (kv_state, k_state) sets
     visited in turn (n_sets x 145 MB at B=128, dv=64: more than the 256 MB last-level cache, and what
     the linear-attention layers of a stack do per token: every layer has its own state), and WARM
@@ -190,6 +191,11 @@ def bench_decode(torch, ops, steps, warmup, B=128, H=16, dv=64, prefill_len=512,
         Cross-check in the result: HIP events around the whole replay, per launch of the hot kernel
         (the 2 x `replays` timestamp launches add about 0.1 %)."""
         step = make_step(sets)
+        if not use_graph:
+            # counter runs (a profiler that collects counters has crashed on replays of graphs this
+            # long): the same launches one by one, HIP events around each sample
+            ev = sorted(_events_ms(torch, step, steps, warmup)[0] for _ in range(replays))
+            return {"median": ev[len(ev) // 2], "min": ev[0], "max": ev[-1], "events_whole_replay": ev[len(ev) // 2]}
         lead_n = max(warmup, 4)
         lib_p = probes()
         khz = lib_p.bench_probe_clock_khz()
@@ -775,6 +781,8 @@ def main():
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="decode legs: launches issued one by one, HIP events (for counter runs under a profiler)")
     ap.add_argument("--only", choices=["decode", "prefill", "swa", "conv", "stack", "projections", "copy", "machine"], default=None,
                     help="one workload only; 'copy' is a plain 256 MiB device copy (the copy probe of bench_probes.hip) used to "
                          "calibrate the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run; 'machine' the memory "
@@ -816,7 +824,7 @@ def main():
         "data": "synthetic",
     }
     if args.only in (None, "decode"):
-        d = bench_decode(torch, ops, args.steps, args.warmup, long_region_too=True)
+        d = bench_decode(torch, ops, args.steps, args.warmup, long_region_too=not args.no_graph, use_graph=not args.no_graph)
         if d["long_region"] is not None:
             d["roofline"]["long_region"] = d["long_region"]
         out.update({"value": round(d["tok_s"], 1), "ms_per_step": round(d["ms"], 5),
@@ -839,7 +847,7 @@ def main():
     if args.only in (None, "prefill"):
         # configs[4]: one 32K-token sequence at head dim 128, and its decode batch of 64
         c5 = bench_prefill(torch, ops, 30, 3, B=1, L=32768, dv=128)
-        d5 = bench_decode(torch, ops, 64, 8, B=64, dv=128, prefill_len=256)
+        d5 = bench_decode(torch, ops, 64, 8, B=64, dv=128, prefill_len=256, use_graph=not args.no_graph)
         out["long_context"] = {"prefill": {k: (round(v, 3) if isinstance(v, float) else v) for k, v in c5.items()},
                                "decode": {"tok_s": round(d5["tok_s"], 1), "ms": round(d5["ms"], 5), "B": 64, "dv": 128,
                                           "cold": d5["cold"], "warm": d5["warm"], "roofline": d5["roofline"]}}
